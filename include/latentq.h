@@ -1,0 +1,136 @@
+/*
+ * latentq.h — C ABI of liblatentq_hip.so: the MI355X (gfx950) kernels behind the
+ * quantized-linear hot path of latentQ_LLM.
+ *
+ * Conventions (all entry points):
+ *   - every pointer is a DEVICE pointer on the current HIP device unless the
+ *     parameter is documented as a host value;
+ *   - the caller allocates every output; the library allocates nothing, never
+ *     synchronises, keeps no mutable global state and is re-entrant;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the
+ *     default stream) and the call returns immediately;
+ *   - return value: LQ_OK (0) on success, a negative LQ_ERR_* code otherwise;
+ *     lq_last_error() returns a thread-local description of the last failure;
+ *   - nothing throws across this boundary.
+ *
+ * Weight layout ("native" = the layout of the reference's QuantTensor.data for
+ * wbit 4, reference utils/quant.py:4-19): a flat byte array of N*K/2 bytes,
+ * row-major over W[N,K]; byte b of row n holds code(n, 2b) in its HIGH nibble
+ * and code(n, 2b+1) in its LOW nibble. Scales and zeros are bf16 arrays of
+ * N*K/group entries, entry n*(K/group) + k/group (reference utils/quant.py:
+ * 66-72, 427-428). `group` must be 128 (reference GROUPSIZE, utils/quant.py:44)
+ * and K a multiple of 128.
+ */
+#ifndef LATENTQ_H
+#define LATENTQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LQ_OK 0
+#define LQ_ERR_BAD_ARG (-1)   /* null pointer, bad shape, misaligned buffer */
+#define LQ_ERR_LAUNCH (-2)    /* HIP reported an error when launching        */
+#define LQ_ERR_UNSUPPORTED (-3)
+
+#define LQ_GROUP 128
+
+/* Version of this ABI; bumped on any incompatible change. */
+int lq_abi_version(void);
+
+/* Thread-local, NUL-terminated description of the last error on this thread
+ * ("" if none). The pointer stays valid until the next failing call. */
+const char *lq_last_error(void);
+
+/* ---------------------------------------------------------------------------
+ * (1) Stochastic-rounding latent requantizer.
+ *
+ * Replaces, on the latent-weight update path, the sequence
+ *   DeQfunc_4bit_g -> (update) -> Qfunc_4bit_g_res -> python_compress
+ * of the reference (utils/quant.py:1073, 1139-1144, 45-72), for the update
+ * rule  code' = clamp(floor((deq(W) - lr*g)/s + z + u), 0, 15)  with
+ *   w  = bf16_rne( bf16_rne(q - z) * s )          (reference dequant arithmetic)
+ *   t  = fma(-lr, g, w)                           (fp32, one rounding)
+ *   v  = ((t / s) + z) + u                        (fp32, IEEE, left to right)
+ *   code' = v<0 or NaN ? 0 : v>15 ? 15 : floor(v)
+ * codes_in / codes_out: N*K/2 bytes, native layout (may alias each other).
+ * scales, zeros: bf16[N*K/128]. grad: bf16[N,K] row-major. lr: host float.
+ * Noise: if u_or_null != NULL it is an fp32[N,K] array of u in [0,1);
+ * otherwise u for flat element index i is word (i & 3) of
+ * Philox4x32-10(counter = philox_offset + i/4 as a 128-bit little-endian
+ * integer in the low 64 bits, key = philox_seed) mapped as (x >> 8) * 2^-24.
+ * ------------------------------------------------------------------------- */
+int lq_requant_sr(const void *codes_in, void *codes_out, const void *scales, const void *zeros,
+                  const void *grad, float lr, int64_t N, int64_t K, int group,
+                  const float *u_or_null, uint64_t philox_seed, uint64_t philox_offset,
+                  void *stream);
+
+/* Materialise the same uniform stream lq_requant_sr draws from: out[i], i < n,
+ * is the u that element i would receive. For exactness checks. */
+int lq_philox_uniform(float *out, int64_t n, uint64_t philox_seed, uint64_t philox_offset,
+                      void *stream);
+
+/* ---------------------------------------------------------------------------
+ * (2) A16W4 dequant-GEMM / GEMV.
+ *
+ * lq_a16w4_fwd replaces DeQfunc_4bit_g + input.mm(weight.t()) (+ bias) of
+ * QLinearFunctionW4.forward / QLinearFunctionW4_eval.forward (reference
+ * utils/quant.py:116-121, 153-158):  Y[M,N] = X[M,K] * deq(W)[N,K]^T (+ bias[N]).
+ * lq_a16w4_dx replaces DeQfunc_4bit_g + grad_output.mm(weight) of
+ * QLinearFunctionW4.backward (utils/quant.py:136-140): dX[M,K] = dY[M,N] * deq(W).
+ * x, y, dy, dx, bias: bf16 row-major; accumulation in fp32, output rounded to
+ * bf16 (round-to-nearest-even). M <= 16 takes the wavefront GEMV path.
+ * Requirements: K % 128 == 0, N % 16 == 0 (fwd), N % 16 == 0 (dx); all
+ * pointers 16-byte aligned.
+ * ------------------------------------------------------------------------- */
+int lq_a16w4_fwd(const void *x, const void *codes, const void *scales, const void *zeros,
+                 const void *bias_or_null, void *y, int64_t M, int64_t N, int64_t K, int group,
+                 void *stream);
+
+int lq_a16w4_dx(const void *dy, const void *codes, const void *scales, const void *zeros,
+                void *dx, int64_t M, int64_t N, int64_t K, int group, void *stream);
+
+/* Dequantise the whole matrix to bf16[N,K] with the reference arithmetic
+ * (DeQfunc_4bit_g, utils/quant.py:66-72). Used for the dW-side consumers and
+ * for checks; not on the forward/backward GEMM path. */
+int lq_a16w4_dequant(const void *codes, const void *scales, const void *zeros, void *w_out,
+                     int64_t N, int64_t K, int group, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * (3) A8W8 int8 GEMM with fused scale epilogue.
+ *
+ * Replaces torch_int._CUDA.linear_a8_w8_bbf16_obf16 and the trailing
+ * `* qscales.view(1,-1)` (reference utils/quant.py:268-271 and its siblings):
+ *   acc[m,n] = sum_k x[m,k] * w[n,k]                    (exact int32)
+ *   y[m,n]   = bf16_rne( (float(acc) * sx[m]) * sw[n] + bias[n] )
+ * x: int8[M,K], w: int8[N,K] row-major; sx: fp32[M]; sw: fp32[N];
+ * bias_or_null: bf16[N]; y: bf16[M,N]; acc_or_null: int32[M,N] (written when
+ * non-NULL, for the bit-exact accumulator check). K % 64 == 0, N % 16 == 0.
+ * ------------------------------------------------------------------------- */
+int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const float *sw,
+                const void *bias_or_null, void *y, int32_t *acc_or_null, int64_t M, int64_t N,
+                int64_t K, void *stream);
+
+/* Per-tensor symmetric activation quantizer used in front of lq_a8w8_fwd:
+ *   x8 = clamp(round_half_even(x * (127/clampv)), -128, 127)
+ * (reference utils/quant.py:264-266). x: bf16[n]; clampv: DEVICE fp32 scalar;
+ * x8: int8[n]. */
+int lq_act_quant_i8(const void *x, const float *clampv_dev, int8_t *x8, int64_t n, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Layout converters (device side).
+ * GPTQ layout (reference PTQ/quant/quant_linear.py:343-389): qweight is
+ * int32[K/8, N] with code(k, n) at bits 4*(k%8) of word [k/8, n].
+ * ------------------------------------------------------------------------- */
+int lq_repack_gptq_to_native(const int32_t *qweight_gptq, void *codes_native, int64_t N, int64_t K,
+                             void *stream);
+int lq_repack_native_to_gptq(const void *codes_native, int32_t *qweight_gptq, int64_t N, int64_t K,
+                             void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LATENTQ_H */

@@ -1,0 +1,76 @@
+// Shared device/host helpers for the gfx950 kernels of liblatentq_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/latentq.h"
+
+// ---- error plumbing (defined in lq_api.hip) --------------------------------
+int lq_fail(int code, const char *fmt, ...);
+int lq_check_launch(const char *what);
+
+#define LQ_REQUIRE(cond, ...)                          \
+    do {                                               \
+        if (!(cond)) return lq_fail(LQ_ERR_BAD_ARG, __VA_ARGS__); \
+    } while (0)
+
+static inline bool lq_aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+// ---- vector types ----------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) int i32x4_t;
+typedef __attribute__((ext_vector_type(16))) int i32x16_t;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
+
+// ---- bf16 <-> fp32 on raw bits ---------------------------------------------
+__device__ __forceinline__ float lq_bf16_lo(unsigned packed) { return __uint_as_float(packed << 16); }
+__device__ __forceinline__ float lq_bf16_hi(unsigned packed) { return __uint_as_float(packed & 0xFFFF0000u); }
+__device__ __forceinline__ float lq_bf16_bits_to_f32(unsigned short b) { return __uint_as_float(((unsigned)b) << 16); }
+
+// Two fp32 -> packed bf16 pair, round-to-nearest-even (v_cvt_pk_bf16_f32): lo = a, hi = b.
+__device__ __forceinline__ unsigned lq_pack_bf16(float a, float b) {
+    bf16x2_t r;
+    r[0] = (__bf16)a;
+    r[1] = (__bf16)b;
+    return __builtin_bit_cast(unsigned, r);
+}
+__device__ __forceinline__ unsigned short lq_f32_to_bf16_bits(float a) {
+    __bf16 r = (__bf16)a;
+    return __builtin_bit_cast(unsigned short, r);
+}
+
+// ---- native int4 layout ----------------------------------------------------
+// A little-endian 32-bit word of the native layout holds the codes of 8
+// consecutive k: code j sits at bit 4*(j^1)  (even index = high nibble of its byte).
+__device__ __forceinline__ unsigned lq_code(unsigned word, int j) { return (word >> (4 * (j ^ 1))) & 0xFu; }
+
+// ---- Philox4x32-10 ---------------------------------------------------------
+#define LQ_PHILOX_M0 0xD2511F53u
+#define LQ_PHILOX_M1 0xCD9E8D57u
+#define LQ_PHILOX_W0 0x9E3779B9u
+#define LQ_PHILOX_W1 0xBB67AE85u
+
+struct lq_u4 {
+    unsigned x, y, z, w;
+};
+
+__host__ __device__ __forceinline__ lq_u4 lq_philox4x32_10(unsigned c0, unsigned c1, unsigned c2, unsigned c3,
+                                                          unsigned k0, unsigned k1) {
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        unsigned long long p0 = (unsigned long long)LQ_PHILOX_M0 * c0;
+        unsigned long long p1 = (unsigned long long)LQ_PHILOX_M1 * c2;
+        unsigned n0 = (unsigned)(p1 >> 32) ^ c1 ^ k0;
+        unsigned n1 = (unsigned)p1;
+        unsigned n2 = (unsigned)(p0 >> 32) ^ c3 ^ k1;
+        unsigned n3 = (unsigned)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += LQ_PHILOX_W0;
+        k1 += LQ_PHILOX_W1;
+    }
+    lq_u4 o = {c0, c1, c2, c3};
+    return o;
+}

@@ -1,0 +1,140 @@
+// Elementwise companions of the GEMM kernels: whole-matrix dequantise, activation
+// quantizer for the int8 path, and GPTQ <-> native layout converters.
+#include "lq_common.h"
+
+namespace {
+
+// One thread = one packed word (8 codes of one row) -> 16 bytes of bf16.
+// Arithmetic of the reference dequantiser: bf16(bf16(q - z) * s).
+__global__ __launch_bounds__(256) void dequant_kernel(const unsigned *__restrict__ codes,
+                                                      const unsigned short *__restrict__ scales,
+                                                      const unsigned short *__restrict__ zeros,
+                                                      u32x4_t *__restrict__ out, long long n_words) {
+    const long long w = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (w >= n_words) return;
+    const unsigned word = codes[w];
+    const float s = lq_bf16_bits_to_f32(scales[w >> 4]);
+    const float z = lq_bf16_bits_to_f32(zeros[w >> 4]);
+    u32x4_t o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float d0 = (float)lq_code(word, 2 * i) - z;
+        float d1 = (float)lq_code(word, 2 * i + 1) - z;
+        unsigned dp = lq_pack_bf16(d0, d1);
+        o[i] = lq_pack_bf16(lq_bf16_lo(dp) * s, lq_bf16_hi(dp) * s);
+    }
+    out[w] = o;
+}
+
+// x8 = clamp(rne(bf16(bf16(x * 127) / clampv)), -128, 127); 8 elements per thread.
+__global__ __launch_bounds__(256) void act_quant_kernel(const unsigned short *__restrict__ x,
+                                                        const float *__restrict__ clampv, signed char *__restrict__ x8,
+                                                        long long n) {
+    const float c = clampv[0];
+    const long long base = ((long long)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (base >= n) return;
+    if (base + 8 <= n && (((uintptr_t)(x + base)) & 15) == 0 && (((uintptr_t)(x8 + base)) & 7) == 0) {
+        u32x4_t v = *reinterpret_cast<const u32x4_t *>(x + base);
+        unsigned r[2] = {0u, 0u};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            float f = (j & 1) ? lq_bf16_hi(v[j >> 1]) : lq_bf16_lo(v[j >> 1]);
+            float a = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(f * 127.0f));
+            float q = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(a / c));
+            float rr = __builtin_amdgcn_fmed3f(rintf(q), -128.0f, 127.0f);
+            int iv = (int)rr;
+            r[j >> 2] |= ((unsigned)iv & 0xFFu) << (8 * (j & 3));
+        }
+        u32x2_t o = {r[0], r[1]};
+        *reinterpret_cast<u32x2_t *>(x8 + base) = o;
+    } else {
+        for (long long i = base; i < n && i < base + 8; ++i) {
+            float f = lq_bf16_bits_to_f32(x[i]);
+            float a = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(f * 127.0f));
+            float q = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(a / c));
+            float rr = __builtin_amdgcn_fmed3f(rintf(q), -128.0f, 127.0f);
+            x8[i] = (signed char)(int)rr;
+        }
+    }
+}
+
+__device__ __forceinline__ unsigned swap_nibbles(unsigned g) {
+    return ((g & 0x0F0F0F0Fu) << 4) | ((g >> 4) & 0x0F0F0F0Fu);
+}
+
+// 32x32-word tile transpose through LDS: GPTQ word [kw][n] <-> native word [n][kw].
+// kToNative: src is [KW][N], dst is [N][KW]; otherwise src is [N][KW], dst is [KW][N].
+template <bool kToNative>
+__global__ __launch_bounds__(256) void repack_kernel(const unsigned *__restrict__ src, unsigned *__restrict__ dst,
+                                                     int N, int KW) {
+    __shared__ unsigned tile[32][33];
+    const int src_rows = kToNative ? KW : N, src_cols = kToNative ? N : KW;
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int r = r0 + ty + 8 * i, c = c0 + tx;
+        if (r < src_rows && c < src_cols) tile[ty + 8 * i][tx] = swap_nibbles(src[(long long)r * src_cols + c]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int r = c0 + ty + 8 * i, c = r0 + tx;  // dst is [src_cols][src_rows]
+        if (r < src_cols && c < src_rows) dst[(long long)r * src_rows + c] = tile[tx][ty + 8 * i];
+    }
+}
+
+}  // namespace
+
+extern "C" int lq_a16w4_dequant(const void *codes, const void *scales, const void *zeros, void *w_out, int64_t N,
+                                int64_t K, int group, void *stream) {
+    LQ_REQUIRE(codes && scales && zeros && w_out, "lq_a16w4_dequant: null pointer argument");
+    LQ_REQUIRE(group == LQ_GROUP, "lq_a16w4_dequant: group must be %d", LQ_GROUP);
+    LQ_REQUIRE(N > 0 && K > 0 && K % LQ_GROUP == 0, "lq_a16w4_dequant: need N > 0, K a positive multiple of %d", LQ_GROUP);
+    LQ_REQUIRE(lq_aligned(codes, 4) && lq_aligned(w_out, 16), "lq_a16w4_dequant: misaligned buffer");
+    const long long n_words = (long long)N * K / 8;
+    const long long blocks = (n_words + 255) / 256;
+    LQ_REQUIRE(blocks <= 0x7FFFFFFFll, "lq_a16w4_dequant: tensor too large");
+    hipLaunchKernelGGL(dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const unsigned *)codes, (const unsigned short *)scales, (const unsigned short *)zeros,
+                       (u32x4_t *)w_out, n_words);
+    return lq_check_launch("lq_a16w4_dequant");
+}
+
+extern "C" int lq_act_quant_i8(const void *x, const float *clampv_dev, int8_t *x8, int64_t n, void *stream) {
+    LQ_REQUIRE(x && clampv_dev && x8 && n >= 0, "lq_act_quant_i8: bad argument");
+    if (n == 0) return LQ_OK;
+    const long long blocks = ((n + 7) / 8 + 255) / 256;
+    LQ_REQUIRE(blocks <= 0x7FFFFFFFll, "lq_act_quant_i8: n too large");
+    hipLaunchKernelGGL(act_quant_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const unsigned short *)x, clampv_dev, (signed char *)x8, (long long)n);
+    return lq_check_launch("lq_act_quant_i8");
+}
+
+static int repack_common(const void *src, void *dst, int64_t N, int64_t K, void *stream, bool to_native, const char *who) {
+    LQ_REQUIRE(src && dst, "%s: null pointer argument", who);
+    LQ_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "%s: need N > 0 and K a positive multiple of 8", who);
+    LQ_REQUIRE(lq_aligned(src, 4) && lq_aligned(dst, 4), "%s: buffers must be 4-byte aligned", who);
+    LQ_REQUIRE(N < (1ll << 30) && K < (1ll << 30), "%s: dimension too large", who);
+    const int KW = (int)(K / 8), n = (int)N;
+    if (to_native) {
+        dim3 grid((n + 31) / 32, (KW + 31) / 32);
+        hipLaunchKernelGGL(repack_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, (const unsigned *)src,
+                           (unsigned *)dst, n, KW);
+    } else {
+        dim3 grid((KW + 31) / 32, (n + 31) / 32);
+        hipLaunchKernelGGL(repack_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, (const unsigned *)src,
+                           (unsigned *)dst, n, KW);
+    }
+    return lq_check_launch(who);
+}
+
+extern "C" int lq_repack_gptq_to_native(const int32_t *qweight_gptq, void *codes_native, int64_t N, int64_t K,
+                                        void *stream) {
+    return repack_common(qweight_gptq, codes_native, N, K, stream, true, "lq_repack_gptq_to_native");
+}
+
+extern "C" int lq_repack_native_to_gptq(const void *codes_native, int32_t *qweight_gptq, int64_t N, int64_t K,
+                                        void *stream) {
+    return repack_common(codes_native, qweight_gptq, N, K, stream, false, "lq_repack_native_to_gptq");
+}

@@ -1,0 +1,173 @@
+"""Tensor-level wrappers over the C ABI: validate, allocate outputs with torch, pass raw pointers
+and the current HIP stream. PyTorch is used for device memory and streams only."""
+from __future__ import annotations
+
+import torch
+
+from . import _C
+
+GROUP = 128
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _chk(t: torch.Tensor, dtype, name: str):
+    if not t.is_cuda:
+        raise _C.LatentQError(f"{name} must be a GPU tensor: the HIP kernels have no CPU fallback")
+    if t.dtype != dtype:
+        raise TypeError(f"{name}: expected {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+
+
+def _codes_ok(codes: torch.Tensor, N: int, K: int):
+    if codes.dtype not in (torch.int8, torch.uint8):
+        raise TypeError(f"codes: expected int8/uint8 bytes, got {codes.dtype}")
+    if not codes.is_cuda or not codes.is_contiguous():
+        raise ValueError("codes must be a contiguous GPU tensor")
+    if codes.numel() != N * K // 2:
+        raise ValueError(f"codes has {codes.numel()} bytes, expected N*K/2 = {N * K // 2}")
+
+
+def _qparam_ok(scales, zeros, N, K):
+    _chk(scales, torch.bfloat16, "scales")
+    _chk(zeros, torch.bfloat16, "zeros")
+    n = N * K // GROUP
+    if scales.numel() != n or zeros.numel() != n:
+        raise ValueError(f"scales/zeros need {n} entries, got {scales.numel()}/{zeros.numel()}")
+
+
+def requant_sr(codes, scales, zeros, grad, lr: float, shape, u=None, seed: int = 0, offset: int = 0, out=None):
+    """New packed codes after one stochastic-rounding latent update (see include/latentq.h, lq_requant_sr)."""
+    N, K = shape
+    _codes_ok(codes, N, K)
+    _qparam_ok(scales, zeros, N, K)
+    _chk(grad, torch.bfloat16, "grad")
+    if grad.numel() != N * K:
+        raise ValueError("grad must have N*K elements")
+    if u is not None:
+        _chk(u, torch.float32, "u")
+        if u.numel() != N * K:
+            raise ValueError("u must have N*K elements")
+    if out is None:
+        out = torch.empty_like(codes)
+    else:
+        _codes_ok(out, N, K)
+    with torch.cuda.device(codes.device):
+        _C.call("lq_requant_sr", codes.data_ptr(), out.data_ptr(), scales.data_ptr(), zeros.data_ptr(),
+                grad.data_ptr(), float(lr), N, K, GROUP, None if u is None else u.data_ptr(),
+                seed & (2**64 - 1), offset & (2**64 - 1), _stream(codes))
+    return out
+
+
+def philox_uniform(n: int, seed: int, offset: int = 0, device="cuda"):
+    out = torch.empty(n, dtype=torch.float32, device=device)
+    with torch.cuda.device(out.device):
+        _C.call("lq_philox_uniform", out.data_ptr(), n, seed & (2**64 - 1), offset & (2**64 - 1), _stream(out))
+    return out
+
+
+def a16w4_forward(x, codes, scales, zeros, shape, bias=None):
+    """Y[M,N] = X[M,K] . deq(W)[N,K]^T (+ bias) in bf16 with fp32 accumulation."""
+    N, K = shape
+    _chk(x, torch.bfloat16, "x")
+    if x.dim() != 2 or x.shape[1] != K:
+        raise ValueError(f"x must be [M,{K}], got {tuple(x.shape)}")
+    _codes_ok(codes, N, K)
+    _qparam_ok(scales, zeros, N, K)
+    if bias is not None:
+        _chk(bias, torch.bfloat16, "bias")
+        if bias.numel() != N:
+            raise ValueError("bias must have N elements")
+    M = x.shape[0]
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    if M == 0:
+        return y
+    with torch.cuda.device(x.device):
+        _C.call("lq_a16w4_fwd", x.data_ptr(), codes.data_ptr(), scales.data_ptr(), zeros.data_ptr(),
+                None if bias is None else bias.data_ptr(), y.data_ptr(), M, N, K, GROUP, _stream(x))
+    return y
+
+
+def a16w4_dx(dy, codes, scales, zeros, shape):
+    """dX[M,K] = dY[M,N] . deq(W)[N,K]."""
+    N, K = shape
+    _chk(dy, torch.bfloat16, "dy")
+    if dy.dim() != 2 or dy.shape[1] != N:
+        raise ValueError(f"dy must be [M,{N}], got {tuple(dy.shape)}")
+    _codes_ok(codes, N, K)
+    _qparam_ok(scales, zeros, N, K)
+    M = dy.shape[0]
+    dx = torch.empty((M, K), dtype=torch.bfloat16, device=dy.device)
+    if M == 0:
+        return dx
+    with torch.cuda.device(dy.device):
+        _C.call("lq_a16w4_dx", dy.data_ptr(), codes.data_ptr(), scales.data_ptr(), zeros.data_ptr(), dx.data_ptr(),
+                M, N, K, GROUP, _stream(dy))
+    return dx
+
+
+def a16w4_dequant(codes, scales, zeros, shape):
+    N, K = shape
+    _codes_ok(codes, N, K)
+    _qparam_ok(scales, zeros, N, K)
+    w = torch.empty((N, K), dtype=torch.bfloat16, device=codes.device)
+    with torch.cuda.device(codes.device):
+        _C.call("lq_a16w4_dequant", codes.data_ptr(), scales.data_ptr(), zeros.data_ptr(), w.data_ptr(), N, K, GROUP,
+                _stream(codes))
+    return w
+
+
+def a8w8_forward(x8, w8, sx, sw, bias=None, want_acc: bool = False):
+    """bf16 Y = ((int32 X8.W8^T) * sx[m]) * sw[n] (+ bias); optionally also the int32 accumulators."""
+    _chk(x8, torch.int8, "x8")
+    _chk(w8, torch.int8, "w8")
+    _chk(sx, torch.float32, "sx")
+    _chk(sw, torch.float32, "sw")
+    M, K = x8.shape
+    N, K2 = w8.shape
+    if K != K2:
+        raise ValueError("x8 and w8 disagree on K")
+    if sx.numel() != M or sw.numel() != N:
+        raise ValueError("sx must have M entries and sw N entries")
+    if bias is not None:
+        _chk(bias, torch.bfloat16, "bias")
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x8.device)
+    acc = torch.empty((M, N), dtype=torch.int32, device=x8.device) if want_acc else None
+    if M > 0:
+        with torch.cuda.device(x8.device):
+            _C.call("lq_a8w8_fwd", x8.data_ptr(), w8.data_ptr(), sx.data_ptr(), sw.data_ptr(),
+                    None if bias is None else bias.data_ptr(), y.data_ptr(), None if acc is None else acc.data_ptr(),
+                    M, N, K, _stream(x8))
+    return (y, acc) if want_acc else y
+
+
+def act_quant_i8(x, clampv):
+    """int8 activations clamp(rne(x*127/clampv)); clampv is a 1-element fp32 GPU tensor (no host sync)."""
+    _chk(x, torch.bfloat16, "x")
+    _chk(clampv, torch.float32, "clampv")
+    out = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    if x.numel():
+        with torch.cuda.device(x.device):
+            _C.call("lq_act_quant_i8", x.data_ptr(), clampv.data_ptr(), out.data_ptr(), x.numel(), _stream(x))
+    return out
+
+
+def repack_gptq_to_native(qweight, shape):
+    N, K = shape
+    _chk(qweight, torch.int32, "qweight")
+    out = torch.empty(N * K // 2, dtype=torch.int8, device=qweight.device)
+    with torch.cuda.device(qweight.device):
+        _C.call("lq_repack_gptq_to_native", qweight.data_ptr(), out.data_ptr(), N, K, _stream(qweight))
+    return out
+
+
+def repack_native_to_gptq(codes, shape):
+    N, K = shape
+    _codes_ok(codes, N, K)
+    out = torch.empty((K // 8, N), dtype=torch.int32, device=codes.device)
+    with torch.cuda.device(codes.device):
+        _C.call("lq_repack_native_to_gptq", codes.data_ptr(), out.data_ptr(), N, K, _stream(codes))
+    return out

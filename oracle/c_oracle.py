@@ -1,0 +1,162 @@
+"""ctypes front end to oracle/lq_oracle.c. bf16 data travels as numpy uint16 bit patterns."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liblq_oracle.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.run(["make", "-C", _HERE] + (["-B"] if force else []), check=True, capture_output=True)
+    return _LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.lqo_bf16_to_f32.restype = C.c_float
+        _lib.lqo_bf16_to_f32.argtypes = [C.c_uint16]
+        _lib.lqo_f32_to_bf16.restype = C.c_uint16
+        _lib.lqo_f32_to_bf16.argtypes = [C.c_float]
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _c(a, dtype):
+    a = np.ascontiguousarray(a)
+    assert a.dtype == dtype, (a.dtype, dtype)
+    return a
+
+
+def f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:
+    """Round-to-nearest-even fp32 -> bf16 bit patterns (vectorised, same rule as the C helper)."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+    r = np.where(nan, (u >> 16) | 0x40, r)
+    return r.astype(np.uint16)
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def pack(codes: np.ndarray) -> np.ndarray:
+    codes = _c(codes.reshape(-1), np.uint8)
+    out = np.empty(codes.size // 2, np.uint8)
+    lib().lqo_pack(_p(codes), _p(out), C.c_int64(codes.size))
+    return out
+
+
+def unpack(packed: np.ndarray) -> np.ndarray:
+    packed = _c(packed.reshape(-1).view(np.uint8), np.uint8)
+    out = np.empty(packed.size * 2, np.uint8)
+    lib().lqo_unpack(_p(packed), _p(out), C.c_int64(out.size))
+    return out
+
+
+def dequant(packed, scales, zeros, N, K, group=128) -> np.ndarray:
+    packed = _c(packed.reshape(-1).view(np.uint8), np.uint8)
+    scales = _c(scales.reshape(-1), np.uint16)
+    zeros = _c(zeros.reshape(-1), np.uint16)
+    out = np.empty((N, K), np.uint16)
+    lib().lqo_dequant(_p(packed), _p(scales), _p(zeros), _p(out), C.c_int64(N), C.c_int64(K), C.c_int(group))
+    return out
+
+
+def a16w4_fwd(x, packed, scales, zeros, bias, M, N, K, group=128, want_f64=False):
+    x = _c(x.reshape(-1), np.uint16)
+    packed = _c(packed.reshape(-1).view(np.uint8), np.uint8)
+    scales = _c(scales.reshape(-1), np.uint16)
+    zeros = _c(zeros.reshape(-1), np.uint16)
+    bias = None if bias is None else _c(bias.reshape(-1), np.uint16)
+    y = np.empty((M, N), np.uint16)
+    y64 = np.empty((M, N), np.float64) if want_f64 else None
+    rc = lib().lqo_a16w4_fwd(_p(x), _p(packed), _p(scales), _p(zeros), _p(bias), _p(y), _p(y64), C.c_int64(M),
+                             C.c_int64(N), C.c_int64(K), C.c_int(group))
+    assert rc == 0
+    return (y, y64) if want_f64 else y
+
+
+def a16w4_dx(dy, packed, scales, zeros, M, N, K, group=128, want_f64=False):
+    dy = _c(dy.reshape(-1), np.uint16)
+    packed = _c(packed.reshape(-1).view(np.uint8), np.uint8)
+    scales = _c(scales.reshape(-1), np.uint16)
+    zeros = _c(zeros.reshape(-1), np.uint16)
+    dx = np.empty((M, K), np.uint16)
+    d64 = np.empty((M, K), np.float64) if want_f64 else None
+    rc = lib().lqo_a16w4_dx(_p(dy), _p(packed), _p(scales), _p(zeros), _p(dx), _p(d64), C.c_int64(M), C.c_int64(N),
+                            C.c_int64(K), C.c_int(group))
+    assert rc == 0
+    return (dx, d64) if want_f64 else dx
+
+
+def philox4x32_10(ctr, key):
+    ctr = np.asarray(ctr, np.uint32)
+    key = np.asarray(key, np.uint32)
+    out = np.empty(4, np.uint32)
+    lib().lqo_philox4x32_10(_p(ctr), _p(key), _p(out))
+    return out
+
+
+def philox_uniform(n, seed, offset=0) -> np.ndarray:
+    out = np.empty(n, np.float32)
+    lib().lqo_philox_uniform(_p(out), C.c_int64(n), C.c_uint64(seed), C.c_uint64(offset))
+    return out
+
+
+def requant(packed, scales, zeros, grad, lr, N, K, group=128, u=None, seed=0, offset=0) -> np.ndarray:
+    packed = _c(packed.reshape(-1).view(np.uint8), np.uint8)
+    scales = _c(scales.reshape(-1), np.uint16)
+    zeros = _c(zeros.reshape(-1), np.uint16)
+    grad = _c(grad.reshape(-1), np.uint16)
+    u = None if u is None else _c(u.reshape(-1), np.float32)
+    out = np.empty_like(packed)
+    lib().lqo_requant(_p(packed), _p(out), _p(scales), _p(zeros), _p(grad), C.c_float(lr), C.c_int64(N),
+                      C.c_int64(K), C.c_int(group), _p(u), C.c_uint64(seed), C.c_uint64(offset))
+    return out
+
+
+def a8w8(x, w, sx, sw, bias, M, N, K, want_y=True):
+    x = _c(x.reshape(-1), np.int8)
+    w = _c(w.reshape(-1), np.int8)
+    sx = _c(sx.reshape(-1), np.float32)
+    sw = _c(sw.reshape(-1), np.float32)
+    bias = None if bias is None else _c(bias.reshape(-1), np.uint16)
+    y = np.empty((M, N), np.uint16) if want_y else None
+    acc = np.empty((M, N), np.int32)
+    lib().lqo_a8w8(_p(x), _p(w), _p(sx), _p(sw), _p(bias), _p(y), _p(acc), C.c_int64(M), C.c_int64(N), C.c_int64(K))
+    return y, acc
+
+
+def act_quant_i8(x, clampv: float) -> np.ndarray:
+    x = _c(x.reshape(-1), np.uint16)
+    out = np.empty(x.size, np.int8)
+    lib().lqo_act_quant_i8(_p(x), C.c_float(clampv), _p(out), C.c_int64(x.size))
+    return out
+
+
+def gptq_to_native(qweight, N, K) -> np.ndarray:
+    qweight = _c(qweight.reshape(-1), np.int32)
+    out = np.empty(N * K // 2, np.uint8)
+    lib().lqo_gptq_to_native(_p(qweight), _p(out), C.c_int64(N), C.c_int64(K))
+    return out
+
+
+def native_to_gptq(packed, N, K) -> np.ndarray:
+    packed = _c(packed.reshape(-1).view(np.uint8), np.uint8)
+    out = np.empty((K // 8, N), np.int32)
+    lib().lqo_native_to_gptq(_p(packed), _p(out), C.c_int64(N), C.c_int64(K))
+    return out

@@ -1,0 +1,273 @@
+/*
+ * lq_oracle.c — CPU restatement of latentQ_LLM's quantized-linear hot path.
+ *
+ * TEST INFRASTRUCTURE ONLY. Nothing shipped by the package may link, load or
+ * call this file; it exists so that tests, the smoke check and the benchmark's
+ * CPU-baseline leg can compare the HIP kernels against an independent
+ * implementation. Plain C99 + OpenMP, no dependency on the package.
+ *
+ * Every function names the reference lines it follows (paths relative to the
+ * reference checkout). Pinning status (what, besides this file, fixes each
+ * result) is listed in the header comment of tests/test_oracle_pins.py; in
+ * short:
+ *   - pack/unpack, dequant, Philox4x32-10, int32 GEMM: pinned (known answers,
+ *     exhaustive checks, Random123 vectors, exact integer arithmetic);
+ *   - requant: the formula is this build's own (the reference has no such
+ *     function); pinned by an exact rational-arithmetic model and invariants;
+ *   - A8W8 bf16 epilogue: "parity unpinned" — the reference calls an external,
+ *     un-vendored cutlass kernel (torch_int, FWkey/torch-int-bf16, no pinned
+ *     version) whose rounding points cannot be read from the reference.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ---------------------------------------------------------------- bf16 -- */
+static inline float bf16_to_f32(uint16_t b) {
+    uint32_t u = ((uint32_t)b) << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* Round-to-nearest-even fp32 -> bf16, NaN kept quiet (what torch's
+ * c10::BFloat16 conversion does). */
+static inline uint16_t f32_to_bf16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7FFFu + lsb;
+    return (uint16_t)(u >> 16);
+}
+static inline float bf16_round(float f) { return bf16_to_f32(f32_to_bf16(f)); }
+
+uint16_t lqo_f32_to_bf16(float f) { return f32_to_bf16(f); }
+float lqo_bf16_to_f32(uint16_t b) { return bf16_to_f32(b); }
+
+/* ------------------------------------------------------- nibble packing -- */
+/* python_compress, utils/quant.py:4-9: byte = (c[2i] << 4) + c[2i+1]. */
+void lqo_pack(const uint8_t *codes, uint8_t *packed, int64_t n_codes) {
+    for (int64_t i = 0; i < n_codes / 2; ++i)
+        packed[i] = (uint8_t)(((codes[2 * i] & 0xF) << 4) | (codes[2 * i + 1] & 0xF));
+}
+/* python_decompress, utils/quant.py:12-19: hi = (b >> 4) % 16, lo = b % 16. */
+void lqo_unpack(const uint8_t *packed, uint8_t *codes, int64_t n_codes) {
+    for (int64_t i = 0; i < n_codes / 2; ++i) {
+        codes[2 * i] = (uint8_t)(packed[i] >> 4);
+        codes[2 * i + 1] = (uint8_t)(packed[i] & 0xF);
+    }
+}
+static inline unsigned code_at(const uint8_t *packed, int64_t i) {
+    uint8_t b = packed[i >> 1];
+    return (i & 1) ? (b & 0xFu) : (b >> 4);
+}
+
+/* ---------------------------------------------------------- dequantise -- */
+/* DeQfunc_4bit_g, utils/quant.py:66-72: (codes - zeros) * scales in bf16
+ * arithmetic: the int8 code is promoted to bf16, the difference is rounded to
+ * bf16, the product is rounded to bf16. */
+static inline float deq_elem(unsigned q, float s, float z) {
+    float d = bf16_round((float)q - z);
+    return bf16_round(d * s);
+}
+
+void lqo_dequant(const uint8_t *packed, const uint16_t *scales, const uint16_t *zeros, uint16_t *w_out,
+                 int64_t N, int64_t K, int group) {
+    int64_t total = N * K;
+#pragma omp parallel for schedule(static)
+    for (int64_t g = 0; g < total / group; ++g) {
+        float s = bf16_to_f32(scales[g]), z = bf16_to_f32(zeros[g]);
+        for (int64_t i = g * group; i < (g + 1) * group; ++i)
+            w_out[i] = f32_to_bf16(deq_elem(code_at(packed, i), s, z));
+    }
+}
+
+static float *dequant_f32(const uint8_t *packed, const uint16_t *scales, const uint16_t *zeros, int64_t N,
+                          int64_t K, int group) {
+    float *w = (float *)malloc(sizeof(float) * (size_t)(N * K));
+    if (!w) return NULL;
+    int64_t total = N * K;
+#pragma omp parallel for schedule(static)
+    for (int64_t g = 0; g < total / group; ++g) {
+        float s = bf16_to_f32(scales[g]), z = bf16_to_f32(zeros[g]);
+        for (int64_t i = g * group; i < (g + 1) * group; ++i) w[i] = deq_elem(code_at(packed, i), s, z);
+    }
+    return w;
+}
+
+/* --------------------------------------------------------- A16W4 GEMMs -- */
+/* QLinearFunctionW4.forward, utils/quant.py:116-121: Y = X . deq(W)^T (+ bias).
+ * Accumulates in double and rounds once to bf16 (the reference accumulates in
+ * fp32 inside cuBLAS with an unspecified order; comparisons use a tolerance).
+ * If y_f64 is non-NULL the unrounded sums are also stored there. */
+int lqo_a16w4_fwd(const uint16_t *x, const uint8_t *packed, const uint16_t *scales, const uint16_t *zeros,
+                  const uint16_t *bias, uint16_t *y, double *y_f64, int64_t M, int64_t N, int64_t K, int group) {
+    float *w = dequant_f32(packed, scales, zeros, N, K, group);
+    if (!w) return -1;
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        float *xf = (float *)malloc(sizeof(float) * (size_t)K);
+        for (int64_t k = 0; k < K; ++k) xf[k] = bf16_to_f32(x[m * K + k]);
+        for (int64_t n = 0; n < N; ++n) {
+            const float *wr = w + n * K;
+            double acc = 0.0;
+            for (int64_t k = 0; k < K; ++k) acc += (double)xf[k] * (double)wr[k];
+            if (bias) acc += (double)bf16_to_f32(bias[n]);
+            if (y_f64) y_f64[m * N + n] = acc;
+            y[m * N + n] = f32_to_bf16((float)acc);
+        }
+        free(xf);
+    }
+    free(w);
+    return 0;
+}
+
+/* QLinearFunctionW4.backward, utils/quant.py:136-140: dX = dY . deq(W). */
+int lqo_a16w4_dx(const uint16_t *dy, const uint8_t *packed, const uint16_t *scales, const uint16_t *zeros,
+                 uint16_t *dx, double *dx_f64, int64_t M, int64_t N, int64_t K, int group) {
+    float *w = dequant_f32(packed, scales, zeros, N, K, group);
+    if (!w) return -1;
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        double *acc = (double *)calloc((size_t)K, sizeof(double));
+        for (int64_t n = 0; n < N; ++n) {
+            double d = (double)bf16_to_f32(dy[m * N + n]);
+            const float *wr = w + n * K;
+            for (int64_t k = 0; k < K; ++k) acc[k] += d * (double)wr[k];
+        }
+        for (int64_t k = 0; k < K; ++k) {
+            if (dx_f64) dx_f64[m * K + k] = acc[k];
+            dx[m * K + k] = f32_to_bf16((float)acc[k]);
+        }
+        free(acc);
+    }
+    free(w);
+    return 0;
+}
+
+/* ------------------------------------------------------------- Philox -- */
+/* Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3",
+ * SC'11; Random123). Not part of the reference: the requantizer's noise
+ * source is this build's choice. */
+void lqo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+    uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3], k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; ++r) {
+        uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+        uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+        uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+        uint32_t n1 = (uint32_t)p1;
+        uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+        uint32_t n3 = (uint32_t)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+static inline float philox_u(int64_t i, uint64_t seed, uint64_t offset) {
+    uint64_t c = offset + (uint64_t)(i >> 2);
+    uint32_t ctr[4] = {(uint32_t)c, (uint32_t)(c >> 32), 0u, 0u};
+    uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    uint32_t o[4];
+    lqo_philox4x32_10(ctr, key, o);
+    return (float)(o[i & 3] >> 8) * 0x1p-24f;
+}
+
+void lqo_philox_uniform(float *out, int64_t n, uint64_t seed, uint64_t offset) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) out[i] = philox_u(i, seed, offset);
+}
+
+/* ------------------------------------------------------------ requant -- */
+/* Stochastic latent requantize (benchmark configuration 1). The reference has
+ * no function with this formula; its nearest relatives are Qfunc_4bit_g_res
+ * (utils/quant.py:45-63, Z = t/s + z then round) and the stochastic rounding
+ * round(x + U(-.5,.5)) of GradientQTensor.quant (utils/quant.py:867-871).
+ * Operation order, all fp32, each line one IEEE rounding:
+ *   w = bf16(bf16(q - z) * s);  t = fma(-lr, g, w);  v = t / s;  v = v + z;
+ *   v = v + u;  code = NaN or v < 0 -> 0, v > 15 -> 15, else floor(v).
+ * u == NULL selects the Philox stream. */
+void lqo_requant(const uint8_t *packed_in, uint8_t *packed_out, const uint16_t *scales, const uint16_t *zeros,
+                 const uint16_t *grad, float lr, int64_t N, int64_t K, int group, const float *u, uint64_t seed,
+                 uint64_t offset) {
+    int64_t total = N * K;
+#pragma omp parallel for schedule(static)
+    for (int64_t b = 0; b < total / 2; ++b) {
+        unsigned nib[2];
+        for (int h = 0; h < 2; ++h) {
+            int64_t i = 2 * b + h;
+            float s = bf16_to_f32(scales[i / group]), z = bf16_to_f32(zeros[i / group]);
+            float w = deq_elem(code_at(packed_in, i), s, z);
+            float t = fmaf(-lr, bf16_to_f32(grad[i]), w);
+            volatile float v = t / s;
+            v = v + z;
+            v = v + (u ? u[i] : philox_u(i, seed, offset));
+            float f = floorf(v);
+            nib[h] = (f != f || f < 0.0f) ? 0u : (f > 15.0f ? 15u : (unsigned)f);
+        }
+        packed_out[b] = (uint8_t)((nib[0] << 4) | nib[1]);
+    }
+}
+
+/* --------------------------------------------------------------- A8W8 -- */
+/* linear_a8_w8_bbf16_obf16 (external torch_int) + `* qscales` as used at
+ * utils/quant.py:268-271: acc = X8 . W8^T exactly in int32; the fused epilogue
+ * of this build is y = bf16((float(acc) * sx[m]) * sw[n] + bias[n]). */
+void lqo_a8w8(const int8_t *x, const int8_t *w, const float *sx, const float *sw, const uint16_t *bias, uint16_t *y,
+              int32_t *acc_out, int64_t M, int64_t N, int64_t K) {
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        for (int64_t n = 0; n < N; ++n) {
+            int32_t acc = 0;
+            const int8_t *xr = x + m * K, *wr = w + n * K;
+            for (int64_t k = 0; k < K; ++k) acc += (int32_t)xr[k] * (int32_t)wr[k];
+            if (acc_out) acc_out[m * N + n] = acc;
+            if (y) {
+                volatile float f = (float)acc * sx[m];
+                f = f * sw[n];
+                if (bias) f = f + bf16_to_f32(bias[n]);
+                y[m * N + n] = f32_to_bf16(f);
+            }
+        }
+    }
+}
+
+/* Activation quantizer of QLinearFunctionA8W8_dynamic.forward,
+ * utils/quant.py:264-266, on a bf16 input with a bf16-valued clamp:
+ * input*127. (bf16 product) / clampv (bf16 quotient), round half-even,
+ * clamp to [-128,127]. */
+void lqo_act_quant_i8(const uint16_t *x, float clampv, int8_t *x8, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) {
+        float a = bf16_round(bf16_to_f32(x[i]) * 127.0f);
+        float q = bf16_round(a / clampv);
+        float r = nearbyintf(q); /* default rounding mode: half to even */
+        if (r != r) r = 0.0f;
+        if (r < -128.0f) r = -128.0f;
+        if (r > 127.0f) r = 127.0f;
+        x8[i] = (int8_t)r;
+    }
+}
+
+/* ------------------------------------------------------- GPTQ layout ---- */
+/* QuantLinearGPTQ.pack, PTQ/quant/quant_linear.py:360-372: qweight[k/8, n]
+ * holds code(k, n) at bits 4*(k%8). */
+void lqo_gptq_to_native(const int32_t *qweight, uint8_t *packed, int64_t N, int64_t K) {
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t k = 0; k < K; k += 2) {
+            unsigned a = ((uint32_t)qweight[(k / 8) * N + n] >> (4 * (k % 8))) & 0xFu;
+            unsigned b = ((uint32_t)qweight[((k + 1) / 8) * N + n] >> (4 * ((k + 1) % 8))) & 0xFu;
+            packed[(n * K + k) / 2] = (uint8_t)((a << 4) | b);
+        }
+}
+void lqo_native_to_gptq(const uint8_t *packed, int32_t *qweight, int64_t N, int64_t K) {
+    memset(qweight, 0, sizeof(int32_t) * (size_t)(N * K / 8));
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t k = 0; k < K; ++k) {
+            uint32_t q = code_at(packed, n * K + k);
+            uint32_t *wd = (uint32_t *)&qweight[(k / 8) * N + n];
+            *wd |= q << (4 * (k % 8));
+        }
+}

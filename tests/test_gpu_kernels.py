@@ -1,0 +1,305 @@
+"""GPU parity tests: every kernel is called through the C ABI (latentq_llm_amd.ops -> ctypes ->
+liblatentq_hip.so) and compared with the CPU oracle on the same seeded inputs.
+
+Bars: bit-exact for codes, int32 accumulators, Philox draws, int8 activations and layout
+converters; rel-L2 <= 1e-2 (max-abs printed) for bf16 GEMM/GEMV outputs.
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests import util
+from tests.util import bits, from_bits, make_w4, randn_bf16, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def ops(hip_lib):
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from latentq_llm_amd import ops as _ops
+    return _ops
+
+
+@pytest.fixture(scope="module")
+def co():
+    from oracle import c_oracle
+    return c_oracle
+
+
+def dev(t):
+    return t.cuda()
+
+
+# ------------------------------------------------------------------ Philox --
+@pytest.mark.parametrize("n,seed,offset", [(1, 0, 0), (7, 1, 0), (4096, 0xDEADBEEFCAFEF00D, 12345),
+                                           (1000003, 42, 2**32 - 5), (64, 7, 2**64 - 3)])
+def test_philox_uniform_bit_exact(ops, co, n, seed, offset):
+    got = ops.philox_uniform(n, seed, offset).cpu().numpy()
+    want = co.philox_uniform(n, seed, offset)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert got.min() >= 0.0 and got.max() < 1.0
+
+
+# ----------------------------------------------------------------- requant --
+def _requant_case(ops, co, N, K, seed, lr, gstd, mode, tweak=None):
+    codes, packed, scales, zeros = make_w4(N, K, seed)
+    grad = randn_bf16((N, K), seed + 1, gstd)
+    if tweak:
+        scales, zeros, grad = tweak(scales, zeros, grad)
+    pseed, poff = 0x1234567 + seed, 1000 * seed
+    if mode == "inject":
+        g = torch.Generator().manual_seed(seed + 2)
+        u = torch.rand((N, K), generator=g, dtype=torch.float32)
+        want = co.requant(packed.numpy(), bits(scales), bits(zeros), bits(grad), lr, N, K, u=u.numpy())
+        got = ops.requant_sr(dev(packed), dev(scales), dev(zeros), dev(grad), lr, (N, K), u=dev(u))
+    else:
+        want = co.requant(packed.numpy(), bits(scales), bits(zeros), bits(grad), lr, N, K, seed=pseed, offset=poff)
+        got = ops.requant_sr(dev(packed), dev(scales), dev(zeros), dev(grad), lr, (N, K), seed=pseed, offset=poff)
+    got = got.cpu().numpy().view(np.uint8)
+    mism = int((got != want).sum())
+    assert mism == 0, f"{mism} of {want.size} bytes differ"
+    return got, packed.numpy().view(np.uint8)
+
+
+@pytest.mark.parametrize("mode", ["inject", "philox"])
+@pytest.mark.parametrize("N,K", [(1, 128), (3, 384), (64, 256), (257, 1024), (1000, 128)])
+def test_requant_bit_exact_small(ops, co, N, K, mode):
+    _requant_case(ops, co, N, K, seed=N + K, lr=1e-4, gstd=1e-3, mode=mode)
+
+
+@pytest.mark.parametrize("mode", ["inject", "philox"])
+def test_requant_bit_exact_large_update(ops, co, mode):
+    # updates of the order of a code step, so that many codes actually move
+    got, old = _requant_case(ops, co, 128, 512, seed=5, lr=1.0, gstd=2e-3, mode=mode)
+    assert (got != old).mean() > 0.2
+
+
+@pytest.mark.parametrize("mode", ["inject", "philox"])
+def test_requant_edge_parameters(ops, co, mode):
+    """Non-integer / large zeros, zero, negative, tiny and huge scales, inf/nan/huge gradients."""
+    def tweak(scales, zeros, grad):
+        s = scales.clone().reshape(-1)
+        z = zeros.clone().reshape(-1)
+        g = grad.clone()
+        special_s = [0.0, -0.003, 2.0 ** -60, 2.0 ** 60, 2.0 ** -120, 3e38, float("inf"), 1.0]
+        special_z = [7.5, 6.28125, 300.0, -3.0, 0.0, 15.0, 241.0, 1e6]
+        for i, v in enumerate(special_s):
+            s[i::17][: 4] = v
+        for i, v in enumerate(special_z):
+            z[3 + i::13][: 4] = v
+        flat = g.reshape(-1)
+        flat[5::97] = float("inf")
+        flat[11::89] = float("-inf")
+        flat[17::83] = float("nan")
+        flat[23::79] = 3e38
+        flat[29::73] = -3e38
+        flat[31::71] = 0.0
+        return s.reshape(scales.shape), z.reshape(zeros.shape), g
+    _requant_case(ops, co, 96, 512, seed=9, lr=0.5, gstd=1e-2, mode=mode, tweak=tweak)
+
+
+def test_requant_in_place_and_properties(ops, co):
+    """codes_out may alias codes_in; g = 0, u = 0.5 leaves codes unchanged; huge |g| saturates."""
+    N, K = 64, 512
+    codes, packed, scales, zeros = make_w4(N, K, 3)
+    d = [dev(t) for t in (packed, scales, zeros)]
+    zero_g = torch.zeros((N, K), dtype=torch.bfloat16, device="cuda")
+    half = torch.full((N, K), 0.5, dtype=torch.float32, device="cuda")
+    buf = d[0].clone()
+    ops.requant_sr(buf, d[1], d[2], zero_g, 1e-4, (N, K), u=half, out=buf)
+    assert torch.equal(buf, d[0])
+    big = torch.full((N, K), 1e30, dtype=torch.bfloat16, device="cuda")
+    lo = ops.requant_sr(d[0], d[1], d[2], big, 1.0, (N, K), u=half)
+    hi = ops.requant_sr(d[0], d[1], d[2], -big, 1.0, (N, K), u=half)
+    assert torch.all(lo.view(torch.uint8) == 0) and torch.all(hi.view(torch.uint8) == 0xFF)
+
+
+def test_requant_full_size_properties(ops, co):
+    """Benchmark size (8192 x 2048): Philox mode equals injected mode fed with the materialised
+    stream, idempotence at g = 0 / u = 0.5, and a sampled bit-exact comparison with the oracle."""
+    N, K = 8192, 2048
+    codes, packed, scales, zeros = make_w4(N, K, 11)
+    grad = randn_bf16((N, K), 12, 1e-3)
+    dp, ds, dz, dg = dev(packed), dev(scales), dev(zeros), dev(grad)
+    seed, off = 2024, 77
+    a = ops.requant_sr(dp, ds, dz, dg, 1e-4, (N, K), seed=seed, offset=off)
+    u = ops.philox_uniform(N * K, seed, off)
+    b = ops.requant_sr(dp, ds, dz, dg, 1e-4, (N, K), u=u)
+    assert torch.equal(a, b)
+    rows = 64  # oracle on a slice of rows (the update is row-local)
+    want = co.requant(packed[: rows * K // 2].numpy(), bits(scales[: rows * K // 128]), bits(zeros[: rows * K // 128]),
+                      bits(grad[:rows]), 1e-4, rows, K, seed=seed, offset=off)
+    assert np.array_equal(a[: rows * K // 2].cpu().numpy().view(np.uint8), want)
+    half = torch.full((N, K), 0.5, dtype=torch.float32, device="cuda")
+    same = ops.requant_sr(dp, ds, dz, torch.zeros_like(dg), 1e-4, (N, K), u=half)
+    assert torch.equal(same, dp)
+
+
+# ----------------------------------------------------------------- dequant --
+@pytest.mark.parametrize("N,K", [(16, 128), (48, 384), (300, 1024)])
+def test_dequant_bit_exact(ops, co, N, K):
+    codes, packed, scales, zeros = make_w4(N, K, N)
+    zeros.view(-1)[::5] = 7.5  # exercise the bf16 rounding of (q - z)
+    want = co.dequant(packed.numpy(), bits(scales), bits(zeros), N, K)
+    got = bits(ops.a16w4_dequant(dev(packed), dev(scales), dev(zeros), (N, K)))
+    assert np.array_equal(got, want)
+
+
+# --------------------------------------------------------------- A16W4 fwd --
+def _fwd_case(ops, co, M, N, K, seed, with_bias):
+    codes, packed, scales, zeros = make_w4(N, K, seed)
+    x = randn_bf16((M, K), seed + 1)
+    bias = randn_bf16((N,), seed + 2) if with_bias else None
+    _, want64 = co.a16w4_fwd(bits(x), packed.numpy(), bits(scales), bits(zeros), None if bias is None else bits(bias),
+                             M, N, K, want_f64=True)
+    got = ops.a16w4_forward(dev(x), dev(packed), dev(scales), dev(zeros), (N, K), None if bias is None else dev(bias))
+    torch.cuda.synchronize()
+    got = got.float().cpu()
+    want = torch.from_numpy(want64)
+    err = rel_l2(got, want)
+    print(f"fwd M={M} N={N} K={K} rel_l2={err:.3e} max_abs={float((got.double() - want).abs().max()):.3e}")
+    assert err <= REL_L2_TOL
+    return err
+
+
+@pytest.mark.parametrize("M,N,K,bias", [(17, 16, 128, False), (33, 48, 256, True), (128, 128, 128, False),
+                                        (129, 256, 384, True), (300, 272, 512, False), (1024, 3072, 768, True)])
+def test_a16w4_fwd_gemm(ops, co, M, N, K, bias):
+    _fwd_case(ops, co, M, N, K, seed=M + N + K, with_bias=bias)
+
+
+@pytest.mark.parametrize("M", [1, 2, 4, 5, 16])
+@pytest.mark.parametrize("N,K,bias", [(16, 128, False), (64, 640, True), (4096, 4096, False), (256, 11008, True)])
+def test_a16w4_fwd_gemv(ops, co, M, N, K, bias):
+    _fwd_case(ops, co, M, N, K, seed=M + N + K, with_bias=bias)
+
+
+def test_a16w4_fwd_identity_is_exact_dequant(ops, co):
+    """X = identity: every output is a single dequantised weight, so the GEMM result must equal
+    the reference dequantisation bit for bit (checks unpack + bf16 rounding through the kernel)."""
+    N, K = 384, 256
+    codes, packed, scales, zeros = make_w4(N, K, 21)
+    x = torch.eye(K, dtype=torch.bfloat16)
+    got = ops.a16w4_forward(dev(x), dev(packed), dev(scales), dev(zeros), (N, K))
+    want = co.dequant(packed.numpy(), bits(scales), bits(zeros), N, K)  # [N, K]
+    assert np.array_equal(bits(got).T, want)
+
+
+def test_a16w4_fwd_integer_exact(ops, co):
+    """scales = 1, zeros = 0, small-integer X: the result is an exact small integer... in fp32;
+    checks the full contraction (every k reaches the right accumulator) without tolerance
+    as long as the sums stay below 2^8 (bf16-exact)."""
+    M, N, K = 64, 32, 128
+    g = torch.Generator().manual_seed(5)
+    codes = torch.randint(0, 2, (N, K), generator=g, dtype=torch.uint8)
+    packed = util.pack_codes(codes)
+    scales = torch.ones(N * K // 128, 1, dtype=torch.bfloat16)
+    zeros = torch.zeros(N * K // 128, 1, dtype=torch.bfloat16)
+    x = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16)
+    got = ops.a16w4_forward(dev(x), dev(packed), dev(scales), dev(zeros), (N, K)).float().cpu()
+    want = x.float() @ codes.float().t()
+    assert want.abs().max() < 256
+    assert torch.equal(got, want)
+
+
+# ---------------------------------------------------------------- A16W4 dX --
+@pytest.mark.parametrize("M,N,K", [(17, 64, 128), (64, 128, 256), (130, 192, 384), (300, 320, 512), (1024, 3072, 768),
+                                   (4, 128, 256)])
+def test_a16w4_dx(ops, co, M, N, K):
+    codes, packed, scales, zeros = make_w4(N, K, M + N)
+    dy = randn_bf16((M, N), 7)
+    _, want64 = co.a16w4_dx(bits(dy), packed.numpy(), bits(scales), bits(zeros), M, N, K, want_f64=True)
+    got = ops.a16w4_dx(dev(dy), dev(packed), dev(scales), dev(zeros), (N, K)).float().cpu()
+    want = torch.from_numpy(want64)
+    err = rel_l2(got, want)
+    print(f"dx M={M} N={N} K={K} rel_l2={err:.3e} max_abs={float((got.double() - want).abs().max()):.3e}")
+    assert err <= REL_L2_TOL
+
+
+def test_a16w4_dx_identity_is_exact_dequant(ops, co):
+    N, K = 256, 384
+    codes, packed, scales, zeros = make_w4(N, K, 22)
+    dy = torch.eye(N, dtype=torch.bfloat16)
+    got = ops.a16w4_dx(dev(dy), dev(packed), dev(scales), dev(zeros), (N, K))
+    want = co.dequant(packed.numpy(), bits(scales), bits(zeros), N, K)
+    assert np.array_equal(bits(got), want)
+
+
+def test_a16w4_adjoint_identity(ops):
+    """<X W^T, dY> == <X, dY W> up to bf16 output rounding, at the OPT-125m fc1 shape."""
+    M, N, K = 1024, 3072, 768
+    codes, packed, scales, zeros = make_w4(N, K, 31)
+    x, dy = randn_bf16((M, K), 32), randn_bf16((M, N), 33)
+    dp, ds, dz = dev(packed), dev(scales), dev(zeros)
+    y = ops.a16w4_forward(dev(x), dp, ds, dz, (N, K)).double().cpu()
+    dx = ops.a16w4_dx(dev(dy), dp, ds, dz, (N, K)).double().cpu()
+    lhs = float((y * dy.double()).sum())
+    rhs = float((x.double() * dx).sum())
+    scale = float(y.norm() * dy.double().norm())
+    assert abs(lhs - rhs) <= 1e-3 * scale
+
+
+# -------------------------------------------------------------------- A8W8 --
+@pytest.mark.parametrize("M,N,K,bias", [(17, 16, 128, False), (64, 128, 256, True), (130, 272, 384, False),
+                                        (300, 512, 1024, True), (2048, 2048, 2048, False)])
+def test_a8w8(ops, co, M, N, K, bias):
+    g = torch.Generator().manual_seed(M + N + K)
+    x8 = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
+    w8 = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    sx = (torch.randn(M, generator=g) * 0.05).abs() + 1e-4
+    sw = (torch.randn(N, generator=g) * 0.01).abs() + 1e-5
+    b = randn_bf16((N,), 3) if bias else None
+    want_y, want_acc = co.a8w8(x8.numpy(), w8.numpy(), sx.numpy(), sw.numpy(), None if b is None else bits(b), M, N, K)
+    y, acc = ops.a8w8_forward(dev(x8), dev(w8), dev(sx), dev(sw), None if b is None else dev(b), want_acc=True)
+    assert np.array_equal(acc.cpu().numpy(), want_acc), "int32 accumulators must be bit-exact"
+    err = rel_l2(y.float().cpu(), from_bits(want_y).float())
+    print(f"a8w8 M={M} N={N} K={K} rel_l2={err:.3e}")
+    assert err <= REL_L2_TOL
+    # the fused epilogue is deterministic fp32 arithmetic: it matches the oracle bit for bit as well
+    assert np.array_equal(bits(y), want_y)
+
+
+def test_a8w8_extreme_accumulators(ops, co):
+    """All +-127 over K = 8192: |acc| = 127*127*8192 = 132 128 768 < 2^31."""
+    M, N, K = 32, 32, 8192
+    x8 = torch.full((M, K), 127, dtype=torch.int8)
+    w8 = torch.full((N, K), -127, dtype=torch.int8)
+    w8[::2] = 127
+    one = torch.ones(M), torch.ones(N)
+    _, acc = ops.a8w8_forward(dev(x8), dev(w8), dev(one[0]), dev(one[1]), want_acc=True)
+    acc = acc.cpu()
+    assert int(acc[0, 0]) == 127 * 127 * 8192 and int(acc[0, 1]) == -127 * 127 * 8192
+
+
+def test_act_quant_bit_exact(ops, co):
+    x = randn_bf16((333, 77), 1, 2.0)
+    clampv = float(x.max())
+    got = ops.act_quant_i8(dev(x), torch.tensor([clampv], device="cuda")).cpu().numpy()
+    want = co.act_quant_i8(bits(x), clampv).reshape(got.shape)
+    assert np.array_equal(got, want)
+
+
+# ------------------------------------------------------------------ repack --
+@pytest.mark.parametrize("N,K", [(16, 128), (100, 384), (4096, 1024)])
+def test_repack_round_trip(ops, co, N, K):
+    codes, packed, _, _ = make_w4(N, K, N + 1)
+    gptq = co.native_to_gptq(packed.numpy(), N, K)
+    got = ops.repack_native_to_gptq(dev(packed), (N, K)).cpu().numpy()
+    assert np.array_equal(got, gptq)
+    back = ops.repack_gptq_to_native(dev(torch.from_numpy(gptq)), (N, K)).cpu()
+    assert torch.equal(back, packed)
+
+
+# ------------------------------------------------------------- error paths --
+def test_error_reporting(ops):
+    from latentq_llm_amd._C import LatentQError
+    N, K = 16, 128
+    codes, packed, scales, zeros = make_w4(N, K, 1)
+    x = randn_bf16((32, K), 2)
+    with pytest.raises(LatentQError, match="CPU"):
+        ops.a16w4_forward(x, packed, scales, zeros, (N, K))
+    with pytest.raises(ValueError):
+        ops.a16w4_forward(dev(x)[:, :64].contiguous(), dev(packed), dev(scales), dev(zeros), (N, K))
