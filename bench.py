@@ -1,0 +1,276 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one pass of the A16W4 Llama-2-7B MLP block at 4 x 512 = 2048 bf16 tokens:
+forward  down(silu(gate(x)) * up(x))  and the dX backward through all three projections
+(six dequant-GEMMs, 1108.1 GFLOP), with synthetic seeded weights and activations already
+resident in HBM. The headline value is GEMM TFLOP/s of that step. The same JSON line also
+carries the kernel roofline of the dominant kernel (measured with HIP events on the launch
+stream), HBM GB/s of the requantizer and of the decode GEMV sweep, the A8W8 GEMM rate, and
+the CPU baseline (the torch restatement of the reference's dequant path on the host cores).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16 = 2.5e15   # dense bf16 MFMA, flop/s
+PEAK_I8 = 5.0e15     # dense int8 MFMA, op/s
+PEAK_HBM = 8.0e12    # byte/s
+
+TOKENS, HID, FFN = 2048, 4096, 11008
+GROUP = 128
+
+
+def synth_w4(N, K, seed, device):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    codes = torch.randint(0, 256, (N * K // 2,), generator=g, dtype=torch.uint8).view(torch.int8)
+    scales = (torch.randn(N * K // GROUP, 1, generator=g) * 0.02).abs().div(7).to(torch.bfloat16)
+    scales = torch.where(scales == 0, torch.full_like(scales, 2.0 ** -10), scales)
+    zeros = torch.randint(6, 10, (N * K // GROUP, 1), generator=g).to(torch.bfloat16)
+    return codes.to(device), scales.to(device), zeros.to(device)
+
+
+def event_time(fn, iters, warm=2):
+    """Average seconds per call of fn(), HIP events on the current (= launch) stream."""
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / iters
+
+
+def graph_time(calls, replays=20):
+    """Average seconds per kernel for launch-latency-scale kernels: the calls (one per rotating
+    buffer set) are captured into one HIP graph so that launches are back to back, and the
+    graph is replayed between two HIP events on the replay stream."""
+    for c in calls:
+        c()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for c in calls:
+            c()
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / (replays * len(calls))
+
+
+class MLPBlock:
+    """A16W4 Llama-2-7B MLP (gate/up 11008x4096, down 4096x11008) on the HIP kernels."""
+
+    def __init__(self, device):
+        from latentq_llm_amd import ops
+        self.ops = ops
+        self.gate = synth_w4(FFN, HID, 1, device)
+        self.up = synth_w4(FFN, HID, 2, device)
+        self.down = synth_w4(HID, FFN, 3, device)
+        g = torch.Generator(device="cpu").manual_seed(4)
+        self.x = torch.randn(TOKENS, HID, generator=g).to(torch.bfloat16).to(device)
+        self.dy = torch.randn(TOKENS, HID, generator=g).to(torch.bfloat16).to(device)
+
+    def step(self):
+        o = self.ops
+        g = o.a16w4_forward(self.x, *self.gate, (FFN, HID))
+        u = o.a16w4_forward(self.x, *self.up, (FFN, HID))
+        sg = torch.sigmoid(g.float())
+        act = (g.float() * sg)
+        h = (act.to(torch.bfloat16) * u)
+        y = o.a16w4_forward(h, *self.down, (HID, FFN))
+        dh = o.a16w4_dx(self.dy, *self.down, (HID, FFN))
+        du = dh * act.to(torch.bfloat16)
+        dg = (dh.float() * u.float() * (sg * (1.0 + g.float() * (1.0 - sg)))).to(torch.bfloat16)
+        dx = o.a16w4_dx(dg, *self.gate, (FFN, HID))
+        dx += o.a16w4_dx(du, *self.up, (FFN, HID))
+        return y, dx
+
+
+MLP_FLOP = 6 * 2 * TOKENS * HID * FFN  # 1 108.1 GFLOP
+
+
+def bench_requant(device):
+    from latentq_llm_amd import ops
+    N, K = 8192, 2048
+    nb = 8  # 8 x 50 MB of distinct buffers > 256 MB of last-level cache
+    sets = []
+    for i in range(nb):
+        p, s, z = synth_w4(N, K, 10 + i, device)
+        g = (torch.randn(N, K, device=device) * 1e-3).to(torch.bfloat16)
+        sets.append((p, s, z, g, torch.empty_like(p)))
+    calls = [(lambda t=t, i=i: ops.requant_sr(t[0], t[1], t[2], t[3], 1e-4, (N, K), seed=7, offset=i, out=t[4]))
+             for i, t in enumerate(sets)]
+    sec = graph_time(calls)
+    nbytes = N * K // 2 * 2 + N * K * 2 + 4 * N * K // GROUP
+    return {"shape": [N, K], "us": sec * 1e6, "GB/s": nbytes / sec / 1e9, "frac_hbm": nbytes / sec / PEAK_HBM,
+            "bytes": nbytes, "noise": "in-kernel Philox4x32-10"}
+
+
+def bench_gemv(device):
+    from latentq_llm_amd import ops
+    out = []
+    for (N, K) in [(4096, 4096), (11008, 4096), (4096, 11008)]:
+        nb = int(300e6 // (N * K // 2)) + 1
+        ws = [synth_w4(N, K, 20 + i, device) for i in range(nb)]
+        for M in (1, 4, 16):
+            x = torch.randn(M, K, device=device).to(torch.bfloat16)
+            ys = [torch.empty(M, N, device=device, dtype=torch.bfloat16) for _ in range(nb)]
+            calls = [(lambda w=w, y=y: ops.a16w4_forward(x, *w, (N, K), out=y)) for w, y in zip(ws, ys)]
+            sec = graph_time(calls)
+            nbytes = N * K // 2 + 4 * N * K // GROUP + 2 * M * K + 2 * M * N
+            out.append({"N": N, "K": K, "M": M, "us": sec * 1e6, "GB/s": nbytes / sec / 1e9,
+                        "frac_hbm": nbytes / sec / PEAK_HBM})
+        del ws
+    return out
+
+
+def bench_a8w8(device):
+    from latentq_llm_amd import ops
+    M = TOKENS
+    out = []
+    for (N, K) in [(2048, 2048), (8192, 2048), (2048, 8192)]:
+        x8 = torch.randint(-127, 128, (M, K), device=device, dtype=torch.int8)
+        w8 = torch.randint(-127, 128, (N, K), device=device, dtype=torch.int8)
+        sx = (torch.randn(M, device=device) * 0.05).abs()
+        sw = (torch.randn(N, device=device) * 0.01).abs()
+        sec = event_time(lambda: ops.a8w8_forward(x8, w8, sx, sw), 20)
+        out.append({"M": M, "N": N, "K": K, "us": sec * 1e6, "TOP/s": 2 * M * N * K / sec / 1e12,
+                    "frac_mfma_i8": 2 * M * N * K / sec / PEAK_I8})
+    return out
+
+
+def cpu_baseline():
+    """The reference's CPU path (nibble unpack -> bf16 group dequant -> bf16 torch.mm), restated in
+    oracle/torch_ref.py, on the host cores: the whole MLP step at 2048 tokens, fwd + dX."""
+    from oracle import torch_ref as tr
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    gate = [t.cpu() for t in synth_w4(FFN, HID, 1, "cpu")] + [(FFN, HID)]
+    up = [t.cpu() for t in synth_w4(FFN, HID, 2, "cpu")] + [(FFN, HID)]
+    down = [t.cpu() for t in synth_w4(HID, FFN, 3, "cpu")] + [(HID, FFN)]
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(TOKENS, HID, generator=g).to(torch.bfloat16)
+    dy = torch.randn(TOKENS, HID, generator=g).to(torch.bfloat16)
+
+    def step():
+        y, (gg, uu, h) = tr.llama_mlp_forward(x, gate, up, down)
+        dh = dy.mm(tr.dequant_4bit_g(*down))
+        sg = torch.sigmoid(gg.float())
+        du = dh * (gg.float() * sg).to(torch.bfloat16)
+        dg = (dh.float() * uu.float() * (sg * (1.0 + gg.float() * (1.0 - sg)))).to(torch.bfloat16)
+        dx = dg.mm(tr.dequant_4bit_g(*gate)) + du.mm(tr.dequant_4bit_g(*up))
+        return y, dx
+
+    step()  # warm-up (thread pool, allocator)
+    runs, t0 = 0, time.time()
+    while runs < 3 or (time.time() - t0 < 10.0 and runs < 10):
+        step()
+        runs += 1
+    sec = (time.time() - t0) / runs
+    return {"value": MLP_FLOP / sec / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"whole workload ({TOKENS} tokens, fwd + dX of the MLP block), 1 warm-up + {runs} timed runs, "
+                      f"torch {torch.__version__} CPU bf16 mm, {sec:.2f} s per step",
+            "cpu": _cpu_model()}
+
+
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only-mlp", action="store_true", help="skip the side measurements (requant, GEMV, A8W8)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (no sharding, no collectives); use --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP kernels have no CPU fallback")
+    from latentq_llm_amd import _C
+    _C.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    blk = MLPBlock(dev)
+    for _ in range(args.warmup):
+        blk.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        blk.step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    value = MLP_FLOP / dt / 1e12
+
+    # Dominant kernel: the dequant-GEMM. Per-launch duration from HIP events on the launch stream.
+    o = blk.ops
+    h = torch.randn(TOKENS, FFN, device=dev).to(torch.bfloat16)
+    kern = {}
+    for name, fn, fl in [
+        ("fwd_gate_up", lambda: o.a16w4_forward(blk.x, *blk.gate, (FFN, HID)), 2 * TOKENS * HID * FFN),
+        ("fwd_down", lambda: o.a16w4_forward(h, *blk.down, (HID, FFN)), 2 * TOKENS * HID * FFN),
+        ("dx_gate_up", lambda: o.a16w4_dx(h, *blk.gate, (FFN, HID)), 2 * TOKENS * HID * FFN),
+        ("dx_down", lambda: o.a16w4_dx(blk.dy, *blk.down, (HID, FFN)), 2 * TOKENS * HID * FFN),
+    ]:
+        sec = event_time(fn, 20)
+        kern[name] = {"us": sec * 1e6, "TFLOP/s": fl / sec / 1e12, "frac_mfma_bf16": fl / sec / PEAK_BF16}
+    # weighted by launches per step: 2 fwd gate/up, 1 fwd down, 2 dx gate/up, 1 dx down
+    tot = 2 * kern["fwd_gate_up"]["us"] + kern["fwd_down"]["us"] + 2 * kern["dx_gate_up"]["us"] + kern["dx_down"]["us"]
+    avg_us = tot / 6
+    achieved = 2 * TOKENS * HID * FFN / (avg_us * 1e-6) / 1e12
+    roofline = {"bound": "mfma", "kernel": "gemm_kernel (A16W4 dequant-GEMM, fwd and dX instantiations)",
+                "achieved": achieved, "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": achieved * 1e12 / PEAK_BF16,
+                "avg_launch_us": avg_us, "flop_per_launch": 2 * TOKENS * HID * FFN, "traffic": None}
+
+    line = {
+        "metric": "A16W4 GEMM TFLOP/s (7B MLP, 2048 tok)", "value": value, "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[2]: A16W4 Llama-2-7B MLP block, 4x512=2048 bf16 tokens, forward + dX "
+                               "through gate/up (11008x4096) and down (4096x11008), int4 group 128",
+                   "tokens": TOKENS, "flop_per_step": MLP_FLOP},
+        "roofline": roofline,
+        "gemm_kernels": kern,
+    }
+    if not args.only_mlp:
+        del blk
+        torch.cuda.empty_cache()
+        line["requant"] = bench_requant(dev)
+        line["gemv"] = bench_gemv(dev)
+        line["a8w8"] = bench_a8w8(dev)
+    line["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -69,7 +69,7 @@ def philox_uniform(n: int, seed: int, offset: int = 0, device="cuda"):
     return out
 
 
-def a16w4_forward(x, codes, scales, zeros, shape, bias=None):
+def a16w4_forward(x, codes, scales, zeros, shape, bias=None, out=None):
     """Y[M,N] = X[M,K] . deq(W)[N,K]^T (+ bias) in bf16 with fp32 accumulation."""
     N, K = shape
     _chk(x, torch.bfloat16, "x")
@@ -82,7 +82,13 @@ def a16w4_forward(x, codes, scales, zeros, shape, bias=None):
         if bias.numel() != N:
             raise ValueError("bias must have N elements")
     M = x.shape[0]
-    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    if out is None:
+        y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    else:
+        _chk(out, torch.bfloat16, "out")
+        if tuple(out.shape) != (M, N):
+            raise ValueError(f"out must be [{M},{N}]")
+        y = out
     if M == 0:
         return y
     with torch.cuda.device(x.device):
@@ -91,7 +97,7 @@ def a16w4_forward(x, codes, scales, zeros, shape, bias=None):
     return y
 
 
-def a16w4_dx(dy, codes, scales, zeros, shape):
+def a16w4_dx(dy, codes, scales, zeros, shape, out=None):
     """dX[M,K] = dY[M,N] . deq(W)[N,K]."""
     N, K = shape
     _chk(dy, torch.bfloat16, "dy")
@@ -100,7 +106,13 @@ def a16w4_dx(dy, codes, scales, zeros, shape):
     _codes_ok(codes, N, K)
     _qparam_ok(scales, zeros, N, K)
     M = dy.shape[0]
-    dx = torch.empty((M, K), dtype=torch.bfloat16, device=dy.device)
+    if out is None:
+        dx = torch.empty((M, K), dtype=torch.bfloat16, device=dy.device)
+    else:
+        _chk(out, torch.bfloat16, "out")
+        if tuple(out.shape) != (M, K):
+            raise ValueError(f"out must be [{M},{K}]")
+        dx = out
     if M == 0:
         return dx
     with torch.cuda.device(dy.device):

@@ -160,3 +160,10 @@ def native_to_gptq(packed, N, K) -> np.ndarray:
     out = np.empty((K // 8, N), np.int32)
     lib().lqo_native_to_gptq(_p(packed), _p(out), C.c_int64(N), C.c_int64(K))
     return out
+
+
+def markstein_check(seed: int, per_scale: int):
+    """(quotient mismatches, code mismatches, cases) of the reciprocal-based divide; see lq_oracle.c."""
+    qm, cm, n = C.c_int64(0), C.c_int64(0), C.c_int64(0)
+    lib().lqo_markstein_check(C.c_uint32(seed), C.c_int(per_scale), C.byref(qm), C.byref(cm), C.byref(n))
+    return qm.value, cm.value, n.value

@@ -271,3 +271,62 @@ void lqo_native_to_gptq(const uint8_t *packed, int32_t *qweight, int64_t N, int6
             *wd |= q << (4 * (k % 8));
         }
 }
+
+/* ------------------------------------------------ reciprocal-based divide -- */
+/* The HIP requantizer replaces t / s by q0 = t*r, e = fma(-q0, s, t), q = fma(e, r, q0) with
+ * r = RN(1/s) (Markstein's correction) whenever |s| is in [2^-40, 2^40] and |t| < 2^60. This
+ * routine sweeps EVERY bf16 scale in that range (both signs) against `per_scale` pseudo-random
+ * numerators and counts (a) quotients that differ from IEEE t/s when |t| >= 2^-60 and (b) final
+ * codes floor(clamp((q + z) + u)) that differ for any t, including tiny and zero ones. Both
+ * counts must be zero for the substitution to be exact. */
+static inline uint32_t xorshift32(uint32_t *st) {
+    uint32_t x = *st;
+    x ^= x << 13; x ^= x >> 17; x ^= x << 5;
+    return *st = x;
+}
+void lqo_markstein_check(uint32_t seed, int per_scale, int64_t *quot_mismatch, int64_t *code_mismatch,
+                         int64_t *cases) {
+    int64_t qm = 0, cm = 0, n = 0;
+    uint32_t st = seed ? seed : 1u;
+    for (uint32_t b = 0; b < 0x10000u; ++b) {
+        float s = bf16_to_f32((uint16_t)b);
+        float as = fabsf(s);
+        if (!(as >= 0x1p-40f && as <= 0x1p40f)) continue;
+        volatile float r = 1.0f / s;
+        for (int i = 0; i < per_scale; ++i) {
+            uint32_t m = xorshift32(&st);
+            int e = (int)(xorshift32(&st) % 180u) - 120; /* 2^-120 .. 2^59 */
+            float t = ldexpf(1.0f + (float)(m >> 9) * 0x1p-23f, e);
+            if (m & 1u) t = -t;
+            if (i == 0) t = 0.0f;
+            if (i == 1) t = 0x1p-149f;
+            if (i == 2) t = -0x1p-130f;
+            if (!(fabsf(t) < 0x1p60f)) continue;
+            volatile float q0 = t * r;
+            volatile float ee = fmaf(-q0, s, t);
+            volatile float q = fmaf(ee, r, q0);
+            volatile float ref = t / s;
+            ++n;
+            if (fabsf(t) >= 0x1p-60f) {
+                uint32_t a, c;
+                float qa = q, qc = ref;
+                memcpy(&a, &qa, 4);
+                memcpy(&c, &qc, 4);
+                if (a != c) ++qm;
+            }
+            float z = (float)(xorshift32(&st) % 16u);
+            float u = (float)(xorshift32(&st) >> 8) * 0x1p-24f;
+            if (i < 3) u = 0.0f;
+            volatile float v1 = q + z, v2 = ref + z;
+            v1 = v1 + u;
+            v2 = v2 + u;
+            float f1 = floorf(v1), f2 = floorf(v2);
+            unsigned c1 = (f1 != f1 || f1 < 0.0f) ? 0u : (f1 > 15.0f ? 15u : (unsigned)f1);
+            unsigned c2 = (f2 != f2 || f2 < 0.0f) ? 0u : (f2 > 15.0f ? 15u : (unsigned)f2);
+            if (c1 != c2) ++cm;
+        }
+    }
+    *quot_mismatch = qm;
+    *code_mismatch = cm;
+    *cases = n;
+}

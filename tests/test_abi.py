@@ -1,0 +1,73 @@
+"""CPU tests of the C-ABI boundary: the shared library loads, exports every symbol that
+include/latentq.h declares, and rejects bad arguments with an error code and message before
+touching a device. No kernel is launched here."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "latentq.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(hip_lib):
+    syms = declared_symbols()
+    assert len(syms) >= 11
+    for s in syms:
+        assert hasattr(hip_lib, s), f"{s} declared in include/latentq.h but not exported"
+
+
+def test_binding_covers_header(hip_lib):
+    from latentq_llm_amd import _C
+    assert set(_C.SIGNATURES) | {"lq_last_error"} == set(declared_symbols())
+    assert hip_lib.lq_abi_version() == _C.ABI_VERSION
+
+
+def test_bad_arguments_are_rejected_without_a_gpu(hip_lib):
+    from latentq_llm_amd import _C
+    lib = hip_lib
+    assert lib.lq_requant_sr(None, None, None, None, None, 0.0, 8, 128, 128, None, 0, 0, None) == -1
+    assert b"null pointer" in lib.lq_last_error()
+    buf = (C.c_char * 4096)()
+    p = C.cast(buf, C.c_void_p)
+    assert lib.lq_requant_sr(p, p, p, p, p, 0.0, 8, 100, 128, None, 0, 0, None) == -1
+    assert b"multiple of 128" in lib.lq_last_error()
+    assert lib.lq_requant_sr(p, p, p, p, p, 0.0, 8, 128, 64, None, 0, 0, None) == -1
+    assert b"group" in lib.lq_last_error()
+    assert lib.lq_a16w4_fwd(p, p, p, p, None, p, 4, 24, 128, 128, None) == -1
+    assert b"multiple of 16" in lib.lq_last_error()
+    assert lib.lq_a16w4_dx(p, p, p, p, p, 4, 48, 128, 128, None) == -1
+    assert b"multiple of 64" in lib.lq_last_error()
+    assert lib.lq_a8w8_fwd(p, p, p, p, None, p, None, 4, 16, 100, None) == -1
+    misaligned = C.c_void_p(p.value + 2)
+    assert lib.lq_a16w4_fwd(misaligned, p, p, p, None, p, 32, 16, 128, 128, None) == -1
+    assert b"aligned" in lib.lq_last_error()
+    with pytest.raises(_C.LatentQError, match="lq_a16w4_dequant"):
+        _C.call("lq_a16w4_dequant", None, None, None, None, 1, 128, 128, None)
+
+
+def test_ops_refuse_cpu_tensors(hip_lib):
+    import torch
+    from latentq_llm_amd import _C, ops
+    x = torch.zeros(4, 128, dtype=torch.bfloat16)
+    codes = torch.zeros(16 * 64, dtype=torch.int8)
+    sz = torch.zeros(16, 1, dtype=torch.bfloat16)
+    with pytest.raises(_C.LatentQError, match="no CPU fallback"):
+        ops.a16w4_forward(x, codes, sz, sz, (16, 128))
+
+
+def test_product_does_not_import_the_oracle():
+    """The package must never route through oracle/ (test infrastructure)."""
+    pkg = os.path.join(ROOT, "latentq_llm_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                src = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", src, flags=re.M), f
+                assert "lq_oracle" not in src, f

@@ -1,0 +1,294 @@
+"""CPU tests that pin the oracle (oracle/lq_oracle.c, oracle/torch_ref.py) WITHOUT retyping it.
+
+The reference ships no tests, golden vectors or fixtures for this path, so each oracle
+function is pinned by what the mathematics fixes:
+
+  pack / unpack          known answers worked out by hand from the two-line rule, exhaustive
+                         round trip over all 256 bytes, little-endian word 0x67452301
+  dequant                torch's own bf16 tensor arithmetic (the arithmetic the reference runs),
+                         an exact rational model with explicit round-to-nearest-even,
+                         the GPTQ identity (q - (z_stored + 1)) * s
+  A16W4 fwd / dX         torch float64 matmul on the dequantised matrix, the adjoint identity,
+                         identity activations, bf16 torch.mm (the reference's CPU path) to tolerance
+  Philox4x32-10          the three Random123 known-answer vectors; uniform mapping range/grid
+  requant                exact rational model (fractions.Fraction, own RNE rounding), invariants
+                         (idempotence, floor at u = 0, saturation), unbiasedness
+  reciprocal divide      exhaustive sweep over every bf16 scale (lqo_markstein_check)
+  A8W8 int32             numpy int64 matmul; extreme value 127*127*8192
+  A8W8 bf16 epilogue     "parity unpinned": the reference's epilogue lives in the external,
+                         un-vendored torch_int (FWkey/torch-int-bf16, no pinned version); only the
+                         closed form bf16((acc*sx)*sw + bias) of this build is checked
+  act quant              torch's bf16 tensor arithmetic
+  GPTQ <-> native        defining bit formula, brute force
+"""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from oracle import torch_ref as tr
+from tests.util import bits, from_bits, make_w4, pack_codes, randn_bf16, rel_l2
+
+
+# ------------------------------------------------------------ exact rounding --
+def rn(x: Fraction, mant_bits: int, emin: int = -126) -> Fraction:
+    """Round an exact rational to a binary float with `mant_bits` significand bits (incl. the
+    hidden one), round-to-nearest-even, gradual underflow below 2^emin."""
+    if x == 0:
+        return Fraction(0)
+    sign = -1 if x < 0 else 1
+    a = abs(x)
+    e = a.numerator.bit_length() - a.denominator.bit_length()
+    if Fraction(2) ** e > a:
+        e -= 1
+    if Fraction(2) ** (e + 1) <= a:
+        e += 1
+    e = max(e, emin)
+    quantum = Fraction(2) ** (e - (mant_bits - 1))
+    n = a / quantum
+    fl = n.numerator // n.denominator
+    rem = n - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        fl += 1
+    return sign * fl * quantum
+
+
+def f32(x):
+    return rn(x, 24)
+
+
+def bf16(x):
+    return rn(x, 8)
+
+
+def frac_of_bits(b: int) -> Fraction:
+    return Fraction(float(co.bf16_bits_to_f32(np.array([b], np.uint16))[0]))
+
+
+def test_rn_helper_against_numpy():
+    rng = np.random.default_rng(0)
+    for v in rng.standard_normal(200) * 10.0 ** rng.integers(-20, 20, 200):
+        assert float(f32(Fraction(float(v)))) == float(np.float32(v))
+    ties = [Fraction(1) + Fraction(1, 2 ** 8), Fraction(1) + Fraction(3, 2 ** 8), Fraction(257, 2), Fraction(259, 2)]
+    assert [bf16(t) for t in ties] == [Fraction(1), Fraction(1) + Fraction(1, 64), Fraction(128), Fraction(130)]
+
+
+# -------------------------------------------------------------------- packing --
+def test_pack_known_answers():
+    assert list(co.pack(np.array([15, 3, 8, 0, 7, 15], np.uint8))) == [0xF3, 0x80, 0x7F]
+    assert co.pack(np.arange(8, dtype=np.uint8)).view("<u4")[0] == 0x67452301
+    t = tr.compress(torch.tensor([15, 3, 8, 0, 7, 15], dtype=torch.uint8))
+    assert t.tolist() == [-13, -128, 127]
+
+
+def test_pack_unpack_exhaustive():
+    allb = np.arange(256, dtype=np.uint8)
+    codes = co.unpack(allb)
+    assert codes.max() == 15 and np.array_equal(codes[0::2], allb >> 4) and np.array_equal(codes[1::2], allb & 15)
+    assert np.array_equal(co.pack(codes), allb)
+    tcodes = tr.decompress(torch.from_numpy(allb.view(np.int8)))
+    assert np.array_equal(tcodes.numpy().reshape(-1).astype(np.uint8), codes)
+    assert np.array_equal(tr.compress(tcodes).numpy().view(np.uint8), allb)
+
+
+# -------------------------------------------------------------------- dequant --
+def test_dequant_matches_torch_bf16_arithmetic():
+    N, K = 24, 384
+    codes, packed, scales, zeros = make_w4(N, K, 0)
+    zeros.view(-1)[::3] = 7.5
+    zeros.view(-1)[1::7] = 6.28125
+    zeros.view(-1)[2::11] = 300.0
+    want = tr.dequant_4bit_g(packed, scales, zeros, (N, K))  # torch's own bf16 ops
+    got = co.dequant(packed.numpy(), bits(scales), bits(zeros), N, K)
+    assert np.array_equal(got, bits(want))
+
+
+def test_dequant_exact_rational_model():
+    rng = np.random.default_rng(1)
+    for _ in range(300):
+        q = int(rng.integers(0, 16))
+        zb = int(co.f32_to_bf16_bits(np.array([rng.choice([6, 7, 8, 9, 7.5, 0.3, 100.25])], np.float32))[0])
+        sb = int(co.f32_to_bf16_bits(np.array([abs(rng.standard_normal()) * 0.02 / 7 + 1e-6], np.float32))[0])
+        z, s = frac_of_bits(zb), frac_of_bits(sb)
+        want = bf16(f32(bf16(f32(q - z)) * s))
+        packed = co.pack(np.array([q] * 128, np.uint8))
+        got = co.dequant(packed, np.array([sb], np.uint16), np.array([zb], np.uint16), 1, 128)
+        assert Fraction(float(co.bf16_bits_to_f32(got.reshape(-1)[:1])[0])) == want
+
+
+def test_dequant_gptq_identity():
+    """GPTQ stores zero - 1 and dequantises (q - (z_stored + 1)) * s (PTQ/quant/quant_linear.py:339)."""
+    N, K = 8, 256
+    codes, packed, scales, zeros = make_w4(N, K, 2)
+    w = co.bf16_bits_to_f32(co.dequant(packed.numpy(), bits(scales), bits(zeros), N, K)).reshape(N, K)
+    z_stored = zeros.float().reshape(N, K // 128) - 1
+    s = scales.float().reshape(N, K // 128)
+    full = (codes.float().reshape(N, K // 128, 128) - (z_stored[..., None] + 1)) * s[..., None]
+    assert np.array_equal(w, full.to(torch.bfloat16).float().reshape(N, K).numpy())
+
+
+# ------------------------------------------------------------------ A16W4 GEMM --
+def test_fwd_and_dx_against_float64_matmul_and_adjoint():
+    M, N, K = 40, 48, 256
+    codes, packed, scales, zeros = make_w4(N, K, 3)
+    x, dy, b = randn_bf16((M, K), 4), randn_bf16((M, N), 5), randn_bf16((N,), 6)
+    w = from_bits(co.dequant(packed.numpy(), bits(scales), bits(zeros), N, K)).double()
+    y, y64 = co.a16w4_fwd(bits(x), packed.numpy(), bits(scales), bits(zeros), bits(b), M, N, K, want_f64=True)
+    assert np.allclose(y64, (x.double() @ w.t() + b.double()).numpy(), rtol=1e-12, atol=1e-12)
+    assert np.array_equal(y, bits(torch.from_numpy(y64).to(torch.float32).to(torch.bfloat16)))
+    dx, d64 = co.a16w4_dx(bits(dy), packed.numpy(), bits(scales), bits(zeros), M, N, K, want_f64=True)
+    assert np.allclose(d64, (dy.double() @ w).numpy(), rtol=1e-12, atol=1e-12)
+    _, y64nb = co.a16w4_fwd(bits(x), packed.numpy(), bits(scales), bits(zeros), None, M, N, K, want_f64=True)
+    lhs = float((torch.from_numpy(y64nb) * dy.double()).sum())
+    rhs = float((x.double() * torch.from_numpy(d64)).sum())
+    assert abs(lhs - rhs) <= 1e-9 * max(1.0, abs(lhs))
+
+
+def test_fwd_identity_and_reference_cpu_path():
+    N, K = 32, 128
+    codes, packed, scales, zeros = make_w4(N, K, 7)
+    eye = torch.eye(K, dtype=torch.bfloat16)
+    y = co.a16w4_fwd(bits(eye), packed.numpy(), bits(scales), bits(zeros), None, K, N, K)
+    assert np.array_equal(y.T, co.dequant(packed.numpy(), bits(scales), bits(zeros), N, K))
+    x = randn_bf16((64, K), 8)
+    ref = tr.w4_forward(x, packed, scales, zeros, (N, K))  # reference CPU path: bf16 torch.mm
+    _, y64 = co.a16w4_fwd(bits(x), packed.numpy(), bits(scales), bits(zeros), None, 64, N, K, want_f64=True)
+    assert rel_l2(ref.float(), torch.from_numpy(y64)) < 5e-3
+
+
+# --------------------------------------------------------------------- Philox --
+def test_philox_known_answers():
+    kat = [
+        ([0, 0, 0, 0], [0, 0], [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]),
+        ([0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2, [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]),
+        ([0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0],
+         [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]),
+    ]
+    for ctr, key, out in kat:
+        assert list(co.philox4x32_10(ctr, key)) == out
+
+
+def test_philox_uniform_mapping():
+    seed, off = 0x0123456789ABCDEF, 2 ** 32 - 2
+    u = co.philox_uniform(4096, seed, off)
+    assert u.min() >= 0 and u.max() < 1 and np.all(u * 2 ** 24 == np.floor(u * 2 ** 24))
+    for i in (0, 1, 5, 4095):
+        c = off + i // 4
+        w = co.philox4x32_10([c & 0xFFFFFFFF, c >> 32, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
+        assert u[i] == np.float32((int(w[i % 4]) >> 8) * 2.0 ** -24)
+    assert 0.48 < u.mean() < 0.52 and abs(np.corrcoef(u[:-1], u[1:])[0, 1]) < 0.05
+
+
+# -------------------------------------------------------------------- requant --
+def requant_model(q, zb, sb, gb, lr, u):
+    z, s, g = frac_of_bits(zb), frac_of_bits(sb), frac_of_bits(gb)
+    w = bf16(f32(bf16(f32(q - z)) * s))
+    t = f32(w - Fraction(float(np.float32(lr))) * g)
+    v = f32(t / s)
+    v = f32(v + z)
+    v = f32(v + Fraction(float(u)))
+    fl = v.numerator // v.denominator
+    return min(max(fl, 0), 15)
+
+
+@pytest.mark.parametrize("lr,gstd", [(1e-4, 1e-3), (1.0, 2e-3), (3e-2, 1.0)])
+def test_requant_exact_rational_model(lr, gstd):
+    N, K = 2, 128
+    codes, packed, scales, zeros = make_w4(N, K, int(lr * 1e4) + 3)
+    zeros.view(-1)[1] = 7.5
+    grad = randn_bf16((N, K), 11, gstd)
+    u = torch.rand((N, K), generator=torch.Generator().manual_seed(12), dtype=torch.float32)
+    u.view(-1)[::9] = 0.0
+    got = co.unpack(co.requant(packed.numpy(), bits(scales), bits(zeros), bits(grad), lr, N, K, u=u.numpy()))
+    sb, zb, gb = bits(scales).reshape(-1), bits(zeros).reshape(-1), bits(grad).reshape(-1)
+    cf = codes.reshape(-1)
+    for i in range(N * K):
+        want = requant_model(int(cf[i]), int(zb[i // 128]), int(sb[i // 128]), int(gb[i]), lr, float(u.view(-1)[i]))
+        assert got[i] == want, i
+
+
+def test_requant_invariants():
+    N, K = 16, 256
+    codes, packed, scales, zeros = make_w4(N, K, 13)
+    zero_g = torch.zeros((N, K), dtype=torch.bfloat16)
+    half = np.full(N * K, 0.5, np.float32)
+    args = (bits(scales), bits(zeros))
+    assert np.array_equal(co.requant(packed.numpy(), *args, bits(zero_g), 1e-4, N, K, u=half), packed.numpy().view(np.uint8))
+    big = torch.full((N, K), 1e30, dtype=torch.bfloat16)
+    assert np.all(co.requant(packed.numpy(), *args, bits(big), 1.0, N, K, u=half) == 0x00)
+    assert np.all(co.requant(packed.numpy(), *args, bits(-big), 1.0, N, K, u=half) == 0xFF)
+    # u = 0 is a plain floor: with g = 0 the code can only stay or drop by one (bf16 rounding of w)
+    fl = co.unpack(co.requant(packed.numpy(), *args, bits(zero_g), 1e-4, N, K, u=np.zeros(N * K, np.float32)))
+    d = codes.reshape(-1).numpy().astype(int) - fl.astype(int)
+    assert set(np.unique(d)) <= {0, 1}
+    # Philox mode == injected mode on the materialised stream
+    g = randn_bf16((N, K), 14, 1e-2)
+    a = co.requant(packed.numpy(), *args, bits(g), 0.05, N, K, seed=99, offset=5)
+    b = co.requant(packed.numpy(), *args, bits(g), 0.05, N, K, u=co.philox_uniform(N * K, 99, 5))
+    assert np.array_equal(a, b)
+
+
+def test_requant_unbiased():
+    """E_u[code'] = (w - lr g)/s + z for non-saturating updates: mean over many seeds."""
+    N, K = 4, 128
+    codes, packed, scales, zeros = make_w4(N, K, 15)
+    codes = torch.randint(3, 12, (N, K), generator=torch.Generator().manual_seed(1), dtype=torch.uint8)
+    packed = pack_codes(codes)
+    g = randn_bf16((N, K), 16, 1.0)
+    lr = 2e-3
+    w = tr.dequant_4bit_g(packed, scales, zeros, (N, K)).float()
+    s = scales.float().repeat_interleave(128).view(N, K)
+    z = zeros.float().repeat_interleave(128).view(N, K)
+    target = ((w - lr * g.float()) / s + z).numpy().reshape(-1)
+    acc = np.zeros(N * K)
+    reps = 400
+    for r in range(reps):
+        acc += co.unpack(co.requant(packed.numpy(), bits(scales), bits(zeros), bits(g), lr, N, K, seed=r, offset=0))
+    inside = (target > 0.5) & (target < 14.5)
+    assert inside.sum() > 100
+    assert np.abs(acc / reps - target)[inside].max() < 0.12  # 4 sigma of a Bernoulli mean over 400 draws
+
+
+def test_reciprocal_divide_exhaustive_over_scales():
+    qm, cm, n = co.markstein_check(12345, 300)
+    assert n > 5_000_000 and qm == 0 and cm == 0
+
+
+# ----------------------------------------------------------------------- A8W8 --
+def test_a8w8_int32_exact_and_extremes():
+    rng = np.random.default_rng(3)
+    M, N, K = 33, 48, 256
+    x = rng.integers(-128, 128, (M, K), dtype=np.int8)
+    w = rng.integers(-128, 128, (N, K), dtype=np.int8)
+    sx, sw = rng.random(M, dtype=np.float32), rng.random(N, dtype=np.float32)
+    y, acc = co.a8w8(x, w, sx, sw, None, M, N, K)
+    assert np.array_equal(acc, (x.astype(np.int64) @ w.astype(np.int64).T).astype(np.int32))
+    assert np.array_equal(acc, tr.int8_matmul_i32(torch.from_numpy(x), torch.from_numpy(w)).numpy())
+    closed = (acc.astype(np.float32) * sx[:, None]) * sw[None, :]
+    assert np.array_equal(y, co.f32_to_bf16_bits(closed).reshape(M, N))
+    xe = np.full((2, 8192), 127, np.int8)
+    we = np.stack([np.full(8192, 127, np.int8), np.full(8192, -127, np.int8)])
+    _, acc = co.a8w8(xe, we, np.ones(2, np.float32), np.ones(2, np.float32), None, 2, 2, 8192, want_y=False)
+    assert acc.tolist() == [[132128768, -132128768]] * 2
+
+
+def test_act_quant_matches_torch_bf16_arithmetic():
+    x = randn_bf16((257,), 9, 3.0)
+    clampv = x.max()
+    want = tr.act_quant_i8(x, clampv).numpy()
+    got = co.act_quant_i8(bits(x), float(clampv))
+    assert np.array_equal(got, want)
+    want2 = tr.act_quant_i8(x, float(clampv)).numpy()  # python-float clamp (the eval path)
+    assert np.array_equal(got, want2)
+
+
+# ---------------------------------------------------------------------- layout --
+def test_gptq_layout_brute_force():
+    N, K = 16, 128
+    codes, packed, _, _ = make_w4(N, K, 10)
+    gptq = co.native_to_gptq(packed.numpy(), N, K)
+    for n, k in [(0, 0), (3, 7), (15, 127), (9, 64), (1, 9)]:
+        assert (int(gptq[k // 8, n]) >> (4 * (k % 8))) & 15 == int(codes[n, k])
+    assert np.array_equal(co.gptq_to_native(gptq, N, K), packed.numpy().view(np.uint8))
