@@ -121,6 +121,27 @@ int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const float *sw,
 int lq_act_quant_i8(const void *x, const float *clampv_dev, int8_t *x8, int64_t n, void *stream);
 
 /* ---------------------------------------------------------------------------
+ * 4-bit residual codec of the latent weight (exact lbit = 4 mode).
+ *
+ * Replaces the MyQuantDequant extension of the reference: pybind names
+ * `quant` / `dequant` (utils/cuda_src/multi_random_quant.cpp:13-21,
+ * kernels multi_random_quant_kernel.cu:9-67, 130-172) for mode 0 and
+ * `uniform_quant` / `uniform_dequant` (multi_random_quant.cpp:23-31, kernels
+ * :241-266, :297-314) for mode 1; called from cuda_quant_3fold /
+ * cuda_dequant_3fold / cuda_quant_linear / cuda_dequant_linear
+ * (utils/quant.py:723-763). Argument meaning as in the reference:
+ * (k1, b1, k2, b2, k3) are the level counts and breakpoints of the three
+ * companding segments (ignored in mode 1).
+ * x_inout / x_out: bf16[8 * n_words]; q: int32[n_words], element k of a word in
+ * bits 28-4k. lq_residual_quant OVERWRITES x with the carry flags (bf16 1.0
+ * where the level rounded up past 7, else 0.0), as the reference does.
+ * ------------------------------------------------------------------------- */
+int lq_residual_quant(void *x_inout, int32_t *q_out, int64_t n_words, int mode, int k1, float b1, int k2,
+                      float b2, int k3, void *stream);
+int lq_residual_dequant(const int32_t *q, void *x_out, int64_t n_words, int mode, int k1, float b1, int k2,
+                        float b2, int k3, void *stream);
+
+/* ---------------------------------------------------------------------------
  * Layout converters (device side).
  * GPTQ layout (reference PTQ/quant/quant_linear.py:343-389): qweight is
  * int32[K/8, N] with code(k, n) at bits 4*(k%8) of word [k/8, n].

@@ -25,6 +25,8 @@ SIGNATURES = {
     "lq_a16w4_dequant": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp],
     "lq_a8w8_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "lq_act_quant_i8": [_vp, _vp, _vp, _i64, _vp],
+    "lq_residual_quant": [_vp, _vp, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],
+    "lq_residual_dequant": [_vp, _vp, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],
     "lq_repack_gptq_to_native": [_vp, _vp, _i64, _i64, _vp],
     "lq_repack_native_to_gptq": [_vp, _vp, _i64, _i64, _vp],
 }

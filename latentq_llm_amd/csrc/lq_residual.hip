@@ -1,0 +1,158 @@
+// 4-bit residual codec of the latent weight (values in [-0.5, 0.5]) for gfx950.
+//
+// Counterpart of the reference's MyQuantDequant extension
+// (utils/cuda_src/multi_random_quant_kernel.cu:9-67 quant, :130-172 dequant, :241-266 uniform
+// quant, :297-314 uniform dequant; host wrappers :345-400). Semantics kept: one 32-bit word
+// holds 8 consecutive elements MSB first (element k in bits 28-4k); a level above 7 stores
+// nibble 1 and reports a carry of 1.0 in place of the input, otherwise nibble level+8 and 0.0;
+// the dither is the deterministic v = frac-centred(|x|*499) (the reference's random offset
+// `rand()%1000/1000` is an integer division and always 0). The reference is built by nvcc,
+// which contracts a*b+c into an FMA by default; the same fused operations are written out
+// here with fmaf. Layout of the work differs: a thread moves 16 bytes in and out instead of
+// eight 2-byte accesses.
+#include "lq_common.h"
+
+namespace {
+
+struct CodecParams {
+    float c1, c2, c3;  // forward slopes (quant) or inverse slopes (dequant)
+    float b1, b2;
+    int t1, t2;
+};
+
+__device__ __forceinline__ float level_3fold(float x, const CodecParams &p) {
+    const float S = fabsf(x);
+    float v = fmaf(S, 499.0f, 0.0f);
+    v -= roundf(v);
+    if (S < p.b1) return roundf(fmaf(x, p.c1, v));
+    float r;
+    if (S < p.b2) r = roundf(fmaf(S - p.b1, p.c2, v)) + (float)p.t1;
+    else r = roundf(fmaf(S - p.b2, p.c3, v)) + (float)p.t2;
+    return x < 0.0f ? -r : r;
+}
+
+__device__ __forceinline__ float level_uniform(float x) {
+    const float S = fabsf(x);
+    float v = fmaf(S, 499.0f, 0.0f);
+    v = roundf(v) - v;
+    return roundf(fmaf(x, 8.0f, v));
+}
+
+// float level -> (nibble, carry). Negative values below -8 saturate to nibble 0 like the
+// float->unsigned conversion of the reference's target.
+__device__ __forceinline__ unsigned nibble_of(float lv, bool &carry) {
+    carry = lv > 7.5f;
+    if (carry) return 1u;
+    const float t = lv + 8.0f;
+    return t > 0.0f ? ((unsigned)t & 0xFu) : 0u;
+}
+
+template <int MODE>  // 0: three-segment companding, 1: uniform with dither
+__global__ __launch_bounds__(256) void residual_quant_kernel(u32x4_t *__restrict__ x, unsigned *__restrict__ q,
+                                                            long long n_words, CodecParams p) {
+    const long long w = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (w >= n_words) return;
+    const u32x4_t in = x[w];
+    unsigned word = 0;
+    unsigned short carry_bits[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const float xv = (k & 1) ? lq_bf16_hi(in[k >> 1]) : lq_bf16_lo(in[k >> 1]);
+        const float lv = MODE == 0 ? level_3fold(xv, p) : level_uniform(xv);
+        bool carry;
+        const unsigned nib = nibble_of(lv, carry);
+        word = (word << 4) | nib;
+        carry_bits[k] = carry ? 0x3F80u : 0u;  // bf16 1.0 / 0.0
+    }
+    u32x4_t out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = (unsigned)carry_bits[2 * i] | ((unsigned)carry_bits[2 * i + 1] << 16);
+    q[w] = word;
+    x[w] = out;
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256) void residual_dequant_kernel(const unsigned *__restrict__ q, u32x4_t *__restrict__ x,
+                                                              long long n_words, CodecParams p) {
+    const long long w = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (w >= n_words) return;
+    const unsigned word = q[w];
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const int s = (int)((word >> (28 - 4 * k)) & 0xFu) - 8;
+        if (MODE == 1) {
+            v[k] = (float)s * 0.125f;
+        } else if (s < -p.t2) {
+            v[k] = fmaf((float)(s + p.t2), p.c3, -p.b2);
+        } else if (s < -p.t1) {
+            v[k] = fmaf((float)(s + p.t1), p.c2, -p.b1);
+        } else if (s <= p.t1) {
+            v[k] = (float)s * p.c1;
+        } else if (s <= p.t2) {
+            v[k] = fmaf((float)(s - p.t1), p.c2, p.b1);
+        } else {
+            v[k] = fmaf((float)(s - p.t2), p.c3, p.b2);
+        }
+    }
+    u32x4_t out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = lq_pack_bf16(v[2 * i], v[2 * i + 1]);
+    x[w] = out;
+}
+
+int check(const char *who, const void *x, const void *q, int64_t n_words, int mode, int k1, float b1, int k2, float b2,
+          int k3) {
+    LQ_REQUIRE(x && q, "%s: null pointer argument", who);
+    LQ_REQUIRE(n_words > 0 && n_words <= (0x7FFFFFFFll * 256), "%s: bad word count %lld", who, (long long)n_words);
+    LQ_REQUIRE(lq_aligned(x, 16) && lq_aligned(q, 4), "%s: x must be 16-byte and q 4-byte aligned", who);
+    LQ_REQUIRE(mode == 0 || mode == 1, "%s: mode must be 0 (three-segment) or 1 (uniform)", who);
+    if (mode == 0)
+        LQ_REQUIRE(k1 > 0 && k2 > 0 && k3 > 0 && b1 > 0.0f && b2 > b1 && b2 < 0.5f,
+                   "%s: need k1,k2,k3 > 0 and 0 < b1 < b2 < 0.5", who);
+    return LQ_OK;
+}
+
+}  // namespace
+
+extern "C" int lq_residual_quant(void *x_inout, int32_t *q_out, int64_t n_words, int mode, int k1, float b1, int k2,
+                                 float b2, int k3, void *stream) {
+    int rc = check("lq_residual_quant", x_inout, q_out, n_words, mode, k1, b1, k2, b2, k3);
+    if (rc) return rc;
+    CodecParams p = {};
+    if (mode == 0) {
+        p.c1 = (float)k1 / b1;
+        p.c2 = (float)k2 / (b2 - b1);
+        p.c3 = (float)((double)k3 / (0.5 - (double)b2));
+        p.b1 = b1; p.b2 = b2; p.t1 = k1; p.t2 = k1 + k2;
+    }
+    const unsigned blocks = (unsigned)((n_words + 255) / 256);
+    if (mode == 0)
+        hipLaunchKernelGGL(residual_quant_kernel<0>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (u32x4_t *)x_inout,
+                           (unsigned *)q_out, (long long)n_words, p);
+    else
+        hipLaunchKernelGGL(residual_quant_kernel<1>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (u32x4_t *)x_inout,
+                           (unsigned *)q_out, (long long)n_words, p);
+    return lq_check_launch("lq_residual_quant");
+}
+
+extern "C" int lq_residual_dequant(const int32_t *q, void *x_out, int64_t n_words, int mode, int k1, float b1, int k2,
+                                   float b2, int k3, void *stream) {
+    int rc = check("lq_residual_dequant", x_out, q, n_words, mode, k1, b1, k2, b2, k3);
+    if (rc) return rc;
+    CodecParams p = {};
+    if (mode == 0) {
+        p.c1 = b1 / (float)k1;
+        p.c2 = (b2 - b1) / (float)k2;
+        p.c3 = (float)((0.5 - (double)b2) / (double)k3);
+        p.b1 = b1; p.b2 = b2; p.t1 = k1; p.t2 = k1 + k2;
+    }
+    const unsigned blocks = (unsigned)((n_words + 255) / 256);
+    if (mode == 0)
+        hipLaunchKernelGGL(residual_dequant_kernel<0>, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                           (const unsigned *)q, (u32x4_t *)x_out, (long long)n_words, p);
+    else
+        hipLaunchKernelGGL(residual_dequant_kernel<1>, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                           (const unsigned *)q, (u32x4_t *)x_out, (long long)n_words, p);
+    return lq_check_launch("lq_residual_dequant");
+}

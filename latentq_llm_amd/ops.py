@@ -183,3 +183,26 @@ def repack_native_to_gptq(codes, shape):
     with torch.cuda.device(codes.device):
         _C.call("lq_repack_native_to_gptq", codes.data_ptr(), out.data_ptr(), N, K, _stream(codes))
     return out
+
+
+def residual_quant(x, q, mode: int, k1=0, b1=0.0, k2=0, b2=0.0, k3=0):
+    """4-bit residual codec, quantise: writes the packed words into q (int32[n/8]) and overwrites the
+    bf16 tensor x with the carry flags (1.0 / 0.0). mode 0 = three-segment companding, 1 = uniform."""
+    _chk(x, torch.bfloat16, "x")
+    _chk(q, torch.int32, "q")
+    if x.numel() != 8 * q.numel():
+        raise ValueError("x must have 8 elements per word of q")
+    with torch.cuda.device(x.device):
+        _C.call("lq_residual_quant", x.data_ptr(), q.data_ptr(), q.numel(), mode, k1, float(b1), k2, float(b2), k3,
+                _stream(x))
+    return x
+
+
+def residual_dequant(q, mode: int, k1=0, b1=0.0, k2=0, b2=0.0, k3=0):
+    """4-bit residual codec, dequantise: int32[n_words] -> bf16[n_words, 8]."""
+    _chk(q, torch.int32, "q")
+    x = torch.empty((q.numel(), 8), dtype=torch.bfloat16, device=q.device)
+    with torch.cuda.device(q.device):
+        _C.call("lq_residual_dequant", q.data_ptr(), x.data_ptr(), q.numel(), mode, k1, float(b1), k2, float(b2), k3,
+                _stream(q))
+    return x

@@ -1,0 +1,964 @@
+"""Drop-in for the reference's ``utils/quant.py`` with the hot ops on the gfx950 HIP kernels.
+
+Same public names, constructor arguments, buffer names and calling conventions as the reference
+module (``utils/quant.py``; used by ``main0.py:36, 208, 300-343, 454-504`` and ``Demo2.py:25,
+37-104``), so ``from utils.quant import ...`` can be pointed here unchanged. What differs is
+underneath: dequantise+matmul, the int8 GEMM with its scale epilogue, the 4-bit residual codec
+and the stochastic latent requantizer are single HIP kernels reached through the C ABI
+(``latentq_llm_amd.ops``); there is no Triton, no torch_int/cutlass and no JIT-compiled CUDA
+extension. GPU tensors are mandatory for those ops (no CPU fallback).
+
+Deliberate deviations from the reference, all on purpose:
+  * ``QLinearFunctionA8W8_dynamic.backward`` multiplies an int8 tensor in place by a bf16 scale
+    (utils/quant.py:281-283), which stock PyTorch rejects; the semantics of its siblings
+    (utils/quant.py:200-201) are used: ``W8.to(bf16) * qscales``.
+  * the dynamic A8W8 forward keeps ``clampv = input.max()`` on the device instead of ``.item()``
+    (utils/quant.py:220, 320): same value, no host sync.
+  * ``lbit=0`` (the constructor default, which in the reference leaves an uninitialised fp32
+    latent copy) selects the stochastic-rounding latent requantizer: no stored residual, the
+    optimizer calls ``ops.requant_sr`` once per parameter (kernel 1).
+  * ``MyAdam.step`` does not synchronise the device and empty the cache after every parameter
+    (utils/quant.py:985, 1137).
+"""
+from __future__ import annotations
+
+import math
+from functools import reduce
+from typing import Optional, Union
+
+import torch
+import torch.nn as nn
+
+from . import ops
+
+GROUPSIZE = 128  # utils/quant.py:44
+EXT_type = torch.bfloat16  # utils/quant.py:722
+
+# dW travels from the autograd Functions to the full-backward hook through this list
+# (utils/quant.py:109-110, 398-411).
+dict_temp = []
+
+
+# --------------------------------------------------------------------------- nibble packing --
+@torch.no_grad()
+def python_compress(fdata, bit=4):
+    """Two 4-bit codes per int8 byte, even index in the high nibble (utils/quant.py:4-9)."""
+    assert bit == 4
+    pairs = fdata.reshape(-1, 2).to(torch.uint8)
+    return ((pairs[:, 0] << 4) | (pairs[:, 1] & 0xF)).view(torch.int8).contiguous()
+
+
+@torch.no_grad()
+def python_decompress(int_data, bit=4):
+    """int8 bytes -> [n, 2] int8 codes in 0..15 (utils/quant.py:12-19)."""
+    assert bit == 4
+    b = int_data.reshape(-1).view(torch.uint8)
+    return torch.stack(((b >> 4), (b & 0xF)), dim=1).to(torch.int8)
+
+
+# ------------------------------------------------------------------ 8-bit optimizer states --
+@torch.no_grad()
+def Qfunc_8bit_opt(tensor, blocksize=1, qparam=None):
+    """Block-wise asymmetric uint8 quantizer of an optimizer moment (utils/quant.py:22-33):
+    ``blocksize`` is the NUMBER of blocks; q = clamp(round((max - x)/scale), 0, 255)."""
+    shape = tensor.shape
+    blocks = tensor.view(blocksize, -1)
+    if qparam is None:
+        lo, hi = torch.aminmax(blocks, dim=1, keepdim=True)
+        scale = (hi - lo) / 255 + 1e-10
+    else:
+        scale, hi = qparam
+    q = torch.clamp_(torch.round_((hi - blocks).div_(scale)), 0, 255)
+    return q.to(torch.uint8).view(shape), [scale, hi]
+
+
+@torch.no_grad()
+def DeQfunc_8bit_opt(qtensor, qparam, dtype=torch.float32):
+    """Inverse of Qfunc_8bit_opt (utils/quant.py:35-41)."""
+    scale, hi = qparam
+    shape = qtensor.shape
+    x = hi - qtensor.view(scale.shape[0], -1).to(dtype) * scale
+    return x.view(shape).to(dtype)
+
+
+# ----------------------------------------------------------------- W4 group (de)quantizers --
+def _flat_qparam(qparam):
+    scales, zeros, shape = qparam
+    return scales.contiguous().reshape(-1), zeros.contiguous().reshape(-1), list(shape)
+
+
+@torch.no_grad()
+def DeQfunc_4bit_g(qtensor, qparam, dtype=torch.float32):
+    """bf16((codes - zeros) * scales) per 128-element group (utils/quant.py:66-72), one HIP pass."""
+    scales, zeros, shape = _flat_qparam(qparam)
+    w = ops.a16w4_dequant(qtensor.contiguous(), scales.to(torch.bfloat16), zeros.to(torch.bfloat16), shape)
+    return w if dtype == torch.bfloat16 else w.to(dtype)
+
+
+@torch.no_grad()
+def Qfunc_4bit_g_res(tensor, residual_handle, qparam, groupsize=GROUPSIZE):
+    """Round-to-nearest group quantizer with residual memory (utils/quant.py:45-63):
+    Z = t/s + z; q = round(Z); the fractional part goes to the 4-bit residual codec, whose carry
+    is added back; clamp to [0, 15] and pack."""
+    scales, zeros, shape = qparam
+    scales = scales.contiguous().reshape(-1, 1)
+    zeros = zeros.contiguous().reshape(-1, 1)
+    t = tensor.data.view(-1, groupsize)
+    Z = t / scales + zeros
+    q = torch.round(Z)
+    if isinstance(residual_handle, ResidualTensor):
+        carry = residual_handle.set_value((Z - q).view(shape), scales)
+        q = q.view(shape) + carry
+    else:
+        residual_handle.data = t.view(shape).to(residual_handle.dtype)
+    return python_compress(torch.clamp(q, 0, 15).to(torch.uint8))
+
+
+@torch.no_grad()
+def Qfunc_8bit_res(tensor, residual_handle, qscales):
+    """Per-channel int8 re-quantizer with residual memory (utils/quant.py:88-103)."""
+    shape = tensor.shape
+    q = tensor / qscales
+    q.round_()
+    if isinstance(residual_handle, ResidualTensor):
+        carry = residual_handle.set_value((tensor / qscales - q).view(shape), qscales)
+        q += carry
+    elif residual_handle is not None:
+        residual_handle.data = tensor.to(residual_handle.dtype)
+    return q.clamp_(-128, 127).to(torch.int8)
+
+
+# ------------------------------------------------------------------------ autograd: A16W4 --
+# The reference gates the bias gradient on needs_input_grad[2] (utils/quant.py:143, 208, 249, 290,
+# 371), which is the flag of the non-tensor qparam argument and therefore always False: QLinear
+# biases never receive a gradient there. Kept as is so that training runs match the reference.
+_BIAS_FLAG = 2
+
+def _as_bf16_2d(x):
+    return x.contiguous() if x.dtype == torch.bfloat16 else x.to(torch.bfloat16).contiguous()
+
+
+def _w4_linear(input, weight_d, qparamw4, bias):
+    scales, zeros, shape = _flat_qparam(qparamw4)
+    b = None if bias is None else bias.detach().to(torch.bfloat16).contiguous()
+    y = ops.a16w4_forward(_as_bf16_2d(input), weight_d, scales, zeros, shape, b)
+    return y if input.dtype == torch.bfloat16 else y.to(input.dtype)
+
+
+class QLinearFunctionW4(torch.autograd.Function):
+    """Training A16W4 linear (utils/quant.py:112-146): Y = X deq(W)^T + b; backward re-reads the
+    packed codes (never a materialised W): dX on the HIP dequant-GEMM, dW = dY^T X pushed to
+    dict_temp for the backward hook, dB = sum dY."""
+
+    @staticmethod
+    def forward(input, weight_d, qparamw4, bias):
+        return _w4_linear(input, weight_d, qparamw4, bias)
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        input, weight_d, qparamw4, bias = inputs
+        ctx.save_for_backward(input, weight_d.data, bias)
+        ctx.save_qparamw4 = qparamw4
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, weight_d, bias = ctx.saved_tensors
+        scales, zeros, shape = _flat_qparam(ctx.save_qparamw4)
+        grad_input = grad_bias = None
+        dy = _as_bf16_2d(grad_output)
+        if ctx.needs_input_grad[0]:
+            grad_input = ops.a16w4_dx(dy, weight_d, scales, zeros, shape)
+            if grad_input.dtype != input.dtype:
+                grad_input = grad_input.to(input.dtype)
+        dict_temp.append(grad_output.t().mm(input))
+        if bias is not None and ctx.needs_input_grad[_BIAS_FLAG]:
+            grad_bias = grad_output.sum(0)
+        return grad_input, None, None, grad_bias
+
+
+class QLinearFunctionW4_eval(torch.autograd.Function):
+    """Inference A16W4 linear (utils/quant.py:149-169): no state saved, no gradients."""
+
+    @staticmethod
+    def forward(input, weight_d, qparamw4, bias):
+        return _w4_linear(input, weight_d, qparamw4, bias)
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        pass
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return None, None, None, None
+
+
+# ------------------------------------------------------------------------- autograd: A8W8 --
+def _clamp_tensor(clampv, device):
+    if torch.is_tensor(clampv):
+        return clampv.detach().to(device=device, dtype=torch.float32).reshape(1)
+    return torch.tensor([float(clampv)], dtype=torch.float32, device=device)
+
+
+def _a8w8_linear(input, weight_i8, qscales, bias, clampv, alpha_in_bf16):
+    """x8 = clamp(round(x*127/clampv)); Y = ((x8 . W8^T) * alpha) * qscales + bias with
+    alpha = clampv/127: the cutlass call `linear_a8_w8_bbf16_obf16(x8, W8, bias/qs, alpha) * qs`
+    of utils/quant.py:268-271 as one int8-MFMA kernel with a fused epilogue. Returns (Y, x8)."""
+    x = _as_bf16_2d(input)
+    cv = _clamp_tensor(clampv, x.device)
+    x8 = ops.act_quant_i8(x, cv)
+    if alpha_in_bf16:  # the training Function divides a 0-dim bf16 tensor: alpha is bf16-rounded
+        alpha = (cv.to(torch.bfloat16) / 127.).float()
+    else:
+        alpha = cv / 127.
+    sx = alpha.expand(x.shape[0]).contiguous()
+    sw = qscales.detach().reshape(-1).float().contiguous()
+    b = None if bias is None else bias.detach().to(torch.bfloat16).contiguous()
+    y = ops.a8w8_forward(x8, weight_i8.contiguous(), sx, sw, b)
+    return (y if input.dtype == torch.bfloat16 else y.to(input.dtype)), x8
+
+
+def _fake_quant_activation(input, clampv):
+    s = 127. / clampv
+    return (input * s).round_().clamp_(-128, 127).div_(s)
+
+
+def _a8w8_backward_common(ctx, grad_output, input_f, weight_f, bias, detach_dw):
+    grad_input = grad_bias = None
+    if ctx.needs_input_grad[0]:
+        grad_input = grad_output.mm(weight_f)
+    dw = grad_output.t().mm(input_f)
+    dict_temp.append(dw.data if detach_dw else dw)
+    if bias is not None and ctx.needs_input_grad[_BIAS_FLAG]:
+        grad_bias = grad_output.sum(0)
+    return grad_input, None, None, grad_bias
+
+
+class QLinearFunctionA8W8_static(torch.autograd.Function):
+    """Static activation clamp (utils/quant.py:172-211)."""
+
+    @staticmethod
+    def forward(input, weight_d, qparamaw, bias):
+        clampv, qscales = qparamaw
+        return _a8w8_linear(input, weight_d, qscales, bias, clampv, alpha_in_bf16=False)[0]
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        input, weight_d, qparamaw, bias = inputs
+        ctx.save_for_backward(input, weight_d.data, bias)
+        ctx.save_qparamaw = qparamaw
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, weight_d, bias = ctx.saved_tensors
+        clampv, qscales = ctx.save_qparamaw
+        input_f = _fake_quant_activation(input, clampv)
+        weight_f = weight_d.to(input.dtype) * qscales
+        return _a8w8_backward_common(ctx, grad_output, input_f, weight_f, bias, detach_dw=False)
+
+
+class QLinearFunctionA8W8_dynamic0(torch.autograd.Function):
+    """Dynamic clamp = input.max(), saves the bf16 input (utils/quant.py:214-252)."""
+
+    @staticmethod
+    def forward(ctx, input, weight_d, qparamaw, bias):
+        _, qscales = qparamaw
+        clampv = input.max().detach()
+        ctx.save_for_backward(input, weight_d.data, bias)
+        ctx.save_qparamaw = (clampv, qscales)
+        return _a8w8_linear(input, weight_d, qscales, bias, clampv, alpha_in_bf16=False)[0]
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, weight_d, bias = ctx.saved_tensors
+        clampv, qscales = ctx.save_qparamaw
+        input_f = _fake_quant_activation(input, clampv)
+        weight_f = weight_d.to(input.dtype) * qscales
+        return _a8w8_backward_common(ctx, grad_output, input_f, weight_f, bias, detach_dw=True)
+
+
+class QLinearFunctionA8W8_dynamic(torch.autograd.Function):
+    """Dynamic clamp, saves the int8 activations (utils/quant.py:254-293). This is the Function
+    QLinearA8W8 dispatches to when training."""
+
+    @staticmethod
+    def forward(ctx, input, weight_d, qparamaw, bias):
+        _, qscales = qparamaw
+        clampv = input.max().detach()
+        out, x8 = _a8w8_linear(input, weight_d, qscales, bias, clampv, alpha_in_bf16=True)
+        ctx.save_qparamaw = (clampv, qscales)
+        ctx.save_for_backward(x8, weight_d.data, bias)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x8, weight_d, bias = ctx.saved_tensors
+        clampv, qscales = ctx.save_qparamaw
+        input_f = x8.to(grad_output.dtype) * (clampv / 127.)
+        weight_f = (weight_d.to(grad_output.dtype) * qscales).to(grad_output.dtype)
+        return _a8w8_backward_common(ctx, grad_output, input_f, weight_f, bias, detach_dw=True)
+
+
+class QLinearFunctionA8W8_static_eval(torch.autograd.Function):
+    """utils/quant.py:296-312."""
+
+    @staticmethod
+    def forward(ctx, input, weight_d, qparamaw, bias):
+        clampv, qscales = qparamaw
+        return _a8w8_linear(input, weight_d, qscales, bias, clampv, alpha_in_bf16=False)[0]
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return None, None, None, None
+
+
+class QLinearFunctionA8W8_dynamic_eval(torch.autograd.Function):
+    """utils/quant.py:314-331 (clamp = input.max(), kept on the device)."""
+
+    @staticmethod
+    def forward(ctx, input, weight_d, qparamaw, bias):
+        _, qscales = qparamaw
+        return _a8w8_linear(input, weight_d, qscales, bias, input.max().detach(), alpha_in_bf16=False)[0]
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return None, None, None, None
+
+
+def _qat_weight_i8(weight_f, qscales):
+    return (weight_f / qscales).round_().clamp_(-128, 127).to(torch.int8)
+
+
+class QLinearFunctionQAT_dynamic(torch.autograd.Function):
+    """bf16 latent weight, quantised to int8 on the fly (utils/quant.py:334-374)."""
+
+    @staticmethod
+    def forward(ctx, input, weight_f, qparamaw, bias):
+        _, qscales = qparamaw
+        clampv = input.max().detach()
+        ctx.save_for_backward(input, weight_f.data, bias)
+        ctx.save_qparamaw = (clampv, qscales)
+        return _a8w8_linear(input, _qat_weight_i8(weight_f, qscales), qscales, bias, clampv, alpha_in_bf16=False)[0]
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, weight_f, bias = ctx.saved_tensors
+        clampv, qscales = ctx.save_qparamaw
+        input_f = _fake_quant_activation(input, clampv)
+        weight_q = (weight_f / qscales).round_().clamp_(-128, 127).mul_(qscales).to(input.dtype)
+        return _a8w8_backward_common(ctx, grad_output, input_f, weight_q, bias, detach_dw=False)
+
+
+class QLinearFunctionQAT_dynamic_eval(torch.autograd.Function):
+    """utils/quant.py:376-394."""
+
+    @staticmethod
+    def forward(ctx, input, weight_f, qparamaw, bias):
+        _, qscales = qparamaw
+        return _a8w8_linear(input, _qat_weight_i8(weight_f, qscales), qscales, bias, input.max().detach(),
+                            alpha_in_bf16=False)[0]
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return None, None, None, None
+
+
+# -------------------------------------------------------------------------- backward hook --
+def backward_hook_fn(module, grad_out, grad_in):
+    """Full-backward hook: move the pending dW into module.weight.grad (utils/quant.py:398-411)."""
+    assert len(dict_temp) == 1
+    dw = dict_temp.pop()
+    g = module.weight.grad
+    if isinstance(g, GradientQTensor):
+        if g.acc_ite == 0:
+            g.set_value(dw)
+        else:
+            g.add_(dw)
+    elif g is None:
+        module.weight.grad = dw
+    else:
+        g.add_(dw)
+
+
+# -------------------------------------------------------------------------------- modules --
+class _QLinearBase(nn.Module):
+    _repr_name = "QLinear"
+
+    def __init__(self, input_features, output_features, bias):
+        super().__init__()
+        self.input_features = input_features
+        self.output_features = output_features
+        if bias:
+            self.bias = nn.Parameter(torch.empty(output_features))
+        else:
+            self.register_parameter('bias', None)
+        self.register_buffer('qweight', torch.tensor([]))  # filled by before_save()
+        self.wshape = [output_features, input_features]
+        self.hook_handle = None
+
+    def add_hook(self):
+        self.hook_handle = self.register_full_backward_hook(backward_hook_fn)
+
+    def _apply_fn(self, fn, x):
+        out = fn.apply(x.reshape(-1, x.shape[-1]), self.weight.data, self._qparam(), self.bias)
+        return out.reshape(x.shape[:-1] + (self.output_features,))
+
+    def forward(self, x):
+        return self._apply_fn(self._fn_eval if self.hook_handle is None else self._fn_train, x)
+
+    def forward_eval(self, x):
+        return self._apply_fn(self._fn_eval, x)
+
+    def before_save(self):
+        self.qweight.data = self.weight.data.cpu()
+
+    def extra_repr(self):
+        return '{} input_features={}, output_features={}, bias={}'.format(
+            self._repr_name, self.input_features, self.output_features, self.bias is not None)
+
+
+class QLinearA16W4(_QLinearBase):
+    """A16W4 linear (utils/quant.py:413-482). Buffers: qweight, zeros, scales (bf16 [(N*K/128),1]);
+    ``weight`` is a QuantTensor holding the packed codes."""
+    _repr_name = "QLinearA16W4"
+    _fn_train, _fn_eval = QLinearFunctionW4, QLinearFunctionW4_eval
+
+    def __init__(self, input_features, output_features, bias=True, lbit=0, gbit=16):
+        super().__init__(input_features, output_features, bias)
+        self.groupsize = GROUPSIZE
+        ngroups = math.ceil(input_features / GROUPSIZE) * output_features
+        self.register_buffer('zeros', torch.zeros((ngroups, 1), dtype=torch.bfloat16))
+        self.register_buffer('scales', torch.zeros((ngroups, 1), dtype=torch.bfloat16))
+        self.weight = QuantTensor([output_features, input_features], lbit=lbit, wbit=4, gbit=gbit)
+
+    def _qparam(self):
+        return self.weight.qparam
+
+    def to(self, device: Optional[Union[int, torch.device]]):
+        """Moves the QuantTensor and re-binds its qparam to the moved buffers; returns None like
+        the reference (utils/quant.py:462-469)."""
+        self.weight = self.weight.to(device=device)
+        self.zeros = self.zeros.to(device=device)
+        self.scales = self.scales.to(device=device)
+        self.weight.set_value(None, [self.scales, self.zeros, self.wshape])
+        if self.bias is not None:
+            self.bias.data = self.bias.data.to(device)
+
+
+class QLinearA8W8(_QLinearBase):
+    """A8W8 linear (utils/quant.py:485-541). Buffers: qweight, clampv[1], qscales bf16 [N,1]."""
+    _repr_name = "QLinearA8W8"
+    _fn_train, _fn_eval = QLinearFunctionA8W8_dynamic, QLinearFunctionA8W8_dynamic_eval
+
+    def __init__(self, input_features, output_features, bias=True, lbit=0, gbit=8):
+        super().__init__(input_features, output_features, bias)
+        self.register_buffer('clampv', torch.ones(1))
+        self.register_buffer('qscales', torch.zeros(output_features, 1, dtype=torch.bfloat16))
+        self.weight = QuantTensor([output_features, input_features], lbit=lbit, wbit=8, gbit=gbit)
+
+    def _qparam(self):
+        # the dynamic Functions ignore the stored clamp (utils/quant.py:259-260): no .item() sync here
+        return (self.clampv, self.qscales.data)
+
+    def to(self, device: Optional[Union[int, torch.device]]):
+        self.weight = self.weight.to(device=device)
+        self.qscales = self.qscales.to(device=device)
+        self.weight.set_value(None, self.qscales)
+        if self.bias is not None:
+            self.bias.data = self.bias.data.to(device)
+
+
+class QLinearQAT(_QLinearBase):
+    """bf16 latent weight + int8 fake-quant forward (utils/quant.py:544-599)."""
+    _repr_name = "QLinearQAT"
+    _fn_train, _fn_eval = QLinearFunctionQAT_dynamic, QLinearFunctionQAT_dynamic_eval
+
+    def __init__(self, input_features, output_features, bias=True, lbit=0, gbit=16):
+        super().__init__(input_features, output_features, bias)
+        self.register_buffer('clampv', torch.ones(1))
+        self.register_buffer('qscales', torch.zeros(output_features, 1, dtype=torch.bfloat16))
+        assert gbit == 16
+        self.weight = FPTensor(torch.empty((output_features, input_features), dtype=torch.bfloat16))
+
+    def _qparam(self):
+        return (self.clampv, self.qscales.data)
+
+    def before_save(self):
+        self.qweight.data = _qat_weight_i8(self.weight.data, self.qscales).cpu()
+
+    def to(self, device: Optional[Union[int, torch.device]]):
+        self.weight = self.weight.to(device=device)
+        if self.bias is not None:
+            self.bias.data = self.bias.data.to(device)
+
+
+# ---------------------------------------------------------------------- latent containers --
+def prodx(ls):
+    return reduce(lambda x, y: x * y, ls)
+
+
+class _LatentBase(object):
+    """Shared behaviour of the non-tensor "parameters" handed to the optimizer."""
+
+    def numel(self):
+        return prodx(self.shape)
+
+    def get_self(self):
+        return self
+
+    def __repr__(self):
+        return "Quant value:\n{}\n with param:\n{}".format(getattr(self, 'data', None), self.qparam)
+
+    def requires_grad_(self, boolv):
+        self.requires_grad = boolv
+        return self
+
+    @property
+    def device(self):
+        return self.data.device
+
+    @property
+    def type(self):
+        return self.data.type
+
+
+class QuantTensor(_LatentBase):
+    """Packed weight + latent information (utils/quant.py:606-663). ``lbit`` selects how the
+    sub-LSB part of the latent weight is kept: 4 -> ResidualTensor (4-bit codec), 16/32 -> a
+    bf16/fp32 copy, 0 -> nothing stored (stochastic-rounding requantizer)."""
+
+    def __init__(self, shape, wbit=8, gbit=8, lbit=4):
+        self.shape = shape
+        self.wbit = wbit
+        self.initial = False
+        self.qparam = None
+        self.lbit = lbit
+        if lbit == 4:
+            channels = shape[0] if wbit == 8 else prodx(shape) // GROUPSIZE
+            self.residual = ResidualTensor(qshape=[channels, prodx(shape) // channels], oshape=shape)
+        elif lbit == 16:
+            self.residual = torch.empty(shape, dtype=torch.bfloat16)
+        elif lbit == 0:
+            self.residual = None
+        else:
+            self.residual = torch.empty(shape, dtype=torch.float32)
+        self.requires_grad = True
+        self.grad = None if gbit == 16 else GradientQTensor(self.shape, bit=gbit)
+
+    def set_value(self, data, qparam=None):
+        if data is not None:
+            self.data = data.clone()
+        self.qparam = qparam
+        self.initial = True
+        self.requires_grad = True
+
+    def to(self, device=None, dtype=None):
+        if device is not None:
+            self.data = self.data.to(device)
+            if isinstance(self.residual, ResidualTensor):
+                self.residual.residual_int = self.residual.residual_int.to(device)
+            elif self.residual is not None:
+                self.residual = self.residual.to(device)
+        return self
+
+
+class FPTensor(_LatentBase):
+    """Plain bf16 latent weight of the QAT layer (utils/quant.py:666-705)."""
+
+    def __init__(self, data, gbit=16):
+        self.data = data
+        self.shape = data.shape
+        self.initial = False
+        self.qparam = None
+        self.requires_grad = True
+        self.grad = None if gbit == 16 else GradientQTensor(self.shape, bit=gbit)
+
+    def to(self, device=None, dtype=None):
+        if device is not None:
+            self.data = self.data.to(device)
+        return self
+
+
+# ------------------------------------------------------------------- 4-bit residual codec --
+def three_fold_curve_4bit(mu):
+    """(levels, breakpoint) pairs of the companding curve per mu level (utils/quant.py:708-716)."""
+    table = {3: (2, 0.4330623539159437, 4, 0.46875), 2: (2, 0.37272211741724515, 4, 0.4375),
+             1: (2, 0.2666300266320331, 4, 0.375)}
+    return table.get(mu, (2, 0.125, 4, 0.25))
+
+
+class _ResidualCodec(object):
+    """Stands in for the reference's JIT-built ``cuda_module`` (utils/quant.py:718-719,
+    multi_random_quant.cpp:38-54) with the same five entry points, backed by the HIP codec."""
+
+    @staticmethod
+    def quant(fp, q, k1, b1, k2, b2, k3):
+        ops.residual_quant(fp, q.view(-1), 0, int(k1), b1, int(k2), b2, int(k3))
+
+    @staticmethod
+    def dequant(q, fp, k1, b1, k2, b2, k3):
+        fp.copy_(ops.residual_dequant(q.view(-1), 0, int(k1), b1, int(k2), b2, int(k3)).view(fp.shape))
+
+    @staticmethod
+    def uniform_quant(fp, q):
+        ops.residual_quant(fp, q.view(-1), 1)
+
+    @staticmethod
+    def uniform_quant_s(fp, q):
+        raise NotImplementedError("uniform_quant_s is not dispatched for bf16 in the reference either "
+                                  "(multi_random_quant_kernel.cu:376-381) and nothing calls it")
+
+    @staticmethod
+    def uniform_dequant(q, fp):
+        fp.copy_(ops.residual_dequant(q.view(-1), 1).view(fp.shape))
+
+
+cuda_module = _ResidualCodec()
+
+
+@torch.no_grad()
+def cuda_quant_linear(residual_fp, q_tensor):
+    """utils/quant.py:723-733."""
+    residual_fp = residual_fp.to(EXT_type)
+    assert residual_fp.is_contiguous()
+    if not residual_fp.is_cuda:
+        return python_quant_linear(residual_fp)
+    cuda_module.uniform_quant(residual_fp, q_tensor)
+    return residual_fp
+
+
+@torch.no_grad()
+def cuda_quant_3fold(residual_fp, q_tensor, p1, y1, p2, y2):
+    """utils/quant.py:735-742: returns the carry tensor (the overwritten bf16 copy of the input)."""
+    residual_fp = residual_fp.to(EXT_type)
+    if not residual_fp.is_contiguous() or residual_fp.data_ptr() % 16:
+        residual_fp = residual_fp.contiguous().clone()
+    assert residual_fp.is_cuda
+    cuda_module.quant(residual_fp, q_tensor, p1, y1, p2 - p1, y2, 8 - p2)
+    return residual_fp
+
+
+@torch.no_grad()
+def cuda_dequant_linear(residual_int):
+    """utils/quant.py:746-755."""
+    assert residual_int.is_contiguous()
+    if not residual_int.is_cuda:
+        return python_dequant_linear(residual_int)
+    return ops.residual_dequant(residual_int.view(-1), 1)
+
+
+@torch.no_grad()
+def cuda_dequant_3fold(residual_int, p1, y1, p2, y2):
+    """utils/quant.py:757-763."""
+    assert residual_int.is_cuda and residual_int.is_contiguous()
+    return ops.residual_dequant(residual_int.view(-1), 0, int(p1), y1, int(p2 - p1), y2, int(8 - p2))
+
+
+@torch.no_grad()
+def python_quant_linear(residual_fp):
+    """CPU stochastic uniform 4-bit quantizer (utils/quant.py:765-778): round((x+.5)*16 + U(-.5,.5)),
+    level 16 wraps to 0 with a carry; eight nibbles per int32, MSB first."""
+    lv = (residual_fp + 0.5) * 16
+    lv.add_(torch.empty_like(lv).uniform_(-0.5, 0.5)).round_()
+    over = lv > 15.9
+    lv[over] = 0.
+    carry = torch.zeros_like(residual_fp)
+    carry[over] = 1.
+    nib = lv.view(-1, 8).to(torch.int32)
+    shifts = torch.arange(28, -4, -4, dtype=torch.int32, device=nib.device)
+    return (nib << shifts).sum(dim=1, dtype=torch.int32).contiguous(), carry
+
+
+@torch.no_grad()
+def python_dequant_linear(residual_int):
+    """utils/quant.py:781-788."""
+    shifts = torch.arange(28, -4, -4, dtype=torch.int32, device=residual_int.device)
+    nib = (residual_int.view(-1, 1) >> shifts) % 16
+    return nib.to(torch.float32) / 16 - 0.5
+
+
+class ResidualTensor(object):
+    """Z - round(Z) in [-0.5, 0.5] at 4 bits per element (utils/quant.py:790-841)."""
+
+    def __init__(self, qshape, oshape):
+        self.weight_scale = None
+        self.qshape = qshape
+        self.oshape = oshape
+        self.lock_mu = self.mu = 0
+        numel_h = prodx(oshape)
+        assert numel_h % 8 == 0
+        dev = 'cuda' if torch.cuda.is_available() else 'cpu'
+        self.residual_int = torch.empty((numel_h // 8, 1), dtype=torch.int32, device=dev)
+        self.name = 'residual'
+        self.init = True
+
+    def set_value(self, residual_fp, weight_scale=None):
+        p1, y1, p2, y2 = three_fold_curve_4bit(self.mu)
+        adj = cuda_quant_3fold(residual_fp, self.residual_int, p1, y1, p2, y2)
+        if weight_scale is not None:
+            self.weight_scale = weight_scale
+        self.lock_mu = self.mu
+        self.init = False
+        return adj
+
+    def update_mu(self, optmizer_std):
+        """Pick the companding curve from the ratio scale / typical update (utils/quant.py:813-824);
+        as in the reference the `> 75.8` test is overwritten by the chain below it."""
+        mu = (self.weight_scale / (optmizer_std + 1e-8)).mean().item()
+        self.mu = 2 if mu > 36.5 else (1 if mu > 16.2 else 0)
+        if self.mu != self.lock_mu:
+            print(f'{self.name} now mu level is {mu}({self.mu}), pre is {self.lock_mu}')
+
+    def dequant(self):
+        p1, y1, p2, y2 = three_fold_curve_4bit(self.lock_mu)
+        return cuda_dequant_3fold(self.residual_int, p1, y1, p2, y2)
+
+    def add(self, tensor: torch.Tensor):
+        if self.init:
+            return tensor
+        r = (self.dequant().view(self.qshape) * self.weight_scale).to(dtype=tensor.dtype)
+        return r.view(self.oshape).add(tensor)
+
+    def __repr__(self):
+        return "ResidualTensor !"
+
+
+class GradientQTensor(object):
+    """8-bit gradient accumulator with stochastic rounding (utils/quant.py:846-922)."""
+
+    def __init__(self, shape, bit=8):
+        self.acc_ite = 0
+        self.bit = bit
+        self.qdata = 0
+        self.scale = None
+        self.qzero = None
+        self.shape = shape
+        self.fixscale = False
+
+    def find_param(self, data):
+        self.vmax = data.abs().amax(dim=1, keepdim=True) * 4
+        self.scale = (torch.clamp(self.vmax, min=1e-5) / (2 ** (self.bit - 1) - 1)).to(data.dtype)
+
+    def quant(self, fdata):
+        noise = torch.empty_like(fdata).uniform_(-0.5, 0.5)
+        q = torch.round(fdata / self.scale + noise)
+        self.qdata = torch.clamp(q, -2 ** (self.bit - 1), 2 ** (self.bit - 1) - 1).to(torch.int8)
+
+    def dequant(self):
+        return self.qdata.to(self.fdtype) * self.scale
+
+    def set_value(self, fdata):
+        if self.bit > 8:
+            self.qdata = fdata
+            return
+        if not (self.fixscale and self.scale is None):
+            self.find_param(fdata)
+        self.quant(fdata)
+        self.fdtype = fdata.dtype
+        self.acc_ite = 1
+
+    def zero(self):
+        self.acc_ite = 0
+        self.qdata = None
+
+    def add_(self, fdata):
+        if self.bit > 8:
+            self.qdata += fdata
+        else:
+            self.acc_ite += 1
+            self.quant(self.dequant() + fdata)
+
+    def get_value(self):
+        return self.qdata if self.bit > 8 else self.dequant()
+
+    def __repr__(self):
+        return f"GradientQTensor bitwidth {self.bit} !"
+
+    def to(self, device):
+        self.qdata = self.qdata.to(device)
+        if self.bit <= 8:
+            self.scale = self.scale.to(device)
+            if self.qzero is not None:
+                self.qzero = self.qzero.to(device)
+        return self
+
+    @property
+    def device(self):
+        return self.qdata.device
+
+
+# ------------------------------------------------------------------------------ optimizer --
+class MyAdam(torch.optim.Adam):
+    """Adam over a mix of nn.Parameters and QuantTensor/FPTensor latents with optional block-wise
+    8-bit moments (utils/quant.py:927-1148). For a QuantTensor the latent weight is rebuilt
+    (dequantised codes + stored residual), stepped, and re-quantised; with ``lbit=0`` the whole
+    rebuild/step/re-quantise tail is one call of the stochastic-rounding requantizer.
+
+    ``sr_seed`` seeds the Philox stream of that requantizer; every call consumes N*K/4 counters."""
+
+    def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), obit=8, mu_updata_f=20, cpu=False, sr_seed=0):
+        super().__init__(params, lr=lr, betas=betas)
+        self.initialized = False
+        self.obit = obit
+        self.mu_updata_f = mu_updata_f
+        self.statedevice = 'cpu' if cpu else 'cuda'
+        self.sr_seed = sr_seed
+        self.sr_offset = 0
+
+    def add_param_group(self, param_group):
+        """Accepts QuantTensor / FPTensor objects next to tensors (utils/quant.py:934-959)."""
+        assert isinstance(param_group, dict), "param group must be a dict"
+        params = param_group['params']
+        if isinstance(params, torch.Tensor):
+            param_group['params'] = [params]
+        elif isinstance(params, set):
+            raise TypeError('optimizer parameters need to be organized in ordered collections, but '
+                            'the ordering of tensors in sets will change between runs. Please use a list instead.')
+        else:
+            param_group['params'] = list(params)
+        for name, default in self.defaults.items():
+            param_group.setdefault(name, default)
+        seen = set()
+        for group in self.param_groups:
+            seen.update(group['params'])
+        if not seen.isdisjoint(param_group['params']):
+            raise ValueError("some parameters appear in more than one parameter group")
+        self.param_groups.append(param_group)
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        for gindex, group in enumerate(self.param_groups):
+            for pindex, p in enumerate(group["params"]):
+                if p.grad is None:
+                    continue
+                if len(self.state[p]) == 0:
+                    self.init_state(group, p, gindex, pindex)
+                self.update_step(group, p, gindex, pindex)
+        return loss
+
+    def to_gpu(self):
+        for group in self.param_groups:
+            for p in group["params"]:
+                if p in self.state:
+                    for k, v in self.state[p].items():
+                        if isinstance(v, torch.Tensor) and not getattr(v, 'is_paged', False):
+                            self.state[p][k] = v.to(p.device)
+
+    def get_config(self, gindex, pindex, group):
+        return {"betas": group["betas"], "eps": group["eps"], "weight_decay": group["weight_decay"],
+                "lr": group["lr"], "block_wise": True}
+
+    def get_state_buffer(self, pshape, pdevice, dtype=torch.float32):
+        return torch.zeros(pshape, dtype=dtype, device=pdevice)
+
+    @torch.no_grad()
+    def init_state(self, group, p, gindex, pindex):
+        """bf16 moments for small tensors or obit=16, else uint8 moments with one (scale, max) pair
+        per block of 2048 (or 128) elements (utils/quant.py:1014-1059)."""
+        config = self.get_config(gindex, pindex, group)
+        dtype = torch.uint8 if self.obit == 8 else torch.bfloat16
+        if p.numel() < 65536:
+            dtype = torch.bfloat16
+        state = self.state[p]
+        state["step"] = 0
+        sdev = self.statedevice if (self.statedevice == 'cpu' or torch.cuda.is_available()) else 'cpu'
+        state["state1"] = self.get_state_buffer(p.shape, sdev, dtype=dtype)
+        state["state2"] = self.get_state_buffer(p.shape, sdev, dtype=dtype)
+        if dtype == torch.uint8:
+            n = p.numel()
+            if not config["block_wise"]:
+                blocks = 1
+            elif n % 2048 == 0:
+                blocks = n // 2048
+            else:
+                assert n % 128 == 0
+                blocks = n // 128
+            for name, fill in (("absmax1", 0.0), ("qmap1", 1e-10), ("absmax2", 0.0), ("qmap2", 1e-10)):
+                state[name] = torch.full((blocks, 1), fill, dtype=torch.float32, device=p.device)
+
+    def _latent(self, p, dtype):
+        """Latent weight of a QuantTensor: dequantised codes + residual (utils/quant.py:1066-1079)."""
+        if isinstance(p.residual, ResidualTensor):
+            if p.wbit == 8:
+                return p.residual.add((p.data * p.qparam).to(dtype))
+            if p.wbit == 4:
+                return p.residual.add(DeQfunc_4bit_g(p.data, p.qparam, dtype))
+            raise AssertionError("wbit must be 4 or 8")
+        return p.residual.data.to(dtype)
+
+    @torch.no_grad()
+    def update_step(self, group, p, gindex, pindex):
+        state = self.state[p]
+        config = self.get_config(gindex, pindex, group)
+        grad = p.grad
+        is_q = isinstance(p, QuantTensor)
+        sr_mode = is_q and p.wbit == 4 and p.residual is None
+        if is_q:
+            if isinstance(grad, GradientQTensor):
+                grad = grad.get_value()
+            pdata = None if sr_mode else self._latent(p, grad.dtype)
+        else:
+            pdata = p.data
+
+        q8 = state["state1"].dtype == torch.uint8
+        if q8:
+            exp_avg = DeQfunc_8bit_opt(state["state1"].to(grad.device), [state["qmap1"], state["absmax1"]]).to(grad.dtype)
+            s2 = DeQfunc_8bit_opt(state["state2"].to(grad.device), [state["qmap2"], state["absmax2"]])
+            exp_avg_sq = (s2 * s2).to(grad.dtype)
+        else:
+            exp_avg = state["state1"].to(grad.device)
+            exp_avg_sq = (state["state2"] * state["state2"]).to(grad.device)
+
+        beta1, beta2 = config["betas"]
+        state["step"] += 1
+        if config["weight_decay"] != 0:
+            wd_base = DeQfunc_4bit_g(p.data, p.qparam, grad.dtype) if sr_mode else pdata
+            grad = grad.add(wd_base, alpha=config["weight_decay"])
+
+        exp_avg.mul_(beta1).add_(grad, alpha=1 - beta1)
+        exp_avg_sq.mul_(beta2).addcmul_(grad, grad, value=1 - beta2)
+        exp_avg_sqrt = exp_avg_sq.sqrt_()
+        denom = exp_avg_sqrt.add_(group["eps"])
+        bias_correction1 = 1 - beta1 ** state["step"]
+        bias_correction2 = 1 - beta2 ** state["step"]
+        step_size = config["lr"] * math.sqrt(bias_correction2) / bias_correction1
+
+        if sr_mode:
+            direction = (exp_avg / denom).to(torch.bfloat16).contiguous()
+        else:
+            pdata.addcdiv_(exp_avg, denom, value=-step_size)
+
+        if (state["step"] > 250 and state["step"] % self.mu_updata_f == (self.mu_updata_f - 1)
+                and isinstance(getattr(p, 'residual', None), ResidualTensor)):
+            std = torch.mean((abs(exp_avg) / denom).view(p.residual.qshape), dim=1, keepdim=True) * step_size
+            p.residual.update_mu(std)
+
+        if q8:
+            nblk = len(state["absmax1"])
+            s1, qp = Qfunc_8bit_opt(exp_avg.float(), blocksize=nblk)
+            state["state1"] = s1.to(state["state1"].device)
+            state["qmap1"], state["absmax1"] = qp
+            s2q, qp = Qfunc_8bit_opt(exp_avg_sqrt.float(), blocksize=nblk)
+            state["state2"] = s2q.to(state["state2"].device)
+            state["qmap2"], state["absmax2"] = qp
+        else:
+            state["state1"] = exp_avg
+            state["state2"] = exp_avg_sq  # holds sqrt(v) + eps after the in-place ops above, as in the reference
+
+        if is_q:
+            if sr_mode:
+                scales, zeros, shape = _flat_qparam(p.qparam)
+                p.data = ops.requant_sr(p.data, scales, zeros, direction.view(shape), step_size, shape,
+                                        seed=self.sr_seed, offset=self.sr_offset)
+                self.sr_offset += (p.numel() + 3) // 4
+            elif p.wbit == 8:
+                p.data = Qfunc_8bit_res(pdata, p.residual, qscales=p.qparam)
+            elif p.wbit == 4:
+                p.data = Qfunc_4bit_g_res(pdata, p.residual, qparam=p.qparam)
+        if isinstance(p.grad, GradientQTensor):
+            p.grad.zero()
+        else:
+            p.grad = None

@@ -167,3 +167,20 @@ def markstein_check(seed: int, per_scale: int):
     qm, cm, n = C.c_int64(0), C.c_int64(0), C.c_int64(0)
     lib().lqo_markstein_check(C.c_uint32(seed), C.c_int(per_scale), C.byref(qm), C.byref(cm), C.byref(n))
     return qm.value, cm.value, n.value
+
+
+def residual_quant(x_bits, mode, k1=0, b1=0.0, k2=0, b2=0.0, k3=0):
+    """-> (words uint32[n/8], carries as bf16 bits); the input array is not modified."""
+    x = _c(x_bits.reshape(-1), np.uint16).copy()
+    q = np.empty(x.size // 8, np.uint32)
+    lib().lqo_residual_quant(_p(x), _p(q), C.c_int64(q.size), C.c_int(mode), C.c_int(k1), C.c_float(b1), C.c_int(k2),
+                             C.c_float(b2), C.c_int(k3))
+    return q, x
+
+
+def residual_dequant(q, mode, k1=0, b1=0.0, k2=0, b2=0.0, k3=0):
+    q = _c(q.reshape(-1).view(np.uint32), np.uint32)
+    x = np.empty(q.size * 8, np.uint16)
+    lib().lqo_residual_dequant(_p(q), _p(x), C.c_int64(q.size), C.c_int(mode), C.c_int(k1), C.c_float(b1), C.c_int(k2),
+                               C.c_float(b2), C.c_int(k3))
+    return x

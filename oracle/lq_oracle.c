@@ -330,3 +330,74 @@ void lqo_markstein_check(uint32_t seed, int per_scale, int64_t *quot_mismatch, i
     *code_mismatch = cm;
     *cases = n;
 }
+
+/* ------------------------------------------------------ residual codec -- */
+/* Restatement of utils/cuda_src/multi_random_quant_kernel.cu for bf16 tensors:
+ * quant_kernel_bf :9-67 and launch_quant :345-362 (mode 0), quant_kernel1_bf :241-266 (mode 1),
+ * dequant_kernel_bf :130-172 and launch_dequant :384-400 (mode 0), dequant_kernel1_bf :297-314
+ * (mode 1). `round` is C's half-away-from-zero; the host-side random offset v0 is
+ * `rand()%1000/1000`, an integer division, i.e. always 0. The reference is compiled by nvcc,
+ * whose default (-fmad=true) contracts a*b+c into one FMA: fmaf is used where the source has
+ * that shape. A float level below -8 converts to unsigned 0 (saturating conversion). */
+static inline float residual_level(float x, int mode, float c1, float c2, float c3, float b1, float b2, int t1,
+                                   int t2) {
+    float S = fabsf(x);
+    float v = fmaf(S, 499.0f, 0.0f);
+    if (mode == 1) {
+        v = roundf(v) - v;
+        return roundf(fmaf(x, 8.0f, v));
+    }
+    v -= roundf(v);
+    if (S < b1) return roundf(fmaf(x, c1, v));
+    float r = (S < b2) ? roundf(fmaf(S - b1, c2, v)) + (float)t1 : roundf(fmaf(S - b2, c3, v)) + (float)t2;
+    return x < 0.0f ? -r : r;
+}
+
+void lqo_residual_quant(uint16_t *x, uint32_t *q, int64_t n_words, int mode, int k1, float b1, int k2, float b2,
+                        int k3) {
+    float c1 = 0, c2 = 0, c3 = 0;
+    if (mode == 0) {
+        c1 = (float)k1 / b1;
+        c2 = (float)k2 / (b2 - b1);
+        c3 = (float)((double)k3 / (0.5 - (double)b2));
+    }
+    for (int64_t w = 0; w < n_words; ++w) {
+        uint32_t word = 0;
+        for (int k = 0; k < 8; ++k) {
+            float lv = residual_level(bf16_to_f32(x[8 * w + k]), mode, c1, c2, c3, b1, b2, k1, k1 + k2);
+            word <<= 4;
+            if (lv > 7.5f) {
+                word += 1u;
+                x[8 * w + k] = 0x3F80u;
+            } else {
+                float t = lv + 8.0f;
+                word |= (t > 0.0f) ? ((uint32_t)t & 0xFu) : 0u;
+                x[8 * w + k] = 0u;
+            }
+        }
+        q[w] = word;
+    }
+}
+
+void lqo_residual_dequant(const uint32_t *q, uint16_t *x, int64_t n_words, int mode, int k1, float b1, int k2,
+                          float b2, int k3) {
+    float ic1 = 0, ic2 = 0, ic3 = 0;
+    int t1 = k1, t2 = k1 + k2;
+    if (mode == 0) {
+        ic1 = b1 / (float)k1;
+        ic2 = (b2 - b1) / (float)k2;
+        ic3 = (float)((0.5 - (double)b2) / (double)k3);
+    }
+    for (int64_t w = 0; w < n_words; ++w)
+        for (int k = 0; k < 8; ++k) {
+            int s = (int)((q[w] >> (28 - 4 * k)) & 0xFu) - 8;
+            float v;
+            if (mode == 1) v = (float)s * 0.125f;
+            else if (s < -t2) v = fmaf((float)(s + t2), ic3, -b2);
+            else if (s < -t1) v = fmaf((float)(s + t1), ic2, -b1);
+            else if (s <= t1) v = (float)s * ic1;
+            else if (s <= t2) v = fmaf((float)(s - t1), ic2, b1);
+            else v = fmaf((float)(s - t2), ic3, b2);
+            x[8 * w + k] = f32_to_bf16(v);
+        }
+}
