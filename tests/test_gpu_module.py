@@ -181,7 +181,7 @@ def test_myadam_stochastic_requant_mode(Q):
     m, (packed, scales, zeros) = _make_w4_layer(Q, N, K, 11, False, lbit=0, train=True)
     assert m.weight.residual is None
     opt = Q.MyAdam([{"params": [m.weight], "weight_decay": 0.0}], lr=5e-3, betas=(0.9, 0.95), obit=8, sr_seed=77)
-    x = randn_bf16((64, K), 12).cuda()
+    x = randn_bf16((64, K), 12).cuda().requires_grad_(True)  # a QLinear only back-propagates through its input
     m(x).float().pow(2).mean().backward()
     grad = m.weight.grad.clone()
     opt.step()
@@ -209,7 +209,7 @@ def test_myadam_latent_modes_run_and_descend(Q, lbit):
     if lbit == 16:
         m.weight.residual = Q.DeQfunc_4bit_g(m.weight.data, m.weight.qparam, torch.bfloat16).clone()
     opt = Q.MyAdam([{"params": [m.weight], "weight_decay": 0.0}], lr=2e-4, betas=(0.9, 0.95), obit=8)
-    x = randn_bf16((256, K), 14).cuda()
+    x = randn_bf16((256, K), 14).cuda().requires_grad_(True)
     target = randn_bf16((256, N), 15, 0.1).cuda()
     losses = []
     for _ in range(6):
