@@ -6,15 +6,35 @@
 //
 // Common structure. "A" is the activation-side operand, row-major with the reduction
 // dimension contiguous. "B" is the weight-side operand, presented in LDS as
-// [output column][reduction] exactly like A. A tile row in LDS is 128 bytes (64 bf16 or
-// 128 int8) = eight 16-byte chunks; chunk c of row r is stored at chunk position
-// c ^ ((r ^ (r >> 3)) & 7), which makes the 16-byte fragment reads of 8 consecutive rows
-// and the staging writes hit distinct banks. One MFMA step consumes 32 bytes of every
-// row (chunks 2s and 2s+1), i.e. 4 steps per tile.
+// [output column][reduction] exactly like A. A tile row holds 128 bytes (64 bf16 or
+// 128 int8) = eight 16-byte chunks; one MFMA step consumes 32 bytes of every row
+// (chunks 2s and 2s+1), i.e. 4 steps per tile. Bank conflicts of the 16-byte fragment
+// reads (consecutive rows, same chunk) are avoided in two ways:
+//   * A rows are padded to 144 bytes, so consecutive rows start 16 bytes further round the
+//     banks and every fragment address is (lane base) + compile-time offset;
+//   * B rows stay 128 bytes and chunk c of row r sits at position c ^ ((r ^ (r >> 3)) & 7),
+//     which also keeps the transposing writes of the dX staging (rows 8 apart) apart.
 //
 // The MFMA is issued with the weight fragment as the first operand and the activation
 // fragment as the second, so that D[i][j] has i = output column (n), j = row (m): a
 // lane then owns 4 consecutive n for one m and the epilogue stores 8-byte bf16 quads.
+//
+// Wave specialisation. A workgroup has 2 x WM x WN waves, two per SIMD.
+//   * The first WM x WN ("math") waves issue the MFMAs. They also fetch the A tiles, but with
+//     LDS-direct loads (global_load_lds_dwordx4): no registers, no vector-ALU work, 8
+//     instructions per tile, two tiles ahead of the tile being multiplied (three A buffers).
+//     An LDS-direct load writes lane l at (wave base) + 16*l, so the padded layout is produced
+//     on the global side: the lane that owns 16-byte slot s fetches chunk s%9 of row s/9
+//     (slot 8 of a row is the padding and re-fetches chunk 7).
+//   * The other WM x WN ("weight") waves turn packed int4 codes into bf16 B tiles: code loads two
+//     tiles ahead into registers, dequantisation on the vector ALUs, LDS writes one tile ahead
+//     (two B buffers). A single wave can issue one instruction every 4 cycles, so this
+//     instruction-heavy work must not sit in the waves that feed the matrix pipe.
+// One s_barrier per reduction tile orders the buffers. The barrier is issued without a memory
+// fence and with explicit s_waitcnt values, so that the LDS-direct loads of tile kt+2 stay in
+// flight across it; the loop is unrolled 6x so that every LDS buffer is a distinct __shared__
+// array addressed by a compile-time index (the compiler then knows that a pending LDS-direct
+// load never aliases the fragment reads it schedules next to it).
 #include "lq_common.h"
 
 #include <type_traits>
@@ -40,201 +60,264 @@ struct GemmParams {
     int tiles_m, tiles_n;
 };
 
+typedef __attribute__((address_space(3))) void lds_void;
+typedef const __attribute__((address_space(1))) void gbl_void;
+
+template <int I>
+using ic = std::integral_constant<int, I>;
+
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
 
-// 8 codes of a native word -> 8 bf16 (k order) = 4 packed dwords, w = bf16((q - z) * s).
-// nzs = -(z*s) is exact for integer zeros, and fma(q, s, nzs) rounds the exact (q-z)*s once.
-__device__ __forceinline__ void dequant_word(unsigned word, float s, float nzs, unsigned o[4]) {
-    const unsigned lo4 = word & 0x0F0F0F0Fu;
-    const unsigned hi4 = (word >> 4) & 0x0F0F0F0Fu;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        float e = fmaf((float)((hi4 >> (8 * i)) & 0xFFu), s, nzs);
-        float d = fmaf((float)((lo4 >> (8 * i)) & 0xFFu), s, nzs);
-        o[i] = lq_pack_bf16(e, d);
-    }
+// byte N of a dword as float, one instruction each
+__device__ __forceinline__ float ubyte0(unsigned x) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(x)); return r; }
+__device__ __forceinline__ float ubyte1(unsigned x) { float r; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(x)); return r; }
+__device__ __forceinline__ float ubyte2(unsigned x) { float r; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(x)); return r; }
+__device__ __forceinline__ float ubyte3(unsigned x) { float r; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(x)); return r; }
+
+// 8 codes of a native word -> 8 floats in k order, f = (q - z) * s exactly rounded once:
+// nzs = -(z*s) is exact for integer zeros, and fma(q, s, nzs) rounds the exact product (q-z)*s.
+__device__ __forceinline__ void dequant_word_f32(unsigned word, float s, float nzs, float f[8]) {
+    const unsigned lo4 = word & 0x0F0F0F0Fu;         // odd k
+    const unsigned hi4 = (word >> 4) & 0x0F0F0F0Fu;  // even k
+    f[0] = fmaf(ubyte0(hi4), s, nzs); f[1] = fmaf(ubyte0(lo4), s, nzs);
+    f[2] = fmaf(ubyte1(hi4), s, nzs); f[3] = fmaf(ubyte1(lo4), s, nzs);
+    f[4] = fmaf(ubyte2(hi4), s, nzs); f[5] = fmaf(ubyte2(lo4), s, nzs);
+    f[6] = fmaf(ubyte3(hi4), s, nzs); f[7] = fmaf(ubyte3(lo4), s, nzs);
 }
 
 template <int MODE, int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
-    constexpr int NT = 64 * WM * WN;
+__global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
+    constexpr int NT = 64 * WM * WN;           // threads per role
     constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
     constexpr int FM = TM / 32, FN = TN / 32;  // 32x32 fragments per wave tile
-    constexpr int ROWB = 128;                  // bytes per LDS tile row
-    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB;
+    constexpr int ROWB = 128;                  // bytes of data per tile row (and per LDS row of B)
+    constexpr int AROW = 144;                  // bytes per LDS row of A (16 bytes of padding)
+    constexpr int APT = (BM * 9 + NT - 1) / NT;  // 16-byte LDS slots of A filled per math thread per tile
+    constexpr int A_BYTES = APT * NT * 16, B_BYTES = BN * ROWB;
     constexpr int ESZ = (MODE == MODE_I8) ? 1 : 2;
     constexpr int RT = ROWB / ESZ;  // reduction elements per tile (64 bf16 / 128 int8)
     static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of 32x32");
-    static_assert((BM * 8) % NT == 0, "A staging must divide evenly");
+    static_assert((BN * 8) % NT == 0, "B staging must divide evenly");
+    static_assert(A_BYTES >= BM * AROW, "A buffer too small");
 
-    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * (A_BYTES + B_BYTES)];
-    unsigned char *lds_a = smem;                // [2][BM][128]
-    unsigned char *lds_b = smem + 2 * A_BYTES;  // [2][BN][128]
+    __shared__ __attribute__((aligned(16))) unsigned char lds_a0[A_BYTES];
+    __shared__ __attribute__((aligned(16))) unsigned char lds_a1[A_BYTES];
+    __shared__ __attribute__((aligned(16))) unsigned char lds_a2[A_BYTES];
+    __shared__ __attribute__((aligned(16))) unsigned char lds_b0[B_BYTES];
+    __shared__ __attribute__((aligned(16))) unsigned char lds_b1[B_BYTES];
+    auto abuf = [&](auto i) -> unsigned char * {
+        constexpr int I = decltype(i)::value;
+        if constexpr (I == 0) return lds_a0;
+        else if constexpr (I == 1) return lds_a1;
+        else return lds_a2;
+    };
+    auto bbuf = [&](auto i) -> unsigned char * {
+        constexpr int I = decltype(i)::value;
+        if constexpr (I == 0) return lds_b0;
+        else return lds_b1;
+    };
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    // wave index as a scalar, so that the role split is a uniform branch and LDS-direct
+    // destinations are wave-uniform
+    const int wave_all = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const bool is_weight_wave = wave_all >= WM * WN;
+    const int wave = wave_all % (WM * WN);
+    const int lane = threadIdx.x & 63;
+    const int tid = wave * 64 + lane;  // index within the role
     const int wm = wave % WM, wn = wave / WM;
 
-    // Workgroup ids are dealt round-robin over the 8 XCDs; give each XCD a contiguous range of
-    // tiles (m fastest) so that the tiles resident on one XCD share weight columns in its L2.
+    // Workgroup ids are dealt round-robin over the 8 XCDs (id % 8). Give each XCD a contiguous
+    // range of the tile sequence, and order that sequence in bands of GN tile columns walked
+    // row by row: the ~32 workgroups resident on an XCD then form a 2 x 16 patch that shares
+    // 2 A row-blocks and 16 B column-blocks in that XCD's L2.
     const int nwg = p.tiles_m * p.tiles_n;
     int id = blockIdx.x;
     {
         const int per = nwg / 8;
         if (id < per * 8) id = (id % 8) * per + id / 8;
     }
-    const int tile_m = id % p.tiles_m, tile_n = id / p.tiles_m;
+    constexpr int GN = 16;
+    const int band = id / (p.tiles_m * GN);
+    const int within = id - band * (p.tiles_m * GN);
+    const int rest = p.tiles_n - band * GN;
+    const int bw = rest < GN ? rest : GN;
+    const int tile_m = within / bw, tile_n = band * GN + within % bw;
     const int m0 = tile_m * BM, c0 = tile_n * BN;
+    const int nk = p.R / RT;
+    const int groups_per_row = p.Kw / LQ_GROUP;
 
-    // ---- staging assignments ------------------------------------------------
-    constexpr int APT = BM * 8 / NT;  // 16-byte chunks of A per thread per tile
-    const unsigned char *a_src[APT];
-    int a_dst[APT];
+    if (is_weight_wave) {
+        // ======================= weight waves: B tiles =======================
+        //   I8      : BPT 16-byte chunks per thread, copied through registers.
+        //   W4_FWD  : NW code words (8 k each) of one weight row -> NW 16-byte chunks of that row.
+        //   W4_DX   : one code word (8 k) from each of RPT consecutive weight rows n -> for each
+        //             of the 8 k, RPT consecutive n (2*RPT bytes) of LDS row k.
+        constexpr int BPT = (MODE == MODE_I8) ? BN * 8 / NT : 1;
+        constexpr int NW = (MODE == MODE_W4_FWD) ? BN * 8 / NT : 1;  // tile has BN rows x 8 words
+        constexpr int RPT = (MODE == MODE_W4_DX) ? 8 * BN / NT : 1;  // tile has 64 rows x BN/8 words
+        static_assert(MODE != MODE_W4_FWD || NW == 2 || NW == 4 || NW == 8, "bad fwd staging split");
+        static_assert(MODE != MODE_W4_DX || RPT == 4, "dX staging expects 4 weight rows per thread");
+        constexpr int NSZ = (MODE == MODE_W4_DX) ? RPT : 1;
+        constexpr int NWORDS = NW > RPT ? NW : RPT;
+
+        const unsigned char *b_src[MODE == MODE_I8 ? BPT : (MODE == MODE_W4_DX ? RPT : 1)];
+        int b_dst[MODE == MODE_I8 ? BPT : 1];
+        const unsigned short *s_src[NSZ];
+        const unsigned short *z_src[NSZ];
+        int b_row = 0, b_w0 = 0;  // W4_FWD: LDS row and first word; W4_DX: first LDS row (k) and n-block
+
+        if constexpr (MODE == MODE_I8) {
+#pragma unroll
+            for (int i = 0; i < BPT; ++i) {
+                const int c = i * NT + tid;
+                const int row = c >> 3, ch = c & 7;
+                int gr = c0 + row;
+                gr = gr < p.C ? gr : p.C - 1;
+                b_src[i] = (const unsigned char *)p.b + (long long)gr * p.Kw + ch * 16;
+                b_dst[i] = row * ROWB + ((ch ^ swz(row)) << 4);
+            }
+        } else if constexpr (MODE == MODE_W4_FWD) {
+            constexpr int TPR = 8 / NW;  // threads per weight row
+            b_row = tid / TPR;
+            b_w0 = (tid % TPR) * NW;
+            int gr = c0 + b_row;
+            gr = gr < p.C ? gr : p.C - 1;
+            b_src[0] = (const unsigned char *)p.b + (long long)gr * (p.Kw / 2) + b_w0 * 4;
+            s_src[0] = p.scales + (long long)gr * groups_per_row;
+            z_src[0] = p.zeros + (long long)gr * groups_per_row;
+        } else {
+            constexpr int KWT = BN / 8;  // code words per weight row in the tile
+            const int kw = tid % KWT, nblk = tid / KWT;
+#pragma unroll
+            for (int r = 0; r < RPT; ++r) {
+                const int n = nblk * RPT + r;  // tile offset along n is added per tile
+                b_src[r] = (const unsigned char *)p.b + (long long)n * (p.Kw / 2) + (c0 / 8 + kw) * 4;
+                const int g = (c0 + kw * 8) / LQ_GROUP;
+                s_src[r] = p.scales + (long long)n * groups_per_row + g;
+                z_src[r] = p.zeros + (long long)n * groups_per_row + g;
+            }
+            b_row = kw * 8;
+            b_w0 = nblk;
+        }
+
+        struct Stage {
+            u32x4_t b[BPT];      // I8
+            unsigned w[NWORDS];  // W4 code words
+            unsigned short s[NSZ], z[NSZ];
+        };
+        Stage S0, S1;
+
+        auto load_b = [&](int kt, Stage &S) {
+            if constexpr (MODE == MODE_I8) {
+#pragma unroll
+                for (int i = 0; i < BPT; ++i) S.b[i] = *reinterpret_cast<const u32x4_t *>(b_src[i] + (long long)kt * ROWB);
+            } else if constexpr (MODE == MODE_W4_FWD) {
+                const unsigned char *src = b_src[0] + (long long)kt * 32;
+                if constexpr (NW == 8) {
+                    u32x4_t v0 = *reinterpret_cast<const u32x4_t *>(src), v1 = *reinterpret_cast<const u32x4_t *>(src + 16);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { S.w[i] = v0[i]; S.w[4 + i] = v1[i]; }
+                } else if constexpr (NW == 4) {
+                    u32x4_t v = *reinterpret_cast<const u32x4_t *>(src);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) S.w[i] = v[i];
+                } else {
+                    u32x2_t v = *reinterpret_cast<const u32x2_t *>(src);
+                    S.w[0] = v[0]; S.w[1] = v[1];
+                }
+                S.s[0] = s_src[0][kt >> 1];
+                S.z[0] = z_src[0][kt >> 1];
+            } else {
+                const long long row_off = (long long)kt * 64;
+#pragma unroll
+                for (int r = 0; r < RPT; ++r) {
+                    S.w[r] = *reinterpret_cast<const unsigned *>(b_src[r] + row_off * (p.Kw / 2));
+                    S.s[r] = s_src[r][row_off * groups_per_row];
+                    S.z[r] = z_src[r][row_off * groups_per_row];
+                }
+            }
+        };
+
+        auto store_b = [&](unsigned char *lb, Stage &S) {
+            if constexpr (MODE == MODE_I8) {
+#pragma unroll
+                for (int i = 0; i < BPT; ++i) *reinterpret_cast<u32x4_t *>(lb + b_dst[i]) = S.b[i];
+            } else if constexpr (MODE == MODE_W4_FWD) {
+                const float s = lq_bf16_bits_to_f32(S.s[0]);
+                const float nzs = -(lq_bf16_bits_to_f32(S.z[0]) * s);
+#pragma unroll
+                for (int w = 0; w < NW; ++w) {
+                    float f[8];
+                    dequant_word_f32(S.w[w], s, nzs, f);
+                    const int ch = b_w0 + w;
+                    u32x4_t v = {lq_pack_bf16(f[0], f[1]), lq_pack_bf16(f[2], f[3]), lq_pack_bf16(f[4], f[5]),
+                                 lq_pack_bf16(f[6], f[7])};
+                    *reinterpret_cast<u32x4_t *>(lb + b_row * ROWB + ((ch ^ swz(b_row)) << 4)) = v;
+                }
+            } else {
+                float f[RPT][8];
+#pragma unroll
+                for (int r = 0; r < RPT; ++r) {
+                    const float s = lq_bf16_bits_to_f32(S.s[r]);
+                    const float nzs = -(lq_bf16_bits_to_f32(S.z[r]) * s);
+                    dequant_word_f32(S.w[r], s, nzs, f[r]);
+                }
+                const int byte0 = b_w0 * RPT * 2;  // byte offset of this thread's n-block inside the LDS row
+                const int ch = byte0 >> 4, sub = byte0 & 15;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int row = b_row + j;
+                    u32x2_t v = {lq_pack_bf16(f[0][j], f[1][j]), lq_pack_bf16(f[2][j], f[3][j])};
+                    *reinterpret_cast<u32x2_t *>(lb + row * ROWB + ((ch ^ swz(row)) << 4) + sub) = v;
+                }
+            }
+        };
+
+        // Barrier after the LDS writes of this wave have completed (no fence: see file header).
+        auto publish = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+        load_b(0, S0);
+        load_b(nk > 1 ? 1 : 0, S1);
+        store_b(lds_b0, S0);
+        publish();
+        // iteration kt: codes of tile kt+2 -> registers, tile kt+1 -> LDS buffer (kt+1)&1
+        int kt = 0;
+        for (; kt + 2 <= nk; kt += 2) {
+            load_b(kt + 2 < nk ? kt + 2 : nk - 1, S0);
+            store_b(lds_b1, S1);
+            publish();
+            load_b(kt + 3 < nk ? kt + 3 : nk - 1, S1);
+            if (kt + 2 < nk) store_b(lds_b0, S0);
+            publish();
+        }
+        if (kt < nk) publish();  // odd tile count: the last tile has nothing left to prepare
+        return;
+    }
+
+    // =========================== math waves: A tiles + MFMA ===========================
+    static_assert(APT <= 30, "vmcnt range");
+    // Lane-varying 32-bit byte offsets into A; the tile offset (kt * 128 bytes) is wave-uniform.
+    unsigned a_off[APT];
     const long long lda = (long long)p.R * ESZ;
 #pragma unroll
     for (int i = 0; i < APT; ++i) {
-        const int c = i * NT + tid;
-        const int row = c >> 3, ch = c & 7;
+        const int slot = i * NT + tid;  // LDS slot: row slot/9, chunk slot%9 (8 = padding)
+        int row = slot / 9, ch = slot % 9;
+        ch = ch < 8 ? ch : 7;
         int gr = m0 + row;
         gr = gr < p.M ? gr : p.M - 1;
-        a_src[i] = (const unsigned char *)p.a + gr * lda + ch * 16;
-        a_dst[i] = row * ROWB + ((ch ^ swz(row)) << 4);
+        a_off[i] = (unsigned)((gr - m0) * lda + ch * 16);
     }
-
-    // B staging registers
-    constexpr int BPT_I8 = (MODE == MODE_I8) ? BN * 8 / NT : 1;
-    constexpr int BPT_W4 = (MODE == MODE_W4_FWD) ? (BN * 2 + NT - 1) / NT : 1;
-    const unsigned char *b_src[MODE == MODE_I8 ? BPT_I8 : (MODE == MODE_W4_FWD ? BPT_W4 : 4)];
-    int b_dst[MODE == MODE_I8 ? BPT_I8 : (MODE == MODE_W4_FWD ? BPT_W4 : 1)];
-    const unsigned short *s_src[MODE == MODE_W4_DX ? 4 : BPT_W4];
-    const unsigned short *z_src[MODE == MODE_W4_DX ? 4 : BPT_W4];
-    int b_row[BPT_W4];
-    int b_half[BPT_W4];
-    const int groups_per_row = p.Kw / LQ_GROUP;
-
-    if (MODE == MODE_I8) {
+    const unsigned char *a_base = (const unsigned char *)p.a + m0 * lda;
+    // LDS-direct load: lane l of the wave writes 16 bytes at (wave-uniform base) + 16*l.
+    auto issue_a = [&](int kt, unsigned char *la) {
+        const unsigned char *src = a_base + (long long)kt * ROWB;
 #pragma unroll
-        for (int i = 0; i < BPT_I8; ++i) {
-            const int c = i * NT + tid;
-            const int row = c >> 3, ch = c & 7;
-            int gr = c0 + row;
-            gr = gr < p.C ? gr : p.C - 1;
-            b_src[i] = (const unsigned char *)p.b + (long long)gr * p.Kw + ch * 16;
-            b_dst[i] = row * ROWB + ((ch ^ swz(row)) << 4);
-        }
-    } else if (MODE == MODE_W4_FWD) {
-        // tile = BN rows x 32 bytes of codes; a thread takes 16 bytes (32 codes) of one row.
-#pragma unroll
-        for (int i = 0; i < BPT_W4; ++i) {
-            const int c = i * NT + tid;
-            const int row = (c >> 1) % BN, half = c & 1;
-            int gr = c0 + row;
-            gr = gr < p.C ? gr : p.C - 1;
-            b_src[i] = (const unsigned char *)p.b + (long long)gr * (p.Kw / 2) + half * 16;
-            s_src[i] = p.scales + (long long)gr * groups_per_row;
-            z_src[i] = p.zeros + (long long)gr * groups_per_row;
-            b_row[i] = row;
-            b_half[i] = half;
-        }
-    } else {
-        // dX: tile = 64 weight rows (reduction n) x BN columns (k); a thread takes one code word
-        // (8 k) from each of 4 consecutive rows and emits, per k, 4 consecutive n (8 bytes).
-        static_assert(MODE != MODE_W4_DX || (NT == 256 && BN == 128), "dX staging assumes 256 threads, 128 columns");
-        const int kw = tid & 15, nblk = tid >> 4;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int n = nblk * 4 + r;  // + tile offset along n added per tile
-            b_src[r] = (const unsigned char *)p.b + (long long)n * (p.Kw / 2) + (c0 / 8 + kw) * 4;
-            const int g = (c0 + kw * 8) / LQ_GROUP;
-            s_src[r] = p.scales + (long long)n * groups_per_row + g;
-            z_src[r] = p.zeros + (long long)n * groups_per_row + g;
-        }
-        b_dst[0] = (kw * 8) * ROWB;  // row base; chunk/half resolved at write time
-        b_row[0] = nblk;
-        b_half[0] = 0;
-    }
-
-    // ---- register staging buffers --------------------------------------------
-    u32x4_t a_reg[APT];
-    u32x4_t b_reg[MODE == MODE_I8 ? BPT_I8 : BPT_W4];
-    unsigned bw_reg[4];
-    unsigned short s_reg[MODE == MODE_W4_DX ? 4 : BPT_W4], z_reg[MODE == MODE_W4_DX ? 4 : BPT_W4];
-
-    auto load_tile = [&](int kt) {
-#pragma unroll
-        for (int i = 0; i < APT; ++i) a_reg[i] = *reinterpret_cast<const u32x4_t *>(a_src[i] + (long long)kt * ROWB);
-        if (MODE == MODE_I8) {
-#pragma unroll
-            for (int i = 0; i < BPT_I8; ++i)
-                b_reg[i] = *reinterpret_cast<const u32x4_t *>(b_src[i] + (long long)kt * ROWB);
-        } else if (MODE == MODE_W4_FWD) {
-#pragma unroll
-            for (int i = 0; i < BPT_W4; ++i) {
-                b_reg[i] = *reinterpret_cast<const u32x4_t *>(b_src[i] + (long long)kt * 32);
-                s_reg[i] = s_src[i][kt >> 1];
-                z_reg[i] = z_src[i][kt >> 1];
-            }
-        } else {
-            const long long row_off = (long long)kt * 64;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                bw_reg[r] = *reinterpret_cast<const unsigned *>(b_src[r] + row_off * (p.Kw / 2));
-                s_reg[r] = s_src[r][row_off * groups_per_row];
-                z_reg[r] = z_src[r][row_off * groups_per_row];
-            }
-        }
+        for (int i = 0; i < APT; ++i)
+            __builtin_amdgcn_global_load_lds((gbl_void *)(src + a_off[i]), (lds_void *)(la + (i * NT + wave * 64) * 16), 16,
+                                             0, 0);
     };
 
-    auto store_tile = [&](int buf) {
-        unsigned char *la = lds_a + buf * A_BYTES;
-        unsigned char *lb = lds_b + buf * B_BYTES;
-#pragma unroll
-        for (int i = 0; i < APT; ++i) *reinterpret_cast<u32x4_t *>(la + a_dst[i]) = a_reg[i];
-        if (MODE == MODE_I8) {
-#pragma unroll
-            for (int i = 0; i < BPT_I8; ++i) *reinterpret_cast<u32x4_t *>(lb + b_dst[i]) = b_reg[i];
-        } else if (MODE == MODE_W4_FWD) {
-#pragma unroll
-            for (int i = 0; i < BPT_W4; ++i) {
-                if (BN * 2 % NT == 0 || i * NT + tid < BN * 2) {
-                    const float s = lq_bf16_bits_to_f32(s_reg[i]);
-                    const float nzs = -(lq_bf16_bits_to_f32(z_reg[i]) * s);
-                    const int row = b_row[i];
-#pragma unroll
-                    for (int w = 0; w < 4; ++w) {
-                        unsigned o[4];
-                        dequant_word(b_reg[i][w], s, nzs, o);
-                        const int ch = b_half[i] * 4 + w;
-                        u32x4_t v = {o[0], o[1], o[2], o[3]};
-                        *reinterpret_cast<u32x4_t *>(lb + row * ROWB + ((ch ^ swz(row)) << 4)) = v;
-                    }
-                }
-            }
-        } else {
-            // 4 rows (n) x 8 k  ->  for each k: 4 consecutive n = 8 bytes at LDS row k.
-            unsigned o[4][4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float s = lq_bf16_bits_to_f32(s_reg[r]);
-                const float nzs = -(lq_bf16_bits_to_f32(z_reg[r]) * s);
-                dequant_word(bw_reg[r], s, nzs, o[r]);
-            }
-            const int nblk = b_row[0];
-            const int ch = nblk >> 1, hf = nblk & 1;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int row = (b_dst[0] / ROWB) + j;
-                // element j of word r: dword j/2, half j&1
-                unsigned e[4];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) e[r] = (j & 1) ? (o[r][j >> 1] >> 16) : (o[r][j >> 1] & 0xFFFFu);
-                u32x2_t v = {e[0] | (e[1] << 16), e[2] | (e[3] << 16)};
-                *reinterpret_cast<u32x2_t *>(lb + row * ROWB + ((ch ^ swz(row)) << 4) + hf * 8) = v;
-            }
-        }
-    };
-
-    // ---- accumulators -------------------------------------------------------
     using acc_t = typename std::conditional<MODE == MODE_I8, i32x16_t, f32x16_t>::type;
     acc_t acc[FN][FM];
 #pragma unroll
@@ -244,51 +327,81 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmParams p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    const int nk = p.R / RT;
     const int frag_row = lane & 31, kh = lane >> 5;
-
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
-
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) load_tile(kt + 1);
-
-        const unsigned char *la = lds_a + buf * A_BYTES + (wm * TM) * ROWB;
-        const unsigned char *lb = lds_b + buf * B_BYTES + (wn * TN) * ROWB;
+    const int a_lane_off = (wm * TM + frag_row) * AROW + kh * 16;  // + i*32*AROW + ks*32: compile-time
+    int b_frag_off[FN], b_frag_swz[FN];
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            const int ch = 2 * ks + kh;
-            u32x4_t af[FM], bf[FN];
-#pragma unroll
-            for (int i = 0; i < FM; ++i) {
-                const int row = i * 32 + frag_row;
-                af[i] = *reinterpret_cast<const u32x4_t *>(la + row * ROWB + ((ch ^ swz(wm * TM + row)) << 4));
-            }
-#pragma unroll
-            for (int i = 0; i < FN; ++i) {
-                const int row = i * 32 + frag_row;
-                bf[i] = *reinterpret_cast<const u32x4_t *>(lb + row * ROWB + ((ch ^ swz(wn * TN + row)) << 4));
-            }
-#pragma unroll
-            for (int i = 0; i < FN; ++i)
-#pragma unroll
-                for (int j = 0; j < FM; ++j) {
-                    if constexpr (MODE == MODE_I8) {
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf[i]),
-                                                                         __builtin_bit_cast(i32x4_t, af[j]),
-                                                                         acc[i][j], 0, 0, 0);
-                    } else {
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[i]),
-                                                                           __builtin_bit_cast(bf16x8_t, af[j]),
-                                                                           acc[i][j], 0, 0, 0);
-                    }
-                }
-        }
-        if (kt + 1 < nk) store_tile(buf ^ 1);
-        __syncthreads();
+    for (int i = 0; i < FN; ++i) {
+        const int row = wn * TN + i * 32 + frag_row;
+        b_frag_off[i] = row * ROWB;
+        b_frag_swz[i] = swz(row);
     }
+    auto read_frags = [&](const unsigned char *la, const unsigned char *lb, int ks, u32x4_t *af, u32x4_t *bf) {
+        const int ch = 2 * ks + kh;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+            af[i] = *reinterpret_cast<const u32x4_t *>(la + a_lane_off + i * 32 * AROW + ks * 32);
+#pragma unroll
+        for (int i = 0; i < FN; ++i)
+            bf[i] = *reinterpret_cast<const u32x4_t *>(lb + b_frag_off[i] + ((ch ^ b_frag_swz[i]) << 4));
+    };
+    auto mfma_step = [&](const u32x4_t *af, const u32x4_t *bf) {
+#pragma unroll
+        for (int i = 0; i < FN; ++i)
+#pragma unroll
+            for (int j = 0; j < FM; ++j) {
+                if constexpr (MODE == MODE_I8) {
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf[i]),
+                                                                     __builtin_bit_cast(i32x4_t, af[j]), acc[i][j], 0, 0, 0);
+                } else {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[i]),
+                                                                       __builtin_bit_cast(bf16x8_t, af[j]), acc[i][j], 0, 0, 0);
+                }
+            }
+    };
+
+    // Tile kt: A in buffer kt%3, B in buffer kt%2. First put the A loads of tile kt+2 in flight
+    // (into the buffer tile kt-1 just left), then 4 MFMA steps with double-buffered fragments,
+    // then wait until this wave's part of tile kt+1 has landed (all but the newest APT loads)
+    // and its fragment reads have returned, and meet the other waves.
+    auto tile_step = [&](int kt, auto ai, auto bi) {
+        constexpr int AI = decltype(ai)::value, BI = decltype(bi)::value;
+        issue_a(kt + 2 < nk ? kt + 2 : nk - 1, abuf(ic<(AI + 2) % 3>()));
+        const unsigned char *la = abuf(ic<AI>()), *lb = bbuf(ic<BI>());
+        u32x4_t af[2][FM], bf[2][FN];
+        read_frags(la, lb, 0, af[0], bf[0]);
+        read_frags(la, lb, 1, af[1], bf[1]);
+        mfma_step(af[0], bf[0]);
+        read_frags(la, lb, 2, af[0], bf[0]);
+        mfma_step(af[1], bf[1]);
+        read_frags(la, lb, 3, af[1], bf[1]);
+        mfma_step(af[0], bf[0]);
+        mfma_step(af[1], bf[1]);
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(APT) : "memory");
+    };
+
+    issue_a(0, lds_a0);
+    issue_a(nk > 1 ? 1 : 0, lds_a1);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(APT) : "memory");
+    int kt = 0;
+    for (; kt + 6 <= nk; kt += 6) {
+        tile_step(kt, ic<0>(), ic<0>());
+        tile_step(kt + 1, ic<1>(), ic<1>());
+        tile_step(kt + 2, ic<2>(), ic<0>());
+        tile_step(kt + 3, ic<0>(), ic<1>());
+        tile_step(kt + 4, ic<1>(), ic<0>());
+        tile_step(kt + 5, ic<2>(), ic<1>());
+    }
+    // remainder of 0..5 tiles; kt is a multiple of 6 here, so the buffer phases restart at 0
+    const int rem = nk - kt;
+    if (rem > 0) tile_step(kt, ic<0>(), ic<0>());
+    if (rem > 1) tile_step(kt + 1, ic<1>(), ic<1>());
+    if (rem > 2) tile_step(kt + 2, ic<2>(), ic<0>());
+    if (rem > 3) tile_step(kt + 3, ic<0>(), ic<1>());
+    if (rem > 4) tile_step(kt + 4, ic<1>(), ic<0>());
+
+    // the clamped prefetches issued by the last two tiles are still writing LDS: drain them
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     // ---- epilogue -----------------------------------------------------------
     // acc[i][j][r]: column c = c0 + wn*TN + i*32 + 8*(r/4) + 4*(lane/32) + r%4, row m = m0 + wm*TM + j*32 + lane%32.
@@ -334,7 +447,7 @@ int launch_gemm(GemmParams p, hipStream_t st, const char *who) {
     auto kern = gemm_kernel<MODE, BM, BN, WM, WN>;
     const long long nwg = (long long)p.tiles_m * p.tiles_n;
     if (nwg > 0x7FFFFFFFll) return lq_fail(LQ_ERR_BAD_ARG, "%s: problem too large", who);
-    hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(64 * WM * WN), 0, st, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(128 * WM * WN), 0, st, p);
     return lq_check_launch(who);
 }
 
