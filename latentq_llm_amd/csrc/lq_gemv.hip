@@ -13,11 +13,19 @@
 // so unpacking costs < 1 VALU operation per weight. The scale is applied in fp32 to the
 // per-group sums, i.e. weights are NOT rounded to bf16 first (slightly more accurate than
 // the dequantise-then-multiply path).
+//
+// Memory access. The MFMA wants lane 16*kq + n to hold 8 k of weight row n, which as a load
+// pattern would put the 4 lanes of every quad on 4 different rows (64 separate cache-line
+// requests per wave instruction). The codes are therefore loaded with lane 4*r + c reading
+// 16-byte chunk c of row r (a quad reads 64 contiguous bytes) and moved to the MFMA layout
+// with one ds_bpermute per dword. For the same reason the scales and zeros of a batch of 4
+// consecutive groups are fetched as one 8-byte load by the 16 lanes kq = 0 only and then
+// broadcast, and activation loads are limited to the lanes of live tokens: what a vector load
+// costs here is cache-line look-ups per quad, not bytes.
 #include "lq_common.h"
 
 namespace {
 
-constexpr int kUnroll = 4;  // groups in flight per wave
 
 // k-slot order produced by the AND-OR unpack of one code word: slots (2i, 2i+1) of dword i
 // hold codes (1,5), (0,4), (3,7), (2,6). The activation fragment is permuted to match.
@@ -34,7 +42,14 @@ __device__ __forceinline__ void permute_x(const u32x4_t &d, unsigned a[4]) {
     a[3] = __builtin_amdgcn_perm(d[3], d[1], 0x05040100u);  // (x2, x6)
 }
 
-template <int WAVES>
+typedef __attribute__((address_space(3))) void lds_void;
+typedef const __attribute__((address_space(1))) void gbl_void;
+
+constexpr int kUnroll = 4;       // groups per batch (scale/zero batches are 4 x bf16 = 8 bytes)
+constexpr int kXRow = 1024 + 16;  // LDS bytes per staged token row: 4 groups x 256 B, padded against bank conflicts
+
+// MP = number of token rows staged per wave and batch (>= M).
+template <int WAVES, int MP>
 __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *__restrict__ x,
                                                           const unsigned char *__restrict__ codes,
                                                           const unsigned short *__restrict__ scales,
@@ -42,64 +57,102 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
                                                           const unsigned short *__restrict__ bias,
                                                           unsigned short *__restrict__ y, int M, int N, int K) {
     __shared__ float red[WAVES][4][64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __shared__ __attribute__((aligned(16))) unsigned char xs[WAVES][MP][kXRow];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // scalar: uniform control flow
     const int n = lane & 15, kq = lane >> 4;
     const int row = blockIdx.x * 16 + n;  // weight row of this lane's B fragment
     const int G = K / LQ_GROUP;
-    const bool has_x = n < M;  // as an A-fragment lane, `n` is the token index
 
-    const unsigned char *wrow = codes + (long long)row * (K / 2) + kq * 16;
-    const unsigned short *xrow = x + (long long)(has_x ? n : 0) * K + kq * 32;
+    // load layout of the codes: lane 4*r + c -> row r of this block, 16-byte chunk c of the group
+    const unsigned char *wrow = codes + (long long)(blockIdx.x * 16 + (lane >> 2)) * (K / 2) + (lane & 3) * 16;
+    const int bperm_src = (4 * n + kq) * 4;  // ds_bpermute: take from lane 4*n + kq
+    const int bcast_src = n * 4;             // ds_bpermute: take from lane n (kq = 0)
     const unsigned short *srow = scales + (long long)row * G;
     const unsigned short *zrow = zeros + (long long)row * G;
+    // As an A-fragment lane, `n` is the token index; lanes of tokens >= M re-read the last staged
+    // row: they only feed accumulator rows m >= M, which are never stored.
+    const unsigned char *xfrag = &xs[wave][n < M ? n : M - 1][kq * 64];
 
     const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 
     for (int g0 = wave * kUnroll; g0 < G; g0 += WAVES * kUnroll) {
+        const bool full = g0 + kUnroll <= G;  // a short tail batch re-reads the last group with zero scale
+        // ---- activations: one LDS-direct load per token row (1 KB = this batch's 512 k), coalesced.
+        //      In a tail batch the lanes past the end of the row re-read its first bytes (dead groups).
+        {
+            const long long xoff = (long long)g0 * (LQ_GROUP * 2) + lane * 16;
+            const long long lim = (long long)K * 2;
+            const long long off = xoff < lim ? xoff : 0;
+#pragma unroll
+            for (int m = 0; m < MP; ++m)
+                if (m < M)
+                    __builtin_amdgcn_global_load_lds((gbl_void *)((const unsigned char *)x + (long long)m * lim + off),
+                                                     (lds_void *)&xs[wave][m][0], 16, 0, 0);
+        }
+        // ---- codes, scales, zeros
         u32x4_t wv[kUnroll];
-        u32x4_t xv[kUnroll][4];
-        unsigned short sb[kUnroll], zb[kUnroll];
+        float sc[kUnroll], zz[kUnroll];
+        u32x2_t sraw = {0u, 0u}, zraw = {0u, 0u};
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            const int g = g0 + u;
-            if (g < G) {
-                wv[u] = *reinterpret_cast<const u32x4_t *>(wrow + g * 64);
-                sb[u] = srow[g];
-                zb[u] = zrow[g];
+            const int g = g0 + u < G ? g0 + u : G - 1;
+            wv[u] = *reinterpret_cast<const u32x4_t *>(wrow + g * 64);
+        }
+        if (full) {
+            if (kq == 0) {
+                sraw = *reinterpret_cast<const u32x2_t *>(srow + g0);
+                zraw = *reinterpret_cast<const u32x2_t *>(zrow + g0);
+            }
+            unsigned s01 = (unsigned)__builtin_amdgcn_ds_bpermute(bcast_src, (int)sraw[0]);
+            unsigned s23 = (unsigned)__builtin_amdgcn_ds_bpermute(bcast_src, (int)sraw[1]);
+            unsigned z01 = (unsigned)__builtin_amdgcn_ds_bpermute(bcast_src, (int)zraw[0]);
+            unsigned z23 = (unsigned)__builtin_amdgcn_ds_bpermute(bcast_src, (int)zraw[1]);
+            sc[0] = lq_bf16_lo(s01); sc[1] = lq_bf16_hi(s01); sc[2] = lq_bf16_lo(s23); sc[3] = lq_bf16_hi(s23);
+            zz[0] = 128.0f + lq_bf16_lo(z01); zz[1] = 128.0f + lq_bf16_hi(z01);
+            zz[2] = 128.0f + lq_bf16_lo(z23); zz[3] = 128.0f + lq_bf16_hi(z23);
+        } else {
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    if (has_x) {
-                        xv[u][t] = *reinterpret_cast<const u32x4_t *>(xrow + g * LQ_GROUP + t * 8);
-                    } else {
-                        xv[u][t] = u32x4_t{0u, 0u, 0u, 0u};
-                    }
-                }
+            for (int u = 0; u < kUnroll; ++u) {
+                const bool live = g0 + u < G;
+                const int g = live ? g0 + u : G - 1;
+                sc[u] = live ? lq_bf16_bits_to_f32(srow[g]) : 0.0f;
+                zz[u] = 128.0f + lq_bf16_bits_to_f32(zrow[g]);
+            }
+        }
+        // ---- codes to the MFMA lane layout
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) wv[u][t] = (unsigned)__builtin_amdgcn_ds_bpermute(bperm_src, (int)wv[u][t]);
+        // ---- MFMAs, step index outermost so that consecutive MFMAs feed different accumulators
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the staged rows have landed in LDS
+        f32x4_t P[kUnroll], S[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) P[u] = S[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                unsigned b[4], a[4];
+                unpack_word_128q(wv[u][t], b);
+                const u32x4_t xv = *reinterpret_cast<const u32x4_t *>(xfrag + u * 256 + t * 16);
+                permute_x(xv, a);
+                const u32x4_t av = {a[0], a[1], a[2], a[3]};
+                const u32x4_t bv = {b[0], b[1], b[2], b[3]};
+                P[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                               __builtin_bit_cast(bf16x8_t, bv), P[u], 0, 0, 0);
+                S[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                               __builtin_bit_cast(bf16x8_t, ones), S[u], 0, 0, 0);
             }
         }
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const int g = g0 + u;
-            if (g < G) {
-                f32x4_t P = {0.f, 0.f, 0.f, 0.f}, S = {0.f, 0.f, 0.f, 0.f};
+        for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    unsigned b[4], a[4];
-                    unpack_word_128q(wv[u][t], b);
-                    permute_x(xv[u][t], a);
-                    const u32x4_t av = {a[0], a[1], a[2], a[3]};
-                    const u32x4_t bv = {b[0], b[1], b[2], b[3]};
-                    P = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
-                                                                __builtin_bit_cast(bf16x8_t, bv), P, 0, 0, 0);
-                    S = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
-                                                                __builtin_bit_cast(bf16x8_t, ones), S, 0, 0, 0);
-                }
-                const float s = lq_bf16_bits_to_f32(sb[u]);
-                const float zz = 128.0f + lq_bf16_bits_to_f32(zb[u]);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) acc[r] = fmaf(s, fmaf(-zz, S[r], P[r]), acc[r]);
-            }
-        }
+            for (int r = 0; r < 4; ++r) acc[r] = fmaf(sc[u], fmaf(-zz[u], S[u][r], P[u][r]), acc[r]);
+        // the next batch overwrites the staged rows: all fragment reads above must have returned
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
 
 #pragma unroll
@@ -123,19 +176,26 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
 
 int lq_gemv_a16w4_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
                          void *y, int M, int N, int K, hipStream_t st) {
-    // N % 16 == 0 and K % 128 == 0 are guaranteed by the caller.
+    // N % 16 == 0, K % 128 == 0 and 1 <= M <= 16 are guaranteed by the caller.
     const int blocks = N / 16;
     const int G = K / LQ_GROUP;
-    // Enough waves to keep every SIMD busy, but at least one batch of groups per wave.
-    int waves = 4;
-    while (waves < 16 && (long long)blocks * waves < 4096 && G >= waves * 2 * kUnroll) waves *= 2;
-#define LQ_GEMV_LAUNCH(W)                                                                                         \
-    hipLaunchKernelGGL(gemv_kernel<W>, dim3(blocks), dim3(64 * W), 0, st, (const unsigned short *)x,               \
+    // One batch of 4 groups per wave when possible: all of a wave's loads are then in flight at once.
+    // With 16 staged token rows a wave needs 16.25 KB of LDS, which caps the workgroup at 8 waves.
+#define LQ_GEMV_LAUNCH(W, MP)                                                                                     \
+    hipLaunchKernelGGL((gemv_kernel<W, MP>), dim3(blocks), dim3(64 * W), 0, st, (const unsigned short *)x,         \
                        (const unsigned char *)codes, (const unsigned short *)scales, (const unsigned short *)zeros, \
                        (const unsigned short *)bias, (unsigned short *)y, M, N, K)
-    if (waves == 4) LQ_GEMV_LAUNCH(4);
-    else if (waves == 8) LQ_GEMV_LAUNCH(8);
-    else LQ_GEMV_LAUNCH(16);
+    const int want = (G + 3) / 4;  // waves for one batch each
+    if (M <= 4) {
+        if (want <= 2) LQ_GEMV_LAUNCH(2, 4);
+        else if (want <= 4) LQ_GEMV_LAUNCH(4, 4);
+        else if (want <= 8) LQ_GEMV_LAUNCH(8, 4);
+        else LQ_GEMV_LAUNCH(16, 4);
+    } else {
+        if (want <= 2) LQ_GEMV_LAUNCH(2, 16);
+        else if (want <= 4) LQ_GEMV_LAUNCH(4, 16);
+        else LQ_GEMV_LAUNCH(8, 16);
+    }
 #undef LQ_GEMV_LAUNCH
     return lq_check_launch("lq_a16w4_fwd(gemv)");
 }
