@@ -58,6 +58,7 @@ const char *lq_last_error(void);
  *   code' = v<0 or NaN ? 0 : v>15 ? 15 : floor(v)
  * codes_in / codes_out: N*K/2 bytes, native layout (may alias each other).
  * scales, zeros: bf16[N*K/128]. grad: bf16[N,K] row-major. lr: host float.
+ * codes_in, codes_out, grad and u must be 16-byte aligned.
  * Noise: if u_or_null != NULL it is an fp32[N,K] array of u in [0,1);
  * otherwise u for flat element index i is word (i & 3) of
  * Philox4x32-10(counter = philox_offset + i/4 as a 128-bit little-endian

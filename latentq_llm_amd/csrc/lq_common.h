@@ -63,9 +63,15 @@ __host__ __device__ __forceinline__ lq_u4 lq_philox4x32_10(unsigned c0, unsigned
     for (int r = 0; r < 10; ++r) {
         unsigned long long p0 = (unsigned long long)LQ_PHILOX_M0 * c0;
         unsigned long long p1 = (unsigned long long)LQ_PHILOX_M1 * c2;
+#if defined(__HIP_DEVICE_COMPILE__)
+        // three-input XOR in one instruction (v_bitop3_b32, truth table 0x96)
+        unsigned n0 = __builtin_amdgcn_bitop3_b32((unsigned)(p1 >> 32), c1, k0, 0x96);
+        unsigned n2 = __builtin_amdgcn_bitop3_b32((unsigned)(p0 >> 32), c3, k1, 0x96);
+#else
         unsigned n0 = (unsigned)(p1 >> 32) ^ c1 ^ k0;
-        unsigned n1 = (unsigned)p1;
         unsigned n2 = (unsigned)(p0 >> 32) ^ c3 ^ k1;
+#endif
+        unsigned n1 = (unsigned)p1;
         unsigned n3 = (unsigned)p0;
         c0 = n0; c1 = n1; c2 = n2; c3 = n3;
         k0 += LQ_PHILOX_W0;

@@ -1,10 +1,12 @@
 // Kernel (1): single-pass stochastic-rounding latent requantizer for gfx950.
 //
-// One 32-bit word of packed codes (8 consecutive k of one row) is the unit of
-// work; a word never straddles a 128-element quantisation group, so scale,
-// zero and the reciprocal of the scale are per-word constants. All loads of a
-// thread's words are issued before any arithmetic so that a wave keeps
-// 4 x (4 B codes + 16 B gradient) per lane in flight.
+// A thread owns 4 consecutive 32-bit words of packed codes (32 consecutive k of
+// one row): they never straddle a 128-element quantisation group, so scale,
+// zero and the reciprocal of the scale are per-thread constants, the codes
+// move as one 16-byte load and one 16-byte store, and the 8 Philox blocks of
+// the thread have consecutive counters. The kernel is bound by vector-ALU
+// instruction issue (Philox4x32-10 alone is ~10 instructions per element), so
+// everything per element is kept to the minimum number of instructions.
 //
 // This translation unit is compiled with -ffp-contract=off: every rounding
 // below is written out explicitly (fmaf where a fused operation is meant).
@@ -13,13 +15,7 @@
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kWordsPerThread = 4;
-
-struct WordIn {
-    unsigned codes;
-    u32x4_t g;  // 8 bf16 gradients, element j in half (j&1) of dword j/2
-    unsigned short s_bits, z_bits;
-};
+constexpr int kWordsPerThread = 4;  // 4 consecutive words = 32 elements of one quantisation group
 
 // Exact restatement of the update rule for one element (any inputs).
 __device__ __forceinline__ unsigned requant_elem_exact(unsigned q, float s, float z, float g, float lr, float u) {
@@ -33,131 +29,105 @@ __device__ __forceinline__ unsigned requant_elem_exact(unsigned q, float s, floa
     return (unsigned)c;                                  // trunc == floor on [0,15]
 }
 
+// One word (8 codes) on the fast path. Preconditions (checked per lane by the caller): z is an
+// integer with |z| <= 240, so q - z is exact in bf16; 2^-40 <= s <= 2^40; r = RN(1/s).
+// m[] holds the noise: in Philox mode the 24-bit integer draw as a float (u = m * 2^-24 is exact,
+// so fmaf(m, 2^-24, a) == a + u with a single rounding, as the definition asks), else u itself.
 template <bool kPhilox>
-__device__ __forceinline__ unsigned requant_word(const WordIn &in, float lr, const float *u8,
-                                                 unsigned c0a, unsigned c1a, unsigned c0b, unsigned c1b,
-                                                 unsigned k0, unsigned k1) {
-    const float s = lq_bf16_bits_to_f32(in.s_bits);
-    const float z = lq_bf16_bits_to_f32(in.z_bits);
-
-    float g[8];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        g[2 * i] = lq_bf16_lo(in.g[i]);
-        g[2 * i + 1] = lq_bf16_hi(in.g[i]);
-    }
-
-    // Noise. Philox mode keeps the 24-bit integer draw as a float m; u = m * 2^-24 is exact,
-    // so fmaf(m, 2^-24, a) == a + u with a single rounding, as the definition asks.
-    float m[8];
-    if (kPhilox) {
-        lq_u4 ra = lq_philox4x32_10(c0a, c1a, 0u, 0u, k0, k1);
-        lq_u4 rb = lq_philox4x32_10(c0b, c1b, 0u, 0u, k0, k1);
-        m[0] = (float)(ra.x >> 8); m[1] = (float)(ra.y >> 8); m[2] = (float)(ra.z >> 8); m[3] = (float)(ra.w >> 8);
-        m[4] = (float)(rb.x >> 8); m[5] = (float)(rb.y >> 8); m[6] = (float)(rb.z >> 8); m[7] = (float)(rb.w >> 8);
-    } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) m[j] = u8[j];
-    }
-
-    // Codes as floats: low nibbles are the odd elements, high nibbles the even ones.
-    const unsigned lo4 = in.codes & 0x0F0F0F0Fu;
-    const unsigned hi4 = (in.codes >> 4) & 0x0F0F0F0Fu;
+__device__ __forceinline__ unsigned requant_word_fast(unsigned codes, const unsigned gp[4], float s, float z, float r,
+                                                      float lr, const float m[8]) {
+    const unsigned lo4 = codes & 0x0F0F0F0Fu;         // odd elements
+    const unsigned hi4 = (codes >> 4) & 0x0F0F0F0Fu;  // even elements
     float qf[8];
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
         qf[2 * b] = (float)((hi4 >> (8 * b)) & 0xFFu);
         qf[2 * b + 1] = (float)((lo4 >> (8 * b)) & 0xFFu);
     }
-
-    // Fast path preconditions: q - z exact in bf16 (integer zero of small magnitude) and a
-    // scale whose reciprocal, products and residuals stay far from overflow/underflow.
-    const float az = fabsf(z), as = fabsf(s);
-    bool fast = (z == floorf(z)) && (az <= 240.0f) && (as >= 0x1p-40f) && (as <= 0x1p40f);
-
     unsigned out = 0;
-    float t[8];
-    if (fast) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            float p = (qf[j] - z) * s;  // exact difference, one fp32 rounding (exact: <= 16 significant bits)
-            t[j] = p;
-        }
-        // bf16 rounding of the dequantised weight, two elements per v_cvt_pk_bf16_f32.
+    for (int i = 0; i < 4; ++i) {
+        // (q - z) * s: exact difference, exact product (<= 16 significant bits); bf16 rounding of the
+        // dequantised weight, two elements per v_cvt_pk_bf16_f32
+        const unsigned pk = lq_pack_bf16((qf[2 * i] - z) * s, (qf[2 * i + 1] - z) * s);
+        float t[2] = {fmaf(-lr, lq_bf16_lo(gp[i]), lq_bf16_lo(pk)), fmaf(-lr, lq_bf16_hi(gp[i]), lq_bf16_hi(pk))};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            unsigned pk = lq_pack_bf16(t[2 * i], t[2 * i + 1]);
-            t[2 * i] = fmaf(-lr, g[2 * i], lq_bf16_lo(pk));
-            t[2 * i + 1] = fmaf(-lr, g[2 * i + 1], lq_bf16_hi(pk));
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) fast = fast && (fabsf(t[j]) < 0x1p60f);
-    }
-    if (fast) {
-        // Correctly rounded t/s from the correctly rounded reciprocal (Markstein): q0 = t*r,
-        // e = t - q0*s (exact residual), q = q0 + e*r.
-        const float r = 1.0f / s;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            float q0 = t[j] * r;
-            float e = fmaf(-q0, s, t[j]);
+        for (int h = 0; h < 2; ++h) {
+            const int j = 2 * i + h;
+            // |t| >= 2^60 already saturates the code (|t/s| >= 2^20), so clamping t changes nothing but
+            // keeps t*r finite; a NaN t becomes -2^60 and ends as code 0, as the definition asks.
+            const float tc = __builtin_amdgcn_fmed3f(t[h], -0x1p60f, 0x1p60f);
+            // correctly rounded tc/s from the correctly rounded reciprocal (Markstein):
+            // q0 = t*r, e = t - q0*s (exact residual), q = q0 + e*r
+            const float q0 = tc * r;
+            const float e = fmaf(-q0, s, tc);
             float v = fmaf(e, r, q0);
             v = v + z;
             v = kPhilox ? fmaf(m[j], 0x1p-24f, v) : (v + m[j]);
-            float c = __builtin_amdgcn_fmed3f(v, 0.0f, 15.0f);
+            const float c = __builtin_amdgcn_fmed3f(v, 0.0f, 15.0f);
             out |= ((unsigned)c) << (4 * (j ^ 1));
-        }
-    } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            float u = kPhilox ? (m[j] * 0x1p-24f) : m[j];
-            out |= requant_elem_exact((unsigned)qf[j], s, z, g[j], lr, u) << (4 * (j ^ 1));
         }
     }
     return out;
 }
 
 template <bool kPhilox>
-__global__ __launch_bounds__(kThreads) void requant_kernel(const unsigned *__restrict__ codes_in,
-                                                           unsigned *__restrict__ codes_out,
+__device__ __forceinline__ unsigned requant_word_exact(unsigned codes, const unsigned gp[4], float s, float z, float lr,
+                                                       const float m[8]) {
+    unsigned out = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float g = (j & 1) ? lq_bf16_hi(gp[j >> 1]) : lq_bf16_lo(gp[j >> 1]);
+        const float u = kPhilox ? (m[j] * 0x1p-24f) : m[j];
+        out |= requant_elem_exact(lq_code(codes, j), s, z, g, lr, u) << (4 * (j ^ 1));
+    }
+    return out;
+}
+
+// A thread owns 4 consecutive code words (16 bytes in, 16 bytes out, 64 bytes of gradient): they
+// share one scale, zero and reciprocal, and their 8 Philox blocks have consecutive counters.
+template <bool kPhilox>
+__global__ __launch_bounds__(kThreads) void requant_kernel(const u32x4_t *__restrict__ codes_in,
+                                                           u32x4_t *__restrict__ codes_out,
                                                            const unsigned short *__restrict__ scales,
                                                            const unsigned short *__restrict__ zeros,
-                                                           const u32x4_t *__restrict__ grad, const float *__restrict__ u,
-                                                           float lr, long long n_words, unsigned long long seed,
+                                                           const u32x4_t *__restrict__ grad, const f32x4_t *__restrict__ u,
+                                                           float lr, long long n_chunks, unsigned long long seed,
                                                            unsigned long long offset) {
-    const long long base = (long long)blockIdx.x * (kThreads * kWordsPerThread) + threadIdx.x;
-    WordIn in[kWordsPerThread];
+    const long long L = (long long)blockIdx.x * kThreads + threadIdx.x;
+    if (L >= n_chunks) return;
+    const u32x4_t codes = codes_in[L];
+    u32x4_t g[kWordsPerThread];
+#pragma unroll
+    for (int i = 0; i < kWordsPerThread; ++i) g[i] = grad[L * kWordsPerThread + i];
+    const float s = lq_bf16_bits_to_f32(scales[L >> 2]);
+    const float z = lq_bf16_bits_to_f32(zeros[L >> 2]);
+
+    // (a negative scale takes the exact path: the NaN handling of the clamp below assumes s > 0)
+    const bool fast = (z == floorf(z)) && (fabsf(z) <= 240.0f) && (s >= 0x1p-40f) && (s <= 0x1p40f);
+    const float r = 1.0f / s;  // correctly rounded (IEEE division)
+    const unsigned long long cbase = offset + 8ull * (unsigned long long)L;  // element i uses block i/4
+
+    u32x4_t out;
 #pragma unroll
     for (int i = 0; i < kWordsPerThread; ++i) {
-        const long long w = base + (long long)i * kThreads;
-        if (w < n_words) {
-            in[i].codes = codes_in[w];
-            in[i].g = grad[w];
-            in[i].s_bits = scales[w >> 4];
-            in[i].z_bits = zeros[w >> 4];
+        float m[8];
+        if (kPhilox) {
+            const unsigned long long ca = cbase + 2 * i, cb = ca + 1;
+            const lq_u4 ra = lq_philox4x32_10((unsigned)ca, (unsigned)(ca >> 32), 0u, 0u, (unsigned)seed, (unsigned)(seed >> 32));
+            const lq_u4 rb = lq_philox4x32_10((unsigned)cb, (unsigned)(cb >> 32), 0u, 0u, (unsigned)seed, (unsigned)(seed >> 32));
+            m[0] = (float)(ra.x >> 8); m[1] = (float)(ra.y >> 8); m[2] = (float)(ra.z >> 8); m[3] = (float)(ra.w >> 8);
+            m[4] = (float)(rb.x >> 8); m[5] = (float)(rb.y >> 8); m[6] = (float)(rb.z >> 8); m[7] = (float)(rb.w >> 8);
+        } else {
+            const f32x4_t ua = u[(L * kWordsPerThread + i) * 2], ub = u[(L * kWordsPerThread + i) * 2 + 1];
+            m[0] = ua[0]; m[1] = ua[1]; m[2] = ua[2]; m[3] = ua[3];
+            m[4] = ub[0]; m[5] = ub[1]; m[6] = ub[2]; m[7] = ub[3];
         }
+        const unsigned gp[4] = {g[i][0], g[i][1], g[i][2], g[i][3]};
+        out[i] = fast ? requant_word_fast<kPhilox>(codes[i], gp, s, z, r, lr, m)
+                      : requant_word_exact<kPhilox>(codes[i], gp, s, z, lr, m);
     }
-#pragma unroll
-    for (int i = 0; i < kWordsPerThread; ++i) {
-        const long long w = base + (long long)i * kThreads;
-        if (w < n_words) {
-            float u8[8];
-            unsigned c0a = 0, c1a = 0, c0b = 0, c1b = 0;
-            if (kPhilox) {
-                const unsigned long long ca = offset + 2ull * (unsigned long long)w;
-                const unsigned long long cb = ca + 1ull;
-                c0a = (unsigned)ca; c1a = (unsigned)(ca >> 32);
-                c0b = (unsigned)cb; c1b = (unsigned)(cb >> 32);
-            } else {
-                const f32x4_t *up = reinterpret_cast<const f32x4_t *>(u) + 2 * w;
-                f32x4_t ua = up[0], ub = up[1];
-                u8[0] = ua[0]; u8[1] = ua[1]; u8[2] = ua[2]; u8[3] = ua[3];
-                u8[4] = ub[0]; u8[5] = ub[1]; u8[6] = ub[2]; u8[7] = ub[3];
-            }
-            codes_out[w] = requant_word<kPhilox>(in[i], lr, u8, c0a, c1a, c0b, c1b, (unsigned)seed,
-                                                 (unsigned)(seed >> 32));
-        }
-    }
+    codes_out[L] = out;
 }
 
 __global__ __launch_bounds__(256) void philox_uniform_kernel(float *__restrict__ out, long long n,
@@ -186,23 +156,22 @@ extern "C" int lq_requant_sr(const void *codes_in, void *codes_out, const void *
     LQ_REQUIRE(group == LQ_GROUP, "lq_requant_sr: group must be %d, got %d", LQ_GROUP, group);
     LQ_REQUIRE(N > 0 && K > 0 && K % LQ_GROUP == 0, "lq_requant_sr: need N > 0 and K a positive multiple of %d (N=%lld K=%lld)",
                LQ_GROUP, (long long)N, (long long)K);
-    LQ_REQUIRE(lq_aligned(codes_in, 4) && lq_aligned(codes_out, 4) && lq_aligned(grad, 16) && lq_aligned(scales, 2) &&
+    LQ_REQUIRE(lq_aligned(codes_in, 16) && lq_aligned(codes_out, 16) && lq_aligned(grad, 16) && lq_aligned(scales, 2) &&
                    lq_aligned(zeros, 2) && (!u_or_null || lq_aligned(u_or_null, 16)),
-               "lq_requant_sr: misaligned buffer (codes 4 B, grad 16 B, u 16 B)");
-    const long long n_words = (long long)N * K / 8;
-    const long long per_block = kThreads * kWordsPerThread;
-    const long long blocks = (n_words + per_block - 1) / per_block;
+               "lq_requant_sr: misaligned buffer (codes, grad and u need 16-byte alignment)");
+    const long long n_chunks = (long long)N * K / (8 * kWordsPerThread);  // K % 128 == 0: no remainder
+    const long long blocks = (n_chunks + kThreads - 1) / kThreads;
     LQ_REQUIRE(blocks <= 0x7FFFFFFFll, "lq_requant_sr: tensor too large");
     hipStream_t st = (hipStream_t)stream;
     if (u_or_null) {
         hipLaunchKernelGGL(requant_kernel<false>, dim3((unsigned)blocks), dim3(kThreads), 0, st,
-                           (const unsigned *)codes_in, (unsigned *)codes_out, (const unsigned short *)scales,
-                           (const unsigned short *)zeros, (const u32x4_t *)grad, u_or_null, lr, n_words,
+                           (const u32x4_t *)codes_in, (u32x4_t *)codes_out, (const unsigned short *)scales,
+                           (const unsigned short *)zeros, (const u32x4_t *)grad, (const f32x4_t *)u_or_null, lr, n_chunks,
                            (unsigned long long)philox_seed, (unsigned long long)philox_offset);
     } else {
         hipLaunchKernelGGL(requant_kernel<true>, dim3((unsigned)blocks), dim3(kThreads), 0, st,
-                           (const unsigned *)codes_in, (unsigned *)codes_out, (const unsigned short *)scales,
-                           (const unsigned short *)zeros, (const u32x4_t *)grad, (const float *)nullptr, lr, n_words,
+                           (const u32x4_t *)codes_in, (u32x4_t *)codes_out, (const unsigned short *)scales,
+                           (const unsigned short *)zeros, (const u32x4_t *)grad, (const f32x4_t *)nullptr, lr, n_chunks,
                            (unsigned long long)philox_seed, (unsigned long long)philox_offset);
     }
     return lq_check_launch("lq_requant_sr");
