@@ -41,7 +41,7 @@ def synth_w4(N, K, seed, device):
     return codes.to(device), scales.to(device), zeros.to(device)
 
 
-def event_time(fn, iters, warm=2):
+def event_time(fn, iters, warm=30):
     """Average seconds per call of fn(), HIP events on the current (= launch) stream."""
     for _ in range(warm):
         fn()
@@ -92,21 +92,39 @@ class MLPBlock:
 
     def step(self):
         o = self.ops
+        # bf16 glue exactly as autograd runs it for  down(silu(gate(x)) * up(x))
         g = o.a16w4_forward(self.x, *self.gate, (FFN, HID))
         u = o.a16w4_forward(self.x, *self.up, (FFN, HID))
-        sg = torch.sigmoid(g.float())
-        act = (g.float() * sg)
-        h = (act.to(torch.bfloat16) * u)
+        act = torch.nn.functional.silu(g)
+        h = act * u
         y = o.a16w4_forward(h, *self.down, (HID, FFN))
         dh = o.a16w4_dx(self.dy, *self.down, (HID, FFN))
-        du = dh * act.to(torch.bfloat16)
-        dg = (dh.float() * u.float() * (sg * (1.0 + g.float() * (1.0 - sg)))).to(torch.bfloat16)
+        du = dh * act
+        dg = torch.ops.aten.silu_backward(dh * u, g)
         dx = o.a16w4_dx(dg, *self.gate, (FFN, HID))
         dx += o.a16w4_dx(du, *self.up, (FFN, HID))
         return y, dx
 
 
 MLP_FLOP = 6 * 2 * TOKENS * HID * FFN  # 1 108.1 GFLOP
+
+# HBM traffic per GEMM launch, from two counter runs of
+#   rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --profile-target gemm     (then WRITE_SIZE)
+# in KiB per dispatch as the counters read, and the reading of the same counters for the
+# 256 MiB calibration copy in the same runs (262 144 KiB fetched and written).
+PMC_GEMM_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
+    "fwd_gate_up": (122755.4, 44051.4), "fwd_down": (92921.5, 16384.0),
+    "dx_gate_up": (96642.8, 16384.0), "dx_down": (136759.2, 44044.9),
+}
+PMC_COPY_KIB = (131083.0, 262158.0)
+PMC_LAUNCHES = {"fwd_gate_up": 2, "fwd_down": 1, "dx_gate_up": 2, "dx_down": 1}  # per MLP step
+
+
+def gemm_traffic_bytes():
+    """Launch-weighted mean HBM bytes (read + written) per GEMM launch of the MLP step."""
+    fs, ws = 262144.0 / PMC_COPY_KIB[0], 262144.0 / PMC_COPY_KIB[1]
+    tot = sum(n * (PMC_GEMM_KIB[k][0] * fs + PMC_GEMM_KIB[k][1] * ws) for k, n in PMC_LAUNCHES.items())
+    return tot * 1024 / sum(PMC_LAUNCHES.values())
 
 
 def bench_requant(device):
@@ -159,6 +177,64 @@ def bench_a8w8(device):
     return out
 
 
+def bench_copy(device):
+    """Plain streaming copy (lq_calib_copy) over buffers larger than the last-level cache: the
+    HBM rate this device sustains for read + write traffic, for comparison with the 8 TB/s peak."""
+    from latentq_llm_amd import _C
+    nbytes = 1 << 30
+    src = torch.empty(nbytes, dtype=torch.uint8, device=device).random_(0, 256)
+    dst = torch.empty_like(src)
+    st = torch.cuda.current_stream().cuda_stream
+    sec = event_time(lambda: _C.call("lq_calib_copy", src.data_ptr(), dst.data_ptr(), nbytes, st), 10, warm=3)
+    return {"bytes_each_way": nbytes, "us": sec * 1e6, "GB/s": 2 * nbytes / sec / 1e9}
+
+
+def profile_target(device, which, launches=5):
+    """A short, fixed sequence of launches for a profiler run (kernel trace or counters): the
+    calibration copy first, then the kernels of the named family, `launches` times each."""
+    from latentq_llm_amd import _C, ops as o
+    st = torch.cuda.current_stream().cuda_stream
+    nbytes = 256 << 20
+    src = torch.empty(nbytes, dtype=torch.uint8, device=device).random_(0, 256)
+    dst = torch.empty_like(src)
+    for _ in range(launches):
+        _C.call("lq_calib_copy", src.data_ptr(), dst.data_ptr(), nbytes, st)
+    del src, dst
+    if which == "gemm":
+        blk = MLPBlock(device)
+        h = torch.randn(TOKENS, FFN, device=device).to(torch.bfloat16)
+        for _ in range(launches):
+            o.a16w4_forward(blk.x, *blk.gate, (FFN, HID))
+        for _ in range(launches):
+            o.a16w4_forward(h, *blk.down, (HID, FFN))
+        for _ in range(launches):
+            o.a16w4_dx(h, *blk.gate, (FFN, HID))
+        for _ in range(launches):
+            o.a16w4_dx(blk.dy, *blk.down, (HID, FFN))
+    elif which == "requant":
+        N, K = 8192, 2048
+        for i in range(launches):
+            p, s, z = synth_w4(N, K, 10 + i, device)
+            g = (torch.randn(N, K, device=device) * 1e-3).to(torch.bfloat16)
+            o.requant_sr(p, s, z, g, 1e-4, (N, K), seed=7, offset=i)
+    elif which == "gemv":
+        for (N, K) in [(4096, 4096), (11008, 4096), (4096, 11008)]:
+            for M in (1, 4, 16):
+                x = torch.randn(M, K, device=device).to(torch.bfloat16)
+                for i in range(launches):
+                    w = synth_w4(N, K, 20 + i, device)
+                    o.a16w4_forward(x, *w, (N, K))
+    elif which == "a8w8":
+        for (N, K) in [(2048, 2048), (8192, 2048), (2048, 8192)]:
+            x8 = torch.randint(-127, 128, (TOKENS, K), device=device, dtype=torch.int8)
+            w8 = torch.randint(-127, 128, (N, K), device=device, dtype=torch.int8)
+            sx = (torch.randn(TOKENS, device=device) * 0.05).abs()
+            sw = (torch.randn(N, device=device) * 0.01).abs()
+            for _ in range(launches):
+                o.a8w8_forward(x8, w8, sx, sw)
+    torch.cuda.synchronize()
+
+
 def cpu_baseline():
     """The reference's CPU path (nibble unpack -> bf16 group dequant -> bf16 torch.mm), restated in
     oracle/torch_ref.py, on the host cores: the whole MLP step at 2048 tokens, fwd + dX."""
@@ -175,9 +251,8 @@ def cpu_baseline():
     def step():
         y, (gg, uu, h) = tr.llama_mlp_forward(x, gate, up, down)
         dh = dy.mm(tr.dequant_4bit_g(*down))
-        sg = torch.sigmoid(gg.float())
-        du = dh * (gg.float() * sg).to(torch.bfloat16)
-        dg = (dh.float() * uu.float() * (sg * (1.0 + gg.float() * (1.0 - sg)))).to(torch.bfloat16)
+        du = dh * torch.nn.functional.silu(gg)
+        dg = torch.ops.aten.silu_backward(dh * uu, gg)
         dx = dg.mm(tr.dequant_4bit_g(*gate)) + du.mm(tr.dequant_4bit_g(*up))
         return y, dx
 
@@ -207,10 +282,12 @@ def _cpu_model():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-mlp", action="store_true", help="skip the side measurements (requant, GEMV, A8W8)")
+    ap.add_argument("--profile-target", choices=["gemm", "requant", "gemv", "a8w8"],
+                    help="run only a short fixed launch sequence of one kernel family (for rocprofv3), print nothing")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no sharding, no collectives); use --gpus 1")
@@ -220,6 +297,10 @@ def main():
     _C.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.profile_target:
+        profile_target(dev, args.profile_target)
+        return
 
     blk = MLPBlock(dev)
     for _ in range(args.warmup):
@@ -242,7 +323,7 @@ def main():
         ("dx_gate_up", lambda: o.a16w4_dx(h, *blk.gate, (FFN, HID)), 2 * TOKENS * HID * FFN),
         ("dx_down", lambda: o.a16w4_dx(blk.dy, *blk.down, (HID, FFN)), 2 * TOKENS * HID * FFN),
     ]:
-        sec = event_time(fn, 20)
+        sec = event_time(fn, 50)
         kern[name] = {"us": sec * 1e6, "TFLOP/s": fl / sec / 1e12, "frac_mfma_bf16": fl / sec / PEAK_BF16}
     # weighted by launches per step: 2 fwd gate/up, 1 fwd down, 2 dx gate/up, 1 dx down
     tot = 2 * kern["fwd_gate_up"]["us"] + kern["fwd_down"]["us"] + 2 * kern["dx_gate_up"]["us"] + kern["dx_down"]["us"]
@@ -250,7 +331,8 @@ def main():
     achieved = 2 * TOKENS * HID * FFN / (avg_us * 1e-6) / 1e12
     roofline = {"bound": "mfma", "kernel": "gemm_kernel (A16W4 dequant-GEMM, fwd and dX instantiations)",
                 "achieved": achieved, "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": achieved * 1e12 / PEAK_BF16,
-                "avg_launch_us": avg_us, "flop_per_launch": 2 * TOKENS * HID * FFN, "traffic": None}
+                "avg_launch_us": avg_us, "flop_per_launch": 2 * TOKENS * HID * FFN, "traffic": gemm_traffic_bytes(),
+                "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated on a copy)"}
 
     line = {
         "metric": "A16W4 GEMM TFLOP/s (7B MLP, 2048 tok)", "value": value, "unit": "TFLOP/s",
@@ -268,6 +350,7 @@ def main():
         line["requant"] = bench_requant(dev)
         line["gemv"] = bench_gemv(dev)
         line["a8w8"] = bench_a8w8(dev)
+        line["hbm_copy"] = bench_copy(dev)
     line["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
     print(json.dumps(line))
 

@@ -152,6 +152,14 @@ int lq_repack_gptq_to_native(const int32_t *qweight_gptq, void *codes_native, in
 int lq_repack_native_to_gptq(const void *codes_native, int32_t *qweight_gptq, int64_t N, int64_t K,
                              void *stream);
 
+/* ---------------------------------------------------------------------------
+ * Measurement aid, no counterpart in the reference: a plain streaming copy of
+ * nbytes (a multiple of 16, both pointers 16-byte aligned) from src to dst.
+ * Its known traffic (nbytes read + nbytes written) calibrates the HBM byte
+ * counters of a profiler run and gives the copy bandwidth this device sustains.
+ * ------------------------------------------------------------------------- */
+int lq_calib_copy(const void *src, void *dst, int64_t nbytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -29,6 +29,7 @@ SIGNATURES = {
     "lq_residual_dequant": [_vp, _vp, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],
     "lq_repack_gptq_to_native": [_vp, _vp, _i64, _i64, _vp],
     "lq_repack_native_to_gptq": [_vp, _vp, _i64, _i64, _vp],
+    "lq_calib_copy": [_vp, _vp, _i64, _vp],
 }
 
 _lib = None

@@ -138,3 +138,25 @@ extern "C" int lq_repack_native_to_gptq(const void *codes_native, int32_t *qweig
                                         void *stream) {
     return repack_common(codes_native, qweight_gptq, N, K, stream, false, "lq_repack_native_to_gptq");
 }
+
+// ---- calibration copy -------------------------------------------------------
+// Grid-stride 16-byte copy: each workgroup streams contiguous 4 KiB pieces.
+__global__ __launch_bounds__(256) void calib_copy_kernel(const u32x4_t *__restrict__ src, u32x4_t *__restrict__ dst,
+                                                        long long n16) {
+    const long long stride = (long long)gridDim.x * 256;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+extern "C" int lq_calib_copy(const void *src, void *dst, int64_t nbytes, void *stream) {
+    LQ_REQUIRE(src && dst, "lq_calib_copy: null pointer argument");
+    LQ_REQUIRE(nbytes >= 0 && nbytes % 16 == 0, "lq_calib_copy: nbytes must be a non-negative multiple of 16");
+    LQ_REQUIRE(lq_aligned(src, 16) && lq_aligned(dst, 16), "lq_calib_copy: buffers must be 16-byte aligned");
+    if (nbytes == 0) return LQ_OK;
+    const long long n16 = nbytes / 16;
+    long long blocks = (n16 + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    hipLaunchKernelGGL(calib_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const u32x4_t *)src, (u32x4_t *)dst, n16);
+    return lq_check_launch("lq_calib_copy");
+}

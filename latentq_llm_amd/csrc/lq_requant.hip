@@ -36,6 +36,7 @@ __device__ __forceinline__ unsigned requant_elem_exact(unsigned q, float s, floa
 template <bool kPhilox>
 __device__ __forceinline__ unsigned requant_word_fast(unsigned codes, const unsigned gp[4], float s, float z, float r,
                                                       float lr, const float m[8]) {
+    const float nzs = -(z * s);
     const unsigned lo4 = codes & 0x0F0F0F0Fu;         // odd elements
     const unsigned hi4 = (codes >> 4) & 0x0F0F0F0Fu;  // even elements
     float qf[8];
@@ -47,9 +48,10 @@ __device__ __forceinline__ unsigned requant_word_fast(unsigned codes, const unsi
     unsigned out = 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        // (q - z) * s: exact difference, exact product (<= 16 significant bits); bf16 rounding of the
-        // dequantised weight, two elements per v_cvt_pk_bf16_f32
-        const unsigned pk = lq_pack_bf16((qf[2 * i] - z) * s, (qf[2 * i + 1] - z) * s);
+        // (q - z) * s as fma(q, s, -(z*s)): z*s and q*s are exact (8-bit significands), the sum has at
+        // most 16 significant bits, so the fma returns (q - z) * s exactly; then the bf16 rounding of
+        // the dequantised weight, two elements per v_cvt_pk_bf16_f32
+        const unsigned pk = lq_pack_bf16(fmaf(qf[2 * i], s, nzs), fmaf(qf[2 * i + 1], s, nzs));
         float t[2] = {fmaf(-lr, lq_bf16_lo(gp[i]), lq_bf16_lo(pk)), fmaf(-lr, lq_bf16_hi(gp[i]), lq_bf16_hi(pk))};
 #pragma unroll
         for (int h = 0; h < 2; ++h) {

@@ -1,0 +1,96 @@
+"""Exact models of the hot path's arithmetic, independent of the C oracle and of the kernels.
+
+Everything here is integer / rational arithmetic (fractions.Fraction) with an explicit
+round-to-nearest-even, plus a pure-Python Philox4x32-10 transcribed from the published
+Random123 description (multipliers 0xD2511F53 / 0xCD9E8D57, Weyl constants 0x9E3779B9 /
+0xBB67AE85). It is the source of the committed vectors in this directory and is only fit
+for small cases (it runs at a few thousand elements per second).
+
+Formulas modelled:
+  dequant  w = bf16(bf16(q - z) * s)                       (utils/quant.py:66-72)
+  requant  t = fma(-lr, g, w); v = t / s; v = v + z; v = v + u; code' = clamp(floor(v), 0, 15)
+           every operation rounded to fp32, NaN-free inputs only
+  uniform  u_i = (word[i & 3] of Philox(counter = offset + i // 4, key = seed) >> 8) * 2^-24
+"""
+import struct
+from fractions import Fraction
+
+
+def rn(x: Fraction, mant_bits: int, emin: int = -126) -> Fraction:
+    """Round an exact rational to a binary float with `mant_bits` significand bits (incl. the
+    hidden one), round-to-nearest-even, gradual underflow below 2^emin."""
+    if x == 0:
+        return Fraction(0)
+    sign = -1 if x < 0 else 1
+    a = abs(x)
+    e = a.numerator.bit_length() - a.denominator.bit_length()
+    if Fraction(2) ** e > a:
+        e -= 1
+    if Fraction(2) ** (e + 1) <= a:
+        e += 1
+    e = max(e, emin)
+    quantum = Fraction(2) ** (e - (mant_bits - 1))
+    n = a / quantum
+    fl = n.numerator // n.denominator
+    rem = n - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        fl += 1
+    return sign * fl * quantum
+
+
+def f32(x):
+    return rn(x, 24)
+
+
+def bf16(x):
+    return rn(x, 8)
+
+
+def frac_of_bf16_bits(b: int) -> Fraction:
+    return Fraction(struct.unpack("<f", struct.pack("<I", (b & 0xFFFF) << 16))[0])
+
+
+def frac_of_f32_bits(b: int) -> Fraction:
+    return Fraction(struct.unpack("<f", struct.pack("<I", b & 0xFFFFFFFF))[0])
+
+
+def bf16_bits_of_frac(x: Fraction) -> int:
+    """Bits of a rational that is exactly representable in bf16."""
+    b = struct.unpack("<I", struct.pack("<f", float(x)))[0]
+    assert b & 0xFFFF == 0
+    return b >> 16
+
+
+def dequant_model(q: int, zb: int, sb: int) -> Fraction:
+    z, s = frac_of_bf16_bits(zb), frac_of_bf16_bits(sb)
+    return bf16(f32(bf16(f32(q - z)) * s))
+
+
+def requant_model(q: int, zb: int, sb: int, gb: int, lr_bits: int, u: Fraction) -> int:
+    z, s, g = frac_of_bf16_bits(zb), frac_of_bf16_bits(sb), frac_of_bf16_bits(gb)
+    w = dequant_model(q, zb, sb)
+    t = f32(w - frac_of_f32_bits(lr_bits) * g)  # one rounding: fused multiply-add
+    v = f32(t / s)
+    v = f32(v + z)
+    v = f32(v + u)
+    fl = v.numerator // v.denominator
+    return min(max(fl, 0), 15)
+
+
+def philox4x32_10(ctr, key):
+    c0, c1, c2, c3 = ctr
+    k0, k1 = key
+    for _ in range(10):
+        p0 = 0xD2511F53 * c0
+        p1 = 0xCD9E8D57 * c2
+        c0, c1, c2, c3 = ((p1 >> 32) ^ c1 ^ k0) & 0xFFFFFFFF, p1 & 0xFFFFFFFF, ((p0 >> 32) ^ c3 ^ k1) & 0xFFFFFFFF, p0 & 0xFFFFFFFF
+        k0 = (k0 + 0x9E3779B9) & 0xFFFFFFFF
+        k1 = (k1 + 0xBB67AE85) & 0xFFFFFFFF
+    return [c0, c1, c2, c3]
+
+
+def uniform_draw(i: int, seed: int, offset: int) -> int:
+    """24-bit integer m of element i; u = m * 2^-24."""
+    c = (offset + i // 4) & 0xFFFFFFFFFFFFFFFF
+    w = philox4x32_10([c & 0xFFFFFFFF, c >> 32, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
+    return w[i & 3] >> 8

@@ -1,0 +1,103 @@
+"""The committed exact-arithmetic vectors (tests/golden/hot_path_vectors.json, written by
+tests/golden/make_golden.py from rational arithmetic and the published Philox known answers)
+against the CPU oracle (no GPU needed) and against the HIP kernels (gpu)."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from tests.util import bits, from_bits
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+@pytest.fixture(scope="module")
+def vec():
+    with open(os.path.join(HERE, "golden", "hot_path_vectors.json")) as f:
+        return json.load(f)
+
+
+@pytest.fixture(scope="module")
+def co():
+    from oracle import c_oracle
+    return c_oracle
+
+
+def _bf16_tensor(bit_list, shape):
+    return from_bits(np.array(bit_list, np.uint16).reshape(shape))
+
+
+def _pack(codes):
+    c = np.array(codes, np.uint8).reshape(-1, 2)
+    return ((c[:, 0] << 4) | c[:, 1]).astype(np.uint8)
+
+
+def _lr(case):
+    return float(np.array([case["lr_bits"]], np.uint32).view(np.float32)[0])
+
+
+# ----------------------------------------------------------------- oracle (CPU) --
+def test_oracle_philox_and_uniform(vec, co):
+    for k in vec["philox_kat"]:
+        assert list(co.philox4x32_10(k["ctr"], k["key"])) == k["out"]
+    for s in vec["uniform"]:
+        u = co.philox_uniform(len(s["m24"]), s["seed"], s["offset"])
+        assert np.array_equal(u, (np.array(s["m24"], np.float64) * 2.0 ** -24).astype(np.float32))
+
+
+def test_oracle_dequant(vec, co):
+    for q, zb, sb, wb in vec["dequant"]:
+        got = co.dequant(_pack([q] * 128), np.array([sb], np.uint16), np.array([zb], np.uint16), 1, 128)
+        assert int(got.reshape(-1)[0]) == wb and int(got.reshape(-1)[127]) == wb
+
+
+def test_oracle_requant(vec, co):
+    for c in vec["requant"]:
+        N, K = c["N"], c["K"]
+        args = (_pack(c["codes"]), np.array(c["scale_bits"], np.uint16), np.array(c["zero_bits"], np.uint16),
+                np.array(c["grad_bits"], np.uint16), _lr(c), N, K)
+        want = _pack(c["new_codes"])
+        u = (np.array(c["m24"], np.float64) * 2.0 ** -24).astype(np.float32)
+        assert np.array_equal(co.requant(*args, u=u), want)
+        assert np.array_equal(co.requant(*args, seed=c["seed"], offset=c["offset"]), want)
+
+
+# ------------------------------------------------------------------ HIP kernels --
+@pytest.mark.gpu
+def test_hip_uniform(vec):
+    from latentq_llm_amd import ops
+    for s in vec["uniform"]:
+        u = ops.philox_uniform(len(s["m24"]), s["seed"], s["offset"]).cpu().numpy()
+        assert np.array_equal(u, (np.array(s["m24"], np.float64) * 2.0 ** -24).astype(np.float32))
+
+
+@pytest.mark.gpu
+def test_hip_dequant(vec):
+    from latentq_llm_amd import ops
+    cases = vec["dequant"]
+    n = len(cases)
+    codes = torch.from_numpy(np.concatenate([_pack([q] * 128) for q, _, _, _ in cases]).view(np.int8)).cuda()
+    scales = _bf16_tensor([c[2] for c in cases], (n, 1)).cuda()
+    zeros = _bf16_tensor([c[1] for c in cases], (n, 1)).cuda()
+    w = bits(ops.a16w4_dequant(codes, scales, zeros, (n, 128)).cpu())
+    assert np.array_equal(w[:, 0], np.array([c[3] for c in cases], np.uint16))
+    assert np.array_equal(w[:, 127], w[:, 0])
+
+
+@pytest.mark.gpu
+def test_hip_requant(vec):
+    from latentq_llm_amd import ops
+    for c in vec["requant"]:
+        N, K = c["N"], c["K"]
+        codes = torch.from_numpy(_pack(c["codes"]).view(np.int8)).cuda()
+        scales = _bf16_tensor(c["scale_bits"], (N, 1)).cuda()
+        zeros = _bf16_tensor(c["zero_bits"], (N, 1)).cuda()
+        grad = _bf16_tensor(c["grad_bits"], (N, K)).cuda()
+        want = _pack(c["new_codes"])
+        u = torch.from_numpy((np.array(c["m24"], np.float64) * 2.0 ** -24).astype(np.float32)).reshape(N, K).cuda()
+        got_u = ops.requant_sr(codes, scales, zeros, grad, _lr(c), (N, K), u=u)
+        got_p = ops.requant_sr(codes, scales, zeros, grad, _lr(c), (N, K), seed=c["seed"], offset=c["offset"])
+        assert np.array_equal(got_u.cpu().numpy().view(np.uint8), want)
+        assert np.array_equal(got_p.cpu().numpy().view(np.uint8), want)

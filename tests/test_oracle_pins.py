@@ -32,35 +32,8 @@ from oracle import torch_ref as tr
 from tests.util import bits, from_bits, make_w4, pack_codes, randn_bf16, rel_l2
 
 
-# ------------------------------------------------------------ exact rounding --
-def rn(x: Fraction, mant_bits: int, emin: int = -126) -> Fraction:
-    """Round an exact rational to a binary float with `mant_bits` significand bits (incl. the
-    hidden one), round-to-nearest-even, gradual underflow below 2^emin."""
-    if x == 0:
-        return Fraction(0)
-    sign = -1 if x < 0 else 1
-    a = abs(x)
-    e = a.numerator.bit_length() - a.denominator.bit_length()
-    if Fraction(2) ** e > a:
-        e -= 1
-    if Fraction(2) ** (e + 1) <= a:
-        e += 1
-    e = max(e, emin)
-    quantum = Fraction(2) ** (e - (mant_bits - 1))
-    n = a / quantum
-    fl = n.numerator // n.denominator
-    rem = n - fl
-    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
-        fl += 1
-    return sign * fl * quantum
-
-
-def f32(x):
-    return rn(x, 24)
-
-
-def bf16(x):
-    return rn(x, 8)
+# exact rounding helpers and models: shared with the generator of the committed vectors
+from tests.golden.exact_model import bf16, f32  # noqa: E402
 
 
 def frac_of_bits(b: int) -> Fraction:
