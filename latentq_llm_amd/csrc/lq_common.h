@@ -47,6 +47,23 @@ __device__ __forceinline__ unsigned short lq_f32_to_bf16_bits(float a) {
 // consecutive k: code j sits at bit 4*(j^1)  (even index = high nibble of its byte).
 __device__ __forceinline__ unsigned lq_code(unsigned word, int j) { return (word >> (4 * (j ^ 1))) & 0xFu; }
 
+// byte N of a dword as float, one instruction each (v_cvt_f32_ubyteN)
+__device__ __forceinline__ float lq_ubyte0(unsigned x) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(x)); return r; }
+__device__ __forceinline__ float lq_ubyte1(unsigned x) { float r; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(x)); return r; }
+__device__ __forceinline__ float lq_ubyte2(unsigned x) { float r; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(x)); return r; }
+__device__ __forceinline__ float lq_ubyte3(unsigned x) { float r; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(x)); return r; }
+
+// 8 codes of a native word -> 8 floats in k order, f = (q - z) * s rounded once:
+// nzs = -(z*s) is exact for bf16 z and s, and fma(q, s, nzs) rounds the exact (q - z) * s.
+__device__ __forceinline__ void lq_dequant_word_f32(unsigned word, float s, float nzs, float f[8]) {
+    const unsigned lo4 = word & 0x0F0F0F0Fu;         // odd k
+    const unsigned hi4 = (word >> 4) & 0x0F0F0F0Fu;  // even k
+    f[0] = fmaf(lq_ubyte0(hi4), s, nzs); f[1] = fmaf(lq_ubyte0(lo4), s, nzs);
+    f[2] = fmaf(lq_ubyte1(hi4), s, nzs); f[3] = fmaf(lq_ubyte1(lo4), s, nzs);
+    f[4] = fmaf(lq_ubyte2(hi4), s, nzs); f[5] = fmaf(lq_ubyte2(lo4), s, nzs);
+    f[6] = fmaf(lq_ubyte3(hi4), s, nzs); f[7] = fmaf(lq_ubyte3(lo4), s, nzs);
+}
+
 // ---- Philox4x32-10 ---------------------------------------------------------
 #define LQ_PHILOX_M0 0xD2511F53u
 #define LQ_PHILOX_M1 0xCD9E8D57u

@@ -309,13 +309,19 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
         a_off[i] = (unsigned)((gr - m0) * lda + ch * 16);
     }
     const unsigned char *a_base = (const unsigned char *)p.a + m0 * lda;
-    // LDS-direct load: lane l of the wave writes 16 bytes at (wave-uniform base) + 16*l.
+    // LDS-direct load: lane l of the wave writes 16 bytes at (wave-uniform base) + 16*l. Written as
+    // inline assembly (M0 = LDS base, one wait state, then the load with a scalar base and a 32-bit
+    // lane offset) so that the compiler's wait-count insertion does not see an LDS write it cannot
+    // tell apart from the fragment reads and park a vmcnt(0) in front of them: the explicit
+    // s_waitcnt before each barrier is the only ordering these loads need.
     auto issue_a = [&](int kt, unsigned char *la) {
         const unsigned char *src = a_base + (long long)kt * ROWB;
 #pragma unroll
-        for (int i = 0; i < APT; ++i)
-            __builtin_amdgcn_global_load_lds((gbl_void *)(src + a_off[i]), (lds_void *)(la + (i * NT + wave * 64) * 16), 16,
-                                             0, 0);
+        for (int i = 0; i < APT; ++i) {
+            const unsigned lds_addr = (unsigned)reinterpret_cast<size_t>((lds_void *)(la + (i * NT + wave * 64) * 16));
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         :: "s"(lds_addr), "v"(a_off[i]), "s"(src) : "memory");
+        }
     };
 
     using acc_t = typename std::conditional<MODE == MODE_I8, i32x16_t, f32x16_t>::type;
@@ -360,17 +366,18 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             }
     };
 
-    // Tile kt: A in buffer kt%3, B in buffer kt%2. First put the A loads of tile kt+2 in flight
-    // (into the buffer tile kt-1 just left), then 4 MFMA steps with double-buffered fragments,
+    // Tile kt: A in buffer kt%3, B in buffer kt%2. Start the first fragment reads, put the A loads
+    // of tile kt+2 in flight behind them (into the buffer tile kt-1 just left), then 4 MFMA steps
+    // with double-buffered fragments,
     // then wait until this wave's part of tile kt+1 has landed (all but the newest APT loads)
     // and its fragment reads have returned, and meet the other waves.
     auto tile_step = [&](int kt, auto ai, auto bi) {
         constexpr int AI = decltype(ai)::value, BI = decltype(bi)::value;
-        issue_a(kt + 2 < nk ? kt + 2 : nk - 1, abuf(ic<(AI + 2) % 3>()));
         const unsigned char *la = abuf(ic<AI>()), *lb = bbuf(ic<BI>());
         u32x4_t af[2][FM], bf[2][FN];
         read_frags(la, lb, 0, af[0], bf[0]);
         read_frags(la, lb, 1, af[1], bf[1]);
+        issue_a(kt + 2 < nk ? kt + 2 : nk - 1, abuf(ic<(AI + 2) % 3>()));
         mfma_step(af[0], bf[0]);
         read_frags(la, lb, 2, af[0], bf[0]);
         mfma_step(af[1], bf[1]);
@@ -453,6 +460,24 @@ int launch_gemm(GemmParams p, hipStream_t st, const char *who) {
 
 }  // namespace
 
+// number of compute units of the current device (cached per device)
+static int lq_device_cu_count() {
+    static int cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+// weights-direct forward GEMM (lq_gemm_fwd.hip)
+long long lq_gemm_fwd_direct_workgroups(int M, int N);
+int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
+                              void *y, int M, int N, int K, hipStream_t st);
+
 // GEMV path (lq_gemv.hip)
 int lq_gemv_a16w4_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
                          void *y, int M, int N, int K, hipStream_t st);
@@ -479,6 +504,11 @@ extern "C" int lq_a16w4_fwd(const void *x, const void *codes, const void *scales
     LQ_REQUIRE(N % 16 == 0, "lq_a16w4_fwd: N=%lld must be a multiple of 16", (long long)N);
     if (M <= 16)
         return lq_gemv_a16w4_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
+    // Two forward kernels. The weights-direct one (128 x 256 tiles, two workgroups per CU) wins when
+    // its tiles can occupy every CU twice; otherwise the staged 256 x 128 kernel, whose producer
+    // waves hide more latency with a single workgroup per CU, is faster.
+    if (lq_gemm_fwd_direct_workgroups((int)M, (int)N) >= 2ll * lq_device_cu_count())
+        return lq_gemm_fwd_direct_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
     GemmParams p = {};
     p.a = x; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.bias = (const unsigned short *)bias_or_null; p.c = y;

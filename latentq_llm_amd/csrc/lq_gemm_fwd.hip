@@ -1,0 +1,302 @@
+// A16W4 forward GEMM for gfx950, M > 16:  Y[M,N] = X[M,K] . deq(W)[N,K]^T (+ bias), bf16 MFMA.
+//
+// The weights never pass through LDS. An MFMA B-side lane needs 8 consecutive k of one weight
+// row, and 8 consecutive k of a row are exactly one 32-bit word of packed codes: every lane
+// loads the 16 bytes (32 codes) of its own weight row straight from global memory, dequantises
+// them in registers and feeds the matrix core. LDS only holds the activation tile, written by
+// LDS-direct loads (no registers, no vector-ALU work) and read as fragments.
+//
+// Per CU this halves the LDS traffic of a tile scheme that stages both operands (LDS write
+// bandwidth on this chip is ~1/3 of its read bandwidth, and the LDS pipe, not the matrix core,
+// is what such a scheme saturates), and it removes the producer/consumer hand-off for B.
+//
+// Workgroup: 128 rows (m) x 256 columns (n), 4 waves side by side along n; a wave owns a
+// 128 x 64 block (4 x 2 MFMA 32x32x16 tiles, 128 accumulator registers). With <= 256 VGPRs and
+// 48 KB of LDS two workgroups share a CU, so one group's barrier and load latencies are covered
+// by the other's MFMAs.
+//
+// Reduction step = 64 k. Lane l of a wave: r = l % 32, h = l / 32.
+//   * B: for each of the wave's two 32-column tiles the lane loads 16 bytes of row n = tile
+//     base + r at k offset 64*step + 32*h. Word t (t = 0..3) holds k = 32h + 8t .. +7 and becomes
+//     the lane's operand of reduction slice t.
+//   * A: slice t therefore needs, for row m and half h, the 16 bytes at k = 32h + 8t: chunk
+//     4h + t of the 128-byte tile row. Chunk c of row m sits at position c ^ ((m >> 1) & 7),
+//     which makes the 16-lane fragment reads conflict-free; the swizzle costs nothing because an
+//     LDS-direct load lets each lane choose which global chunk lands in its (fixed) LDS slot.
+//   * D = Wfrag x Xfrag^T: D[i][j] has i = n, j = m, so a lane owns 4 consecutive n of one m
+//     and the epilogue stores 8-byte bf16 quads.
+//
+// Dequantisation is bf16(fma(q, s, -(z*s))): z*s and q*s are exact in fp32, so the fma rounds
+// the exact (q - z)*s once; for integer zeros this equals the reference's bf16(bf16(q-z)*s).
+//
+// Pipeline: A tiles are loaded two steps ahead into three LDS stages, codes one step ahead into
+// registers, scales/zeros once per 128-k group. One s_barrier per step, issued without a fence;
+// the LDS-direct loads are inline assembly with explicit s_waitcnt so that they stay in flight
+// across barriers and the compiler's wait insertion never sees them.
+#include "lq_common.h"
+
+#include <type_traits>
+
+namespace {
+
+struct FwdParams {
+    const unsigned char *x;   // bf16 [M, K]
+    const unsigned char *w;   // packed codes, K/2 bytes per row
+    const unsigned short *scales;
+    const unsigned short *zeros;
+    const unsigned short *bias;  // bf16 [N] or null
+    unsigned short *y;           // bf16 [M, N]
+    int M, N, K;
+    int tiles_m, tiles_n;
+};
+
+typedef __attribute__((address_space(3))) void lds_void;
+
+template <int I>
+using ic = std::integral_constant<int, I>;
+
+constexpr int BM = 128, BN = 256, KT = 64;
+constexpr int STAGE = BM * KT * 2;  // 16 KB per A stage
+
+__global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds_a0[STAGE];
+    __shared__ __attribute__((aligned(16))) unsigned char lds_a1[STAGE];
+    __shared__ __attribute__((aligned(16))) unsigned char lds_a2[STAGE];
+    auto abuf = [&](auto i) -> unsigned char * {
+        constexpr int I = decltype(i)::value;
+        return I == 0 ? lds_a0 : I == 1 ? lds_a1 : lds_a2;
+    };
+
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int r = lane & 31, h = lane >> 5;
+
+    // Workgroup ids are dealt round-robin over the 8 XCDs (id % 8): give each XCD a contiguous
+    // range of the tile sequence, ordered in bands of GN tile columns walked row by row, so the
+    // workgroups resident on one XCD share a few A row-blocks and B column-blocks in its L2.
+    const int nwg = p.tiles_m * p.tiles_n;
+    int id = blockIdx.x;
+    {
+        const int per = nwg / 8;
+        if (id < per * 8) id = (id % 8) * per + id / 8;
+    }
+    constexpr int GN = 8;
+    const int band = id / (p.tiles_m * GN);
+    const int within = id - band * (p.tiles_m * GN);
+    const int rest = p.tiles_n - band * GN;
+    const int bw = rest < GN ? rest : GN;
+    const int tile_m = within / bw, tile_n = band * GN + within % bw;
+    const int m0 = tile_m * BM, c0 = tile_n * BN;
+    const int nk = p.K / KT;
+    const long long lda = (long long)p.K * 2;
+
+    // ---- A staging: 1024 16-byte slots per stage; slot s = i*256 + thread -> row s/8, position s%8
+    unsigned a_off[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = i * 32 + (int)(threadIdx.x >> 3);
+        const int pos = threadIdx.x & 7;
+        const int chunk = pos ^ ((row >> 1) & 7);
+        int gr = m0 + row;
+        gr = gr < p.M ? gr : p.M - 1;
+        a_off[i] = (unsigned)((long long)(gr - m0) * lda + chunk * 16);
+    }
+    const unsigned char *a_base = p.x + (long long)m0 * lda;
+    auto issue_a = [&](int kt, unsigned char *la) {
+        const unsigned char *src = a_base + (long long)kt * (KT * 2);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const unsigned lds_addr = (unsigned)reinterpret_cast<size_t>((lds_void *)(la + (i * 256 + wave * 64) * 16));
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         :: "s"(lds_addr), "v"(a_off[i]), "s"(src) : "memory");
+        }
+    };
+
+    // ---- A fragments: row 32j + r, chunk (4h + t) ^ ((r >> 1) & 7)
+    int a_frag[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) a_frag[t] = r * 128 + (((4 * h + t) ^ ((r >> 1) & 7)) << 4);
+
+    // ---- B: buffer descriptors over this workgroup's weight rows (rows past N read as zero), the
+    // lane's two rows as 32-bit offsets, the reduction step as the scalar offset
+    const int groups_per_row = p.K / LQ_GROUP;
+    const int rows_here = p.N - c0 < BN ? p.N - c0 : BN;
+    auto make_rsrc = [](const void *base, unsigned bytes) {
+        const unsigned long long a = (unsigned long long)base;
+        u32x4_t d = {(unsigned)a, (unsigned)(a >> 32) & 0xFFFFu, bytes, 0x00020000u};
+        return d;
+    };
+    const u32x4_t w_rsrc = make_rsrc(p.w + (long long)c0 * (p.K / 2), (unsigned)rows_here * (unsigned)(p.K / 2));
+    const u32x4_t s_rsrc = make_rsrc(p.scales + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u);
+    const u32x4_t z_rsrc = make_rsrc(p.zeros + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u);
+    unsigned w_off[2], q_off[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const unsigned n = wave * 64 + i * 32 + r;
+        w_off[i] = n * (unsigned)(p.K / 2) + h * 16;
+        q_off[i] = n * (unsigned)groups_per_row * 2u;
+    }
+
+    f32x16_t acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0;
+
+    // All global loads of the loop are inline assembly: the compiler then inserts no vmcnt waits of
+    // its own (it could only wait for everything, LDS-direct loads included); the single
+    // s_waitcnt at the end of a step is tied to the loaded registers instead.
+    u32x4_t cw[2], cn[2];   // codes of the current and of the next step
+    unsigned qs[2], qz[2];  // raw bf16 scale / zero of the next group
+    float s[2], nzs[2];
+    auto load_codes = [&](int kt, u32x4_t *c) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(c[i]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * 32));
+    };
+    auto load_qparams = [&](int g) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            asm volatile("buffer_load_ushort %0, %1, %2, %3 offen" : "=v"(qs[i]) : "v"(q_off[i]), "s"(s_rsrc), "s"(g * 2));
+            asm volatile("buffer_load_ushort %0, %1, %2, %3 offen" : "=v"(qz[i]) : "v"(q_off[i]), "s"(z_rsrc), "s"(g * 2));
+        }
+    };
+    auto use_qparams = [&]() {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            s[i] = __uint_as_float(qs[i] << 16);
+            nzs[i] = -(__uint_as_float(qz[i] << 16) * s[i]);
+        }
+    };
+    auto read_a = [&](const unsigned char *la, int t, u32x4_t *af) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) af[j] = *reinterpret_cast<const u32x4_t *>(la + j * 4096 + a_frag[t]);
+    };
+    auto deq = [&](int t, u32x4_t *bf) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            float f[8];
+            lq_dequant_word_f32(cw[i][t], s[i], nzs[i], f);
+            bf[i] = u32x4_t{lq_pack_bf16(f[0], f[1]), lq_pack_bf16(f[2], f[3]), lq_pack_bf16(f[4], f[5]),
+                            lq_pack_bf16(f[6], f[7])};
+        }
+    };
+    auto mfma = [&](const u32x4_t *af, const u32x4_t *bf) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[i]),
+                                                                   __builtin_bit_cast(bf16x8_t, af[j]), acc[i][j], 0, 0, 0);
+    };
+
+    // One reduction step on stage AI with the codes in cw. Even steps start a quantisation group
+    // (its scale and zero were fetched during the previous, odd step); odd steps fetch the next
+    // group's. Within the step, the fragment reads and the dequantisation of slice t+1 are issued
+    // together with the MFMAs of slice t.
+    auto step = [&](int kt, auto ai, auto odd) {
+        constexpr int AI = decltype(ai)::value;
+        constexpr bool ODD = decltype(odd)::value != 0;
+        const unsigned char *la = abuf(ic<AI>());
+        u32x4_t af[2][4], bf[2][2];
+        if (!ODD) use_qparams();
+        read_a(la, 0, af[0]);
+        if (ODD) load_qparams(kt + 1 < nk ? (kt + 1) >> 1 : kt >> 1);
+        load_codes(kt + 1 < nk ? kt + 1 : kt, cn);
+        issue_a(kt + 2 < nk ? kt + 2 : nk - 1, abuf(ic<(AI + 2) % 3>()));
+        deq(0, bf[0]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            if (t < 3) {
+                read_a(la, t + 1, af[(t + 1) & 1]);
+                deq(t + 1, bf[(t + 1) & 1]);
+            }
+            mfma(af[t & 1], bf[t & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // Everything this wave loaded for step kt+1 has arrived (all but the 4 newest loads, the
+        // LDS-direct loads of tile kt+2) and its fragment reads of tile kt have returned: meet the
+        // other waves.
+        if (ODD)
+            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier"
+                         : "+v"(cn[0]), "+v"(cn[1]), "+v"(qs[0]), "+v"(qs[1]), "+v"(qz[0]), "+v"(qz[1]) :: "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" : "+v"(cn[0]), "+v"(cn[1]) :: "memory");
+        cw[0] = cn[0];
+        cw[1] = cn[1];
+    };
+
+    load_qparams(0);
+    load_codes(0, cn);
+    issue_a(0, lds_a0);
+    issue_a(nk > 1 ? 1 : 0, lds_a1);
+    asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier"
+                 : "+v"(cn[0]), "+v"(cn[1]), "+v"(qs[0]), "+v"(qs[1]), "+v"(qz[0]), "+v"(qz[1]) :: "memory");
+    cw[0] = cn[0];
+    cw[1] = cn[1];
+    int kt = 0;
+    for (; kt + 6 <= nk; kt += 6) {
+        step(kt, ic<0>(), ic<0>());
+        step(kt + 1, ic<1>(), ic<1>());
+        step(kt + 2, ic<2>(), ic<0>());
+        step(kt + 3, ic<0>(), ic<1>());
+        step(kt + 4, ic<1>(), ic<0>());
+        step(kt + 5, ic<2>(), ic<1>());
+    }
+    // nk is even (K is a multiple of 128) and kt a multiple of 6: 0, 2 or 4 steps remain
+    const int rem = nk - kt;
+    if (rem > 0) { step(kt, ic<0>(), ic<0>()); step(kt + 1, ic<1>(), ic<1>()); }
+    if (rem > 2) { step(kt + 2, ic<2>(), ic<0>()); step(kt + 3, ic<0>(), ic<1>()); }
+    // the clamped prefetches of the last two steps are still writing LDS: drain them
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    // ---- epilogue: acc[i][j][q]: column c0 + 64*wave + 32i + 8*(q/4) + 4h + q%4, row m0 + 32j + r
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int m = m0 + j * 32 + r;
+        if (m >= p.M) continue;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int c = c0 + wave * 64 + i * 32 + 8 * q + 4 * h;
+                if (c >= p.N) continue;  // N is a multiple of 4: a quad is all-in or all-out
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = acc[i][j][4 * q + e];
+                    if (p.bias) v[e] += lq_bf16_bits_to_f32(p.bias[c + e]);
+                }
+                u32x2_t o = {lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3])};
+                *reinterpret_cast<u32x2_t *>(p.y + (long long)m * p.N + c) = o;
+            }
+        }
+    }
+}
+
+}  // namespace
+
+// Number of workgroups this kernel would launch; the dispatcher in lq_gemm.hip prefers it when they
+// can fill the device two per CU.
+long long lq_gemm_fwd_direct_workgroups(int M, int N) { return (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN); }
+
+// Called by lq_a16w4_fwd (lq_gemm.hip) after argument validation: K % 128 == 0, N % 16 == 0, M > 16.
+int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
+                              void *y, int M, int N, int K, hipStream_t st) {
+    FwdParams p = {};
+    p.x = (const unsigned char *)x; p.w = (const unsigned char *)codes;
+    p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
+    p.bias = (const unsigned short *)bias; p.y = (unsigned short *)y;
+    p.M = M; p.N = N; p.K = K;
+    p.tiles_m = (M + BM - 1) / BM;
+    p.tiles_n = (N + BN - 1) / BN;
+    const long long nwg = (long long)p.tiles_m * p.tiles_n;
+    if (nwg > 0x7FFFFFFFll) return lq_fail(LQ_ERR_BAD_ARG, "lq_a16w4_fwd: problem too large");
+    // the 32-bit lane offsets of the A loads span 128 rows of K bf16
+    if ((long long)BM * K * 2 >= (1ll << 32)) return lq_fail(LQ_ERR_BAD_ARG, "lq_a16w4_fwd: K too large");
+    hipLaunchKernelGGL(gemm_fwd_direct_kernel, dim3((unsigned)nwg), dim3(256), 0, st, p);
+    return lq_check_launch("lq_a16w4_fwd");
+}

@@ -166,7 +166,9 @@ def _fwd_case(ops, co, M, N, K, seed, with_bias):
 
 
 @pytest.mark.parametrize("M,N,K,bias", [(17, 16, 128, False), (33, 48, 256, True), (128, 128, 128, False),
-                                        (129, 256, 384, True), (300, 272, 512, False), (1024, 3072, 768, True)])
+                                        (129, 256, 384, True), (300, 272, 512, False), (1024, 3072, 768, True),
+                                        # ragged in M and N and large enough for the weights-direct kernel
+                                        (4100, 4112, 128, True), (3000, 6160, 384, False)])
 def test_a16w4_fwd_gemm(ops, co, M, N, K, bias):
     _fwd_case(ops, co, M, N, K, seed=M + N + K, with_bias=bias)
 
