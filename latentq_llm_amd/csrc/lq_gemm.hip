@@ -1,19 +1,24 @@
 // Kernels (2a) and (3): LDS-tiled MFMA GEMMs for gfx950.
 //
 //   MODE_W4_FWD : Y[M,N]  = X[M,K]  . deq(W)[N,K]^T     (bf16 MFMA, int4 W dequantised into LDS)
-//   MODE_W4_DX  : dX[M,K] = dY[M,N] . deq(W)[N,K]       (same, W tile transposed while staging)
+//   MODE_W4_DX  : dX[M,K] = dY[M,N] . deq(W)[N,K]       (same, W tile transposed on the way out of LDS)
 //   MODE_I8     : acc     = X8[M,K] . W8[N,K]^T         (int8 MFMA, int32 accumulate, scaled epilogue)
+//
+// (The forward pass of large grids runs the weights-direct kernel of lq_gemm_fwd.hip instead.)
 //
 // Common structure. "A" is the activation-side operand, row-major with the reduction
 // dimension contiguous. "B" is the weight-side operand, presented in LDS as
-// [output column][reduction] exactly like A. A tile row holds 128 bytes (64 bf16 or
+// [output column][reduction] exactly like A, except in MODE_W4_DX: there the reduction runs
+// over n, the tile is kept in the weights' own [n][k] order (64 rows of 256 bytes, written as
+// plain 16-byte pieces) and the math waves fetch their operands with the transposing LDS read
+// ds_read_b64_tr_b16, so that the weight waves do the same cheap work in both directions. A tile row holds 128 bytes (64 bf16 or
 // 128 int8) = eight 16-byte chunks; one MFMA step consumes 32 bytes of every row
 // (chunks 2s and 2s+1), i.e. 4 steps per tile. Bank conflicts of the 16-byte fragment
 // reads (consecutive rows, same chunk) are avoided in two ways:
 //   * A rows are padded to 144 bytes, so consecutive rows start 16 bytes further round the
 //     banks and every fragment address is (lane base) + compile-time offset;
-//   * B rows stay 128 bytes and chunk c of row r sits at position c ^ ((r ^ (r >> 3)) & 7),
-//     which also keeps the transposing writes of the dX staging (rows 8 apart) apart.
+//   * B rows stay 128 bytes and chunk c of row r sits at position c ^ ((r ^ (r >> 3)) & 7)
+//     (MODE_W4_DX: see swz_dx).
 //
 // The MFMA is issued with the weight fragment as the first operand and the activation
 // fragment as the second, so that D[i][j] has i = output column (n), j = row (m): a
@@ -62,11 +67,17 @@ struct GemmParams {
 
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void gbl_void;
+typedef short v4s_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 
 template <int I>
 using ic = std::integral_constant<int, I>;
 
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
+// dX tile ([n][k], 256-byte rows of eight 32-byte pieces): piece c of row n sits at c ^ swz_dx(n).
+// A transposing read touches rows n..n+3 and n+8..n+11 at two adjacent pieces: the row's low two
+// bits move it to a different 64-byte pair, bit 2 spreads the writes of rows 4 apart.
+__device__ __forceinline__ int swz_dx(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
 
 // byte N of a dword as float, one instruction each
 __device__ __forceinline__ float ubyte0(unsigned x) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(x)); return r; }
@@ -150,21 +161,21 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
         // ======================= weight waves: B tiles =======================
         //   I8      : BPT 16-byte chunks per thread, copied through registers.
         //   W4_FWD  : NW code words (8 k each) of one weight row -> NW 16-byte chunks of that row.
-        //   W4_DX   : one code word (8 k) from each of RPT consecutive weight rows n -> for each
-        //             of the 8 k, RPT consecutive n (2*RPT bytes) of LDS row k.
+        //   W4_DX   : 4 code words (32 k) of one weight row n -> four 16-byte pieces of LDS row n. The
+        //             tile stays in the weights' own [n][k] order; the math waves transpose it on
+        //             the way out of LDS (ds_read_b64_tr_b16).
         constexpr int BPT = (MODE == MODE_I8) ? BN * 8 / NT : 1;
         constexpr int NW = (MODE == MODE_W4_FWD) ? BN * 8 / NT : 1;  // tile has BN rows x 8 words
-        constexpr int RPT = (MODE == MODE_W4_DX) ? 8 * BN / NT : 1;  // tile has 64 rows x BN/8 words
         static_assert(MODE != MODE_W4_FWD || NW == 2 || NW == 4 || NW == 8, "bad fwd staging split");
-        static_assert(MODE != MODE_W4_DX || RPT == 4, "dX staging expects 4 weight rows per thread");
-        constexpr int NSZ = (MODE == MODE_W4_DX) ? RPT : 1;
-        constexpr int NWORDS = NW > RPT ? NW : RPT;
+        static_assert(MODE != MODE_W4_DX || (BN == 128 && NT == 256), "dX staging: 64 rows x 4 threads");
+        constexpr int NSZ = 1;
+        constexpr int NWORDS = (MODE == MODE_W4_DX) ? 4 : NW;
 
-        const unsigned char *b_src[MODE == MODE_I8 ? BPT : (MODE == MODE_W4_DX ? RPT : 1)];
+        const unsigned char *b_src[MODE == MODE_I8 ? BPT : 1];
         int b_dst[MODE == MODE_I8 ? BPT : 1];
         const unsigned short *s_src[NSZ];
         const unsigned short *z_src[NSZ];
-        int b_row = 0, b_w0 = 0;  // W4_FWD: LDS row and first word; W4_DX: first LDS row (k) and n-block
+        int b_row = 0, b_w0 = 0;  // W4_FWD: LDS row and first word; W4_DX: LDS row (n) and quarter of the row
 
         if constexpr (MODE == MODE_I8) {
 #pragma unroll
@@ -186,18 +197,12 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             s_src[0] = p.scales + (long long)gr * groups_per_row;
             z_src[0] = p.zeros + (long long)gr * groups_per_row;
         } else {
-            constexpr int KWT = BN / 8;  // code words per weight row in the tile
-            const int kw = tid % KWT, nblk = tid / KWT;
-#pragma unroll
-            for (int r = 0; r < RPT; ++r) {
-                const int n = nblk * RPT + r;  // tile offset along n is added per tile
-                b_src[r] = (const unsigned char *)p.b + (long long)n * (p.Kw / 2) + (c0 / 8 + kw) * 4;
-                const int g = (c0 + kw * 8) / LQ_GROUP;
-                s_src[r] = p.scales + (long long)n * groups_per_row + g;
-                z_src[r] = p.zeros + (long long)n * groups_per_row + g;
-            }
-            b_row = kw * 8;
-            b_w0 = nblk;
+            b_row = tid >> 2;  // n within the tile (the tile offset along n is added per tile)
+            b_w0 = tid & 3;    // 32 of the tile's 128 output columns k
+            b_src[0] = (const unsigned char *)p.b + (long long)b_row * (p.Kw / 2) + c0 / 2 + b_w0 * 16;
+            const int g = (c0 + b_w0 * 32) / LQ_GROUP;
+            s_src[0] = p.scales + (long long)b_row * groups_per_row + g;
+            z_src[0] = p.zeros + (long long)b_row * groups_per_row + g;
         }
 
         struct Stage {
@@ -229,12 +234,11 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
                 S.z[0] = z_src[0][kt >> 1];
             } else {
                 const long long row_off = (long long)kt * 64;
+                u32x4_t v = *reinterpret_cast<const u32x4_t *>(b_src[0] + row_off * (p.Kw / 2));
 #pragma unroll
-                for (int r = 0; r < RPT; ++r) {
-                    S.w[r] = *reinterpret_cast<const unsigned *>(b_src[r] + row_off * (p.Kw / 2));
-                    S.s[r] = s_src[r][row_off * groups_per_row];
-                    S.z[r] = z_src[r][row_off * groups_per_row];
-                }
+                for (int i = 0; i < 4; ++i) S.w[i] = v[i];
+                S.s[0] = s_src[0][row_off * groups_per_row];
+                S.z[0] = z_src[0][row_off * groups_per_row];
             }
         };
 
@@ -255,20 +259,16 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
                     *reinterpret_cast<u32x4_t *>(lb + b_row * ROWB + ((ch ^ swz(b_row)) << 4)) = v;
                 }
             } else {
-                float f[RPT][8];
+                const float s = lq_bf16_bits_to_f32(S.s[0]);
+                const float nzs = -(lq_bf16_bits_to_f32(S.z[0]) * s);
 #pragma unroll
-                for (int r = 0; r < RPT; ++r) {
-                    const float s = lq_bf16_bits_to_f32(S.s[r]);
-                    const float nzs = -(lq_bf16_bits_to_f32(S.z[r]) * s);
-                    dequant_word_f32(S.w[r], s, nzs, f[r]);
-                }
-                const int byte0 = b_w0 * RPT * 2;  // byte offset of this thread's n-block inside the LDS row
-                const int ch = byte0 >> 4, sub = byte0 & 15;
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int row = b_row + j;
-                    u32x2_t v = {lq_pack_bf16(f[0][j], f[1][j]), lq_pack_bf16(f[2][j], f[3][j])};
-                    *reinterpret_cast<u32x2_t *>(lb + row * ROWB + ((ch ^ swz(row)) << 4) + sub) = v;
+                for (int w = 0; w < 4; ++w) {
+                    float f[8];
+                    dequant_word_f32(S.w[w], s, nzs, f);
+                    u32x4_t v = {lq_pack_bf16(f[0], f[1]), lq_pack_bf16(f[2], f[3]), lq_pack_bf16(f[4], f[5]),
+                                 lq_pack_bf16(f[6], f[7])};
+                    const int c32 = b_w0 * 2 + (w >> 1);  // 32-byte piece of the 256-byte row
+                    *reinterpret_cast<u32x4_t *>(lb + b_row * 256 + ((c32 ^ swz_dx(b_row)) << 5) + (w & 1) * 16) = v;
                 }
             }
         };
@@ -342,14 +342,42 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
         b_frag_off[i] = row * ROWB;
         b_frag_swz[i] = swz(row);
     }
+    // dX: the B tile is stored [n][k]; an MFMA lane needs 8 consecutive n of one k. A transposing
+    // read hands lane i of each 16-lane block the column i%4 of the four 8-byte rows addressed by
+    // lanes i/4, i/4 + 4, i/4 + 8, i/4 + 12 of that block. Let block lane r address row n0 + r/4
+    // at columns k0 + 4*(r%4): lane i then receives W[n0 .. n0+3][k0 + i]. The four blocks of a
+    // wave are (k0, n0) = (0, 0), (16, 0), (0, 8), (16, 8); a second read 4 rows further down
+    // completes the 8 n of the operand.
+    int dx_off[FN][2];
+    if constexpr (MODE == MODE_W4_DX) {
+        const int i16 = lane & 15, blk = lane >> 4;
+        const int row_lane = 8 * (blk >> 1) + (i16 >> 2), colblk = blk & 1, jj = (i16 >> 2) & 3;
+#pragma unroll
+        for (int i = 0; i < FN; ++i)
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int c32 = (wn * TN + i * 32) / 16 + colblk;
+                dx_off[i][e] = (row_lane + 4 * e) * 256 + ((c32 ^ ((jj << 1) | e)) << 5) + 8 * (i16 & 3);
+            }
+    }
     auto read_frags = [&](const unsigned char *la, const unsigned char *lb, int ks, u32x4_t *af, u32x4_t *bf) {
         const int ch = 2 * ks + kh;
 #pragma unroll
         for (int i = 0; i < FM; ++i)
             af[i] = *reinterpret_cast<const u32x4_t *>(la + a_lane_off + i * 32 * AROW + ks * 32);
+        if constexpr (MODE == MODE_W4_DX) {
 #pragma unroll
-        for (int i = 0; i < FN; ++i)
-            bf[i] = *reinterpret_cast<const u32x4_t *>(lb + b_frag_off[i] + ((ch ^ b_frag_swz[i]) << 4));
+            for (int i = 0; i < FN; ++i) {
+                const v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)(lb + dx_off[i][0] + ks * 4096));
+                const v4s_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)(lb + dx_off[i][1] + ks * 4096));
+                const u32x2_t l2 = __builtin_bit_cast(u32x2_t, lo), h2 = __builtin_bit_cast(u32x2_t, hi);
+                bf[i] = u32x4_t{l2[0], l2[1], h2[0], h2[1]};
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < FN; ++i)
+                bf[i] = *reinterpret_cast<const u32x4_t *>(lb + b_frag_off[i] + ((ch ^ b_frag_swz[i]) << 4));
+        }
     };
     auto mfma_step = [&](const u32x4_t *af, const u32x4_t *bf) {
 #pragma unroll
@@ -473,6 +501,13 @@ static int lq_device_cu_count() {
     return cached[dev];
 }
 
+// 128 x 128 tiles when 256 x 128 tiles would leave compute units without a workgroup
+static bool small_tiles(const GemmParams &p) {
+    if (p.M <= 128) return true;
+    const long long big = (long long)((p.M + 255) / 256) * ((p.C + 127) / 128);
+    return big < lq_device_cu_count();
+}
+
 // weights-direct forward GEMM (lq_gemm_fwd.hip)
 long long lq_gemm_fwd_direct_workgroups(int M, int N);
 int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
@@ -513,7 +548,7 @@ extern "C" int lq_a16w4_fwd(const void *x, const void *codes, const void *scales
     p.a = x; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.bias = (const unsigned short *)bias_or_null; p.c = y;
     p.M = (int)M; p.C = (int)N; p.R = (int)K; p.Kw = (int)K;
-    if (M <= 128) return launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, "lq_a16w4_fwd");
+    if (small_tiles(p)) return launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, "lq_a16w4_fwd");
     return launch_gemm<MODE_W4_FWD, 256, 128, 2, 2>(p, (hipStream_t)stream, "lq_a16w4_fwd");
 }
 
@@ -526,7 +561,7 @@ extern "C" int lq_a16w4_dx(const void *dy, const void *codes, const void *scales
     p.a = dy; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.c = dx;
     p.M = (int)M; p.C = (int)K; p.R = (int)N; p.Kw = (int)K;
-    if (M <= 128) return launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, "lq_a16w4_dx");
+    if (small_tiles(p)) return launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, "lq_a16w4_dx");
     return launch_gemm<MODE_W4_DX, 256, 128, 2, 2>(p, (hipStream_t)stream, "lq_a16w4_dx");
 }
 
@@ -544,6 +579,6 @@ extern "C" int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const 
     p.a = x; p.b = w; p.sx = sx; p.sw = sw; p.bias = (const unsigned short *)bias_or_null; p.c = y;
     p.acc_out = acc_or_null;
     p.M = (int)M; p.C = (int)N; p.R = (int)K; p.Kw = (int)K;
-    if (M <= 128) return launch_gemm<MODE_I8, 128, 128, 2, 2>(p, (hipStream_t)stream, "lq_a8w8_fwd");
+    if (small_tiles(p)) return launch_gemm<MODE_I8, 128, 128, 2, 2>(p, (hipStream_t)stream, "lq_a8w8_fwd");
     return launch_gemm<MODE_I8, 256, 128, 2, 2>(p, (hipStream_t)stream, "lq_a8w8_fwd");
 }
