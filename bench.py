@@ -189,7 +189,7 @@ def bench_copy(device):
     return {"bytes_each_way": nbytes, "us": sec * 1e6, "GB/s": 2 * nbytes / sec / 1e9}
 
 
-def profile_target(device, which, launches=5):
+def profile_target(device, which, launches=10):
     """A short, fixed sequence of launches for a profiler run (kernel trace or counters): the
     calibration copy first, then the kernels of the named family, `launches` times each."""
     from latentq_llm_amd import _C, ops as o

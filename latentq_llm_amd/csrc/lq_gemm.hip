@@ -18,7 +18,7 @@
 //   * A rows are padded to 144 bytes, so consecutive rows start 16 bytes further round the
 //     banks and every fragment address is (lane base) + compile-time offset;
 //   * B rows stay 128 bytes and chunk c of row r sits at position c ^ ((r ^ (r >> 3)) & 7)
-//     (MODE_W4_DX: see swz_dx).
+//     (MODE_W4_DX: see swz_dx_piece).
 //
 // The MFMA is issued with the weight fragment as the first operand and the activation
 // fragment as the second, so that D[i][j] has i = output column (n), j = row (m): a
@@ -74,10 +74,13 @@ template <int I>
 using ic = std::integral_constant<int, I>;
 
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
-// dX tile ([n][k], 256-byte rows of eight 32-byte pieces): piece c of row n sits at c ^ swz_dx(n).
-// A transposing read touches rows n..n+3 and n+8..n+11 at two adjacent pieces: the row's low two
-// bits move it to a different 64-byte pair, bit 2 spreads the writes of rows 4 apart.
-__device__ __forceinline__ int swz_dx(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
+// dX tile ([n][k], 256-byte rows of eight 32-byte pieces, each two 16-byte halves): with j = n & 3,
+// piece c of row n sits at c ^ (2j | (j & 1)) and its halves are swapped when j >= 2. The 16
+// lanes of a staging write (4 consecutive rows x 4 quarter rows) then fall on 16 different
+// 16-byte slots of the bank space, and a transposing read (rows n..n+3 at two adjacent pieces,
+// per 32 lanes) covers every bank once.
+__device__ __forceinline__ int swz_dx_piece(int row) { return ((row & 3) << 1) | (row & 1); }
+__device__ __forceinline__ int swz_dx_half(int row) { return (row >> 1) & 1; }
 
 // byte N of a dword as float, one instruction each
 __device__ __forceinline__ float ubyte0(unsigned x) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(x)); return r; }
@@ -268,7 +271,8 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
                     u32x4_t v = {lq_pack_bf16(f[0], f[1]), lq_pack_bf16(f[2], f[3]), lq_pack_bf16(f[4], f[5]),
                                  lq_pack_bf16(f[6], f[7])};
                     const int c32 = b_w0 * 2 + (w >> 1);  // 32-byte piece of the 256-byte row
-                    *reinterpret_cast<u32x4_t *>(lb + b_row * 256 + ((c32 ^ swz_dx(b_row)) << 5) + (w & 1) * 16) = v;
+                    *reinterpret_cast<u32x4_t *>(lb + b_row * 256 + ((c32 ^ swz_dx_piece(b_row)) << 5) +
+                                                 (((w & 1) ^ swz_dx_half(b_row)) << 4)) = v;
                 }
             }
         };
@@ -348,17 +352,16 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
     // at columns k0 + 4*(r%4): lane i then receives W[n0 .. n0+3][k0 + i]. The four blocks of a
     // wave are (k0, n0) = (0, 0), (16, 0), (0, 8), (16, 8); a second read 4 rows further down
     // completes the 8 n of the operand.
-    int dx_off[FN][2];
+    int dx_off[FN];
     if constexpr (MODE == MODE_W4_DX) {
         const int i16 = lane & 15, blk = lane >> 4;
-        const int row_lane = 8 * (blk >> 1) + (i16 >> 2), colblk = blk & 1, jj = (i16 >> 2) & 3;
+        const int row_lane = 8 * (blk >> 1) + (i16 >> 2), colblk = blk & 1;  // row_lane & 3 is the row's j
 #pragma unroll
-        for (int i = 0; i < FN; ++i)
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const int c32 = (wn * TN + i * 32) / 16 + colblk;
-                dx_off[i][e] = (row_lane + 4 * e) * 256 + ((c32 ^ ((jj << 1) | e)) << 5) + 8 * (i16 & 3);
-            }
+        for (int i = 0; i < FN; ++i) {
+            const int c32 = (wn * TN + i * 32) / 16 + colblk;
+            dx_off[i] = row_lane * 256 + ((c32 ^ swz_dx_piece(row_lane)) << 5) +
+                        ((((i16 & 3) >> 1) ^ swz_dx_half(row_lane)) << 4) + (i16 & 1) * 8;
+        }
     }
     auto read_frags = [&](const unsigned char *la, const unsigned char *lb, int ks, u32x4_t *af, u32x4_t *bf) {
         const int ch = 2 * ks + kh;
@@ -368,8 +371,8 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
         if constexpr (MODE == MODE_W4_DX) {
 #pragma unroll
             for (int i = 0; i < FN; ++i) {
-                const v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)(lb + dx_off[i][0] + ks * 4096));
-                const v4s_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)(lb + dx_off[i][1] + ks * 4096));
+                const v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)(lb + dx_off[i] + ks * 4096));
+                const v4s_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)(lb + dx_off[i] + ks * 4096 + 1024));
                 const u32x2_t l2 = __builtin_bit_cast(u32x2_t, lo), h2 = __builtin_bit_cast(u32x2_t, hi);
                 bf[i] = u32x4_t{l2[0], l2[1], h2[0], h2[1]};
             }
