@@ -11,14 +11,12 @@
 // [output column][reduction] exactly like A, except in MODE_W4_DX: there the reduction runs
 // over n, the tile is kept in the weights' own [n][k] order (64 rows of 256 bytes, written as
 // plain 16-byte pieces) and the math waves fetch their operands with the transposing LDS read
-// ds_read_b64_tr_b16, so that the weight waves do the same cheap work in both directions. A tile row holds 128 bytes (64 bf16 or
-// 128 int8) = eight 16-byte chunks; one MFMA step consumes 32 bytes of every row
-// (chunks 2s and 2s+1), i.e. 4 steps per tile. Bank conflicts of the 16-byte fragment
-// reads (consecutive rows, same chunk) are avoided in two ways:
-//   * A rows are padded to 144 bytes, so consecutive rows start 16 bytes further round the
-//     banks and every fragment address is (lane base) + compile-time offset;
-//   * B rows stay 128 bytes and chunk c of row r sits at position c ^ ((r ^ (r >> 3)) & 7)
-//     (MODE_W4_DX: see swz_dx_piece).
+// ds_read_b64_tr_b16, so that the weight waves do the same cheap work in both directions.
+// A tile row holds 128 bytes (64 bf16 or 128 int8) = eight 16-byte chunks; one MFMA step
+// consumes 32 bytes of every row (chunks 2s and 2s+1), i.e. 4 steps per tile. Bank conflicts of
+// the 16-byte fragment reads (consecutive rows, same chunk) are avoided by XOR swizzles:
+//   * chunk c of A row r sits at position c ^ ((r >> 1) & 7);
+//   * chunk c of B row r sits at position c ^ ((r ^ (r >> 3)) & 7) (MODE_W4_DX: see swz_dx_piece).
 //
 // The MFMA is issued with the weight fragment as the first operand and the activation
 // fragment as the second, so that D[i][j] has i = output column (n), j = row (m): a
@@ -28,9 +26,8 @@
 //   * The first WM x WN ("math") waves issue the MFMAs. They also fetch the A tiles, but with
 //     LDS-direct loads (global_load_lds_dwordx4): no registers, no vector-ALU work, 8
 //     instructions per tile, two tiles ahead of the tile being multiplied (three A buffers).
-//     An LDS-direct load writes lane l at (wave base) + 16*l, so the padded layout is produced
-//     on the global side: the lane that owns 16-byte slot s fetches chunk s%9 of row s/9
-//     (slot 8 of a row is the padding and re-fetches chunk 7).
+//     An LDS-direct load writes lane l at (wave base) + 16*l, so the swizzle is applied on the
+//     global side: the lane that owns 16-byte slot s fetches the chunk that belongs there.
 //   * The other WM x WN ("weight") waves turn packed int4 codes into bf16 B tiles: code loads two
 //     tiles ahead into registers, dequantisation on the vector ALUs, LDS writes one tile ahead
 //     (two B buffers). A single wave can issue one instruction every 4 cycles, so this
@@ -105,14 +102,14 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
     constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
     constexpr int FM = TM / 32, FN = TN / 32;  // 32x32 fragments per wave tile
     constexpr int ROWB = 128;                  // bytes of data per tile row (and per LDS row of B)
-    constexpr int AROW = 144;                  // bytes per LDS row of A (16 bytes of padding)
-    constexpr int APT = (BM * 9 + NT - 1) / NT;  // 16-byte LDS slots of A filled per math thread per tile
+    constexpr int AROW = 128;                  // bytes per LDS row of A
+    constexpr int APT = BM * 8 / NT;           // 16-byte LDS slots of A filled per math thread per tile
     constexpr int A_BYTES = APT * NT * 16, B_BYTES = BN * ROWB;
     constexpr int ESZ = (MODE == MODE_I8) ? 1 : 2;
     constexpr int RT = ROWB / ESZ;  // reduction elements per tile (64 bf16 / 128 int8)
     static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of 32x32");
     static_assert((BN * 8) % NT == 0, "B staging must divide evenly");
-    static_assert(A_BYTES >= BM * AROW, "A buffer too small");
+    static_assert(A_BYTES == BM * AROW && (BM * 8) % NT == 0, "A staging must divide evenly");
 
     __shared__ __attribute__((aligned(16))) unsigned char lds_a0[A_BYTES];
     __shared__ __attribute__((aligned(16))) unsigned char lds_a1[A_BYTES];
@@ -305,9 +302,9 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
     const long long lda = (long long)p.R * ESZ;
 #pragma unroll
     for (int i = 0; i < APT; ++i) {
-        const int slot = i * NT + tid;  // LDS slot: row slot/9, chunk slot%9 (8 = padding)
-        int row = slot / 9, ch = slot % 9;
-        ch = ch < 8 ? ch : 7;
+        const int slot = i * NT + tid;  // LDS slot: row slot/8, position slot%8 holds chunk pos ^ swizzle
+        const int row = slot >> 3;
+        const int ch = (slot & 7) ^ ((row >> 1) & 7);
         int gr = m0 + row;
         gr = gr < p.M ? gr : p.M - 1;
         a_off[i] = (unsigned)((gr - m0) * lda + ch * 16);
@@ -338,7 +335,11 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
     const int frag_row = lane & 31, kh = lane >> 5;
-    const int a_lane_off = (wm * TM + frag_row) * AROW + kh * 16;  // + i*32*AROW + ks*32: compile-time
+    // A fragment of slice ks: row wm*TM + 32i + frag_row, chunk 2ks + kh at position chunk ^ ((row >> 1) & 7)
+    int a_frag[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+        a_frag[ks] = (wm * TM + frag_row) * AROW + (((2 * ks + kh) ^ ((frag_row >> 1) & 7)) << 4);  // + i*32*AROW
     int b_frag_off[FN], b_frag_swz[FN];
 #pragma unroll
     for (int i = 0; i < FN; ++i) {
@@ -367,7 +368,7 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
         const int ch = 2 * ks + kh;
 #pragma unroll
         for (int i = 0; i < FM; ++i)
-            af[i] = *reinterpret_cast<const u32x4_t *>(la + a_lane_off + i * 32 * AROW + ks * 32);
+            af[i] = *reinterpret_cast<const u32x4_t *>(la + a_frag[ks] + i * 32 * AROW);
         if constexpr (MODE == MODE_W4_DX) {
 #pragma unroll
             for (int i = 0; i < FN; ++i) {
