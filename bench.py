@@ -108,23 +108,21 @@ class MLPBlock:
 
 MLP_FLOP = 6 * 2 * TOKENS * HID * FFN  # 1 108.1 GFLOP
 
-# HBM traffic per GEMM launch, from two counter runs of
+# HBM traffic per GEMM launch in MB (read, written), from two counter runs of
 #   rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --profile-target gemm     (then WRITE_SIZE)
-# in KiB per dispatch as the counters read, and the reading of the same counters for the
-# 256 MiB calibration copy in the same runs (262 144 KiB fetched and written).
-PMC_GEMM_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
-    "fwd_gate_up": (122755.4, 44051.4), "fwd_down": (92921.5, 16384.0),
-    "dx_gate_up": (96642.8, 16384.0), "dx_down": (136759.2, 44044.9),
+# each scaled by what the same counter reads for the 256 MiB calibration copy of the same run
+# (FETCH_SIZE reads half the bytes fetched: factor 2.000; WRITE_SIZE factor 1.000).
+PMC_GEMM_MB = {
+    "fwd_gate_up": (221.77, 45.16), "fwd_down": (190.62, 16.78),
+    "dx_gate_up": (195.82, 16.78), "dx_down": (280.18, 45.10),
 }
-PMC_COPY_KIB = (131083.0, 262158.0)
 PMC_LAUNCHES = {"fwd_gate_up": 2, "fwd_down": 1, "dx_gate_up": 2, "dx_down": 1}  # per MLP step
 
 
 def gemm_traffic_bytes():
     """Launch-weighted mean HBM bytes (read + written) per GEMM launch of the MLP step."""
-    fs, ws = 262144.0 / PMC_COPY_KIB[0], 262144.0 / PMC_COPY_KIB[1]
-    tot = sum(n * (PMC_GEMM_KIB[k][0] * fs + PMC_GEMM_KIB[k][1] * ws) for k, n in PMC_LAUNCHES.items())
-    return tot * 1024 / sum(PMC_LAUNCHES.values())
+    tot = sum(n * sum(PMC_GEMM_MB[k]) for k, n in PMC_LAUNCHES.items())
+    return tot * 1e6 / sum(PMC_LAUNCHES.values())
 
 
 def bench_requant(device):
@@ -329,7 +327,7 @@ def main():
     tot = 2 * kern["fwd_gate_up"]["us"] + kern["fwd_down"]["us"] + 2 * kern["dx_gate_up"]["us"] + kern["dx_down"]["us"]
     avg_us = tot / 6
     achieved = 2 * TOKENS * HID * FFN / (avg_us * 1e-6) / 1e12
-    roofline = {"bound": "mfma", "kernel": "gemm_kernel (A16W4 dequant-GEMM, fwd and dX instantiations)",
+    roofline = {"bound": "mfma", "kernel": "A16W4 dequant-GEMM: gemm_fwd_direct_kernel (forward gate/up), gemm_kernel<0> (forward down), gemm_kernel<1> (dX)",
                 "achieved": achieved, "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": achieved * 1e12 / PEAK_BF16,
                 "avg_launch_us": avg_us, "flop_per_launch": 2 * TOKENS * HID * FFN, "traffic": gemm_traffic_bytes(),
                 "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated on a copy)"}
