@@ -1,4 +1,7 @@
-// A16W4 forward GEMM for gfx950, M > 16:  Y[M,N] = X[M,K] . deq(W)[N,K]^T (+ bias), bf16 MFMA.
+// Weights-direct forward GEMMs for gfx950:
+//   A16W4, M > 16:  Y[M,N] = X[M,K] . deq(W)[N,K]^T (+ bias), bf16 MFMA
+//   A8W8 (template flag I8): the same structure on int8 operands, int32 accumulators and the fused
+//   scale epilogue; a lane then loads 64 bytes of its weight row per step and no dequantisation is needed.
 //
 // The weights never pass through LDS. An MFMA B-side lane needs 8 consecutive k of one weight
 // row, and 8 consecutive k of a row are exactly one 32-bit word of packed codes: every lane
@@ -40,11 +43,13 @@
 namespace {
 
 struct FwdParams {
-    const unsigned char *x;   // bf16 [M, K]
-    const unsigned char *w;   // packed codes, K/2 bytes per row
+    const unsigned char *x;   // bf16 [M, K] (int8 variant: int8 [M, K])
+    const unsigned char *w;   // packed codes, K/2 bytes per row (int8 variant: int8 [N, K])
     const unsigned short *scales;
     const unsigned short *zeros;
     const unsigned short *bias;  // bf16 [N] or null
+    const float *sx, *sw;        // int8 variant: per-row and per-column scales
+    int *acc_out;                // int8 variant: optional int32 [M, N]
     unsigned short *y;           // bf16 [M, N]
     int M, N, K;
     int tiles_m, tiles_n;
@@ -55,10 +60,15 @@ typedef __attribute__((address_space(3))) void lds_void;
 template <int I>
 using ic = std::integral_constant<int, I>;
 
-constexpr int BM = 128, BN = 256, KT = 64;
-constexpr int STAGE = BM * KT * 2;  // 16 KB per A stage
+constexpr int BM = 128, BN = 256;
+constexpr int ROWB = 128;            // bytes of A per tile row and step: 64 bf16 or 128 int8
+constexpr int STAGE = BM * ROWB;     // 16 KB per A stage
 
+template <bool I8>
 __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
+    constexpr int ESZ = I8 ? 1 : 2;          // bytes per A element
+    constexpr int WROW = I8 ? 128 : 32;      // bytes of one weight row consumed per step
+    constexpr int NB = I8 ? 4 : 1;           // 16-byte weight loads per lane, column tile and step
     __shared__ __attribute__((aligned(16))) unsigned char lds_a0[STAGE];
     __shared__ __attribute__((aligned(16))) unsigned char lds_a1[STAGE];
     __shared__ __attribute__((aligned(16))) unsigned char lds_a2[STAGE];
@@ -87,8 +97,8 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     const int bw = rest < GN ? rest : GN;
     const int tile_m = within / bw, tile_n = band * GN + within % bw;
     const int m0 = tile_m * BM, c0 = tile_n * BN;
-    const int nk = p.K / KT;
-    const long long lda = (long long)p.K * 2;
+    const int nk = p.K * ESZ / ROWB;
+    const long long lda = (long long)p.K * ESZ;
 
     // ---- A staging: 1024 16-byte slots per stage; slot s = i*256 + thread -> row s/8, position s%8
     unsigned a_off[4];
@@ -103,7 +113,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     }
     const unsigned char *a_base = p.x + (long long)m0 * lda;
     auto issue_a = [&](int kt, unsigned char *la) {
-        const unsigned char *src = a_base + (long long)kt * (KT * 2);
+        const unsigned char *src = a_base + (long long)kt * ROWB;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const unsigned lds_addr = (unsigned)reinterpret_cast<size_t>((lds_void *)(la + (i * 256 + wave * 64) * 16));
@@ -126,18 +136,20 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         u32x4_t d = {(unsigned)a, (unsigned)(a >> 32) & 0xFFFFu, bytes, 0x00020000u};
         return d;
     };
-    const u32x4_t w_rsrc = make_rsrc(p.w + (long long)c0 * (p.K / 2), (unsigned)rows_here * (unsigned)(p.K / 2));
+    const unsigned wpitch = I8 ? (unsigned)p.K : (unsigned)(p.K / 2);  // bytes per weight row
+    const u32x4_t w_rsrc = make_rsrc(p.w + (long long)c0 * wpitch, (unsigned)rows_here * wpitch);
     const u32x4_t s_rsrc = make_rsrc(p.scales + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u);
     const u32x4_t z_rsrc = make_rsrc(p.zeros + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u);
     unsigned w_off[2], q_off[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const unsigned n = wave * 64 + i * 32 + r;
-        w_off[i] = n * (unsigned)(p.K / 2) + h * 16;
+        w_off[i] = n * wpitch + h * (WROW / 2);
         q_off[i] = n * (unsigned)groups_per_row * 2u;
     }
 
-    f32x16_t acc[2][4];
+    using acc_t = typename std::conditional<I8, i32x16_t, f32x16_t>::type;
+    acc_t acc[2][4];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -148,13 +160,19 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     // All global loads of the loop are inline assembly: the compiler then inserts no vmcnt waits of
     // its own (it could only wait for everything, LDS-direct loads included); the single
     // s_waitcnt at the end of a step is tied to the loaded registers instead.
-    u32x4_t cw[2], cn[2];   // codes of the current and of the next step
+    u32x4_t cw[2][NB], cn[2][NB];  // weights of the current and of the next step (int4 codes or int8)
     unsigned qs[2], qz[2];  // raw bf16 scale / zero of the next group
     float s[2], nzs[2];
-    auto load_codes = [&](int kt, u32x4_t *c) {
+    auto load_codes = [&](int kt, u32x4_t (*c)[NB]) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-            asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(c[i]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * 32));
+        for (int i = 0; i < 2; ++i) {
+            asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(c[i][0]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
+            if constexpr (I8) {
+                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:16" : "=v"(c[i][1]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
+                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:32" : "=v"(c[i][2]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
+                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:48" : "=v"(c[i][3]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
+            }
+        }
     };
     auto load_qparams = [&](int g) {
 #pragma unroll
@@ -177,8 +195,12 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     auto deq = [&](int t, u32x4_t *bf) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
+            if constexpr (I8) {
+                bf[i] = cw[i][t];  // 16 int8 of the lane's row: already the MFMA operand
+                continue;
+            }
             float f[8];
-            lq_dequant_word_f32(cw[i][t], s[i], nzs[i], f);
+            lq_dequant_word_f32(cw[i][0][t], s[i], nzs[i], f);
             bf[i] = u32x4_t{lq_pack_bf16(f[0], f[1]), lq_pack_bf16(f[2], f[3]), lq_pack_bf16(f[4], f[5]),
                             lq_pack_bf16(f[6], f[7])};
         }
@@ -188,8 +210,33 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[i]),
-                                                                   __builtin_bit_cast(bf16x8_t, af[j]), acc[i][j], 0, 0, 0);
+                if constexpr (I8)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf[i]),
+                                                                     __builtin_bit_cast(i32x4_t, af[j]), acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[i]),
+                                                                       __builtin_bit_cast(bf16x8_t, af[j]), acc[i][j], 0, 0, 0);
+    };
+
+    // End of a step (and of the prologue): everything this wave loaded for the next step has
+    // arrived (all but the 4 newest loads, the LDS-direct loads of the tile after it), its fragment
+    // reads have returned: meet the other waves, then make the next step's weights current. The
+    // wait is tied to the registers the assembly loads wrote.
+    auto end_of_step = [&](auto with_qparams) {
+        if constexpr (I8) {
+            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier"
+                         : "+v"(cn[0][0]), "+v"(cn[0][1]), "+v"(cn[0][2]), "+v"(cn[0][3]), "+v"(cn[1][0]), "+v"(cn[1][1]),
+                           "+v"(cn[1][2]), "+v"(cn[1][3]) :: "memory");
+        } else if constexpr (decltype(with_qparams)::value != 0) {
+            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier"
+                         : "+v"(cn[0][0]), "+v"(cn[1][0]), "+v"(qs[0]), "+v"(qs[1]), "+v"(qz[0]), "+v"(qz[1]) :: "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" : "+v"(cn[0][0]), "+v"(cn[1][0]) :: "memory");
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int b = 0; b < NB; ++b) cw[i][b] = cn[i][b];
     };
 
     // One reduction step on stage AI with the codes in cw. Even steps start a quantisation group
@@ -201,9 +248,9 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         constexpr bool ODD = decltype(odd)::value != 0;
         const unsigned char *la = abuf(ic<AI>());
         u32x4_t af[2][4], bf[2][2];
-        if (!ODD) use_qparams();
+        if (!I8 && !ODD) use_qparams();
         read_a(la, 0, af[0]);
-        if (ODD) load_qparams(kt + 1 < nk ? (kt + 1) >> 1 : kt >> 1);
+        if (!I8 && ODD) load_qparams(kt + 1 < nk ? (kt + 1) >> 1 : kt >> 1);
         load_codes(kt + 1 < nk ? kt + 1 : kt, cn);
         issue_a(kt + 2 < nk ? kt + 2 : nk - 1, abuf(ic<(AI + 2) % 3>()));
         deq(0, bf[0]);
@@ -220,23 +267,14 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         // Everything this wave loaded for step kt+1 has arrived (all but the 4 newest loads, the
         // LDS-direct loads of tile kt+2) and its fragment reads of tile kt have returned: meet the
         // other waves.
-        if (ODD)
-            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier"
-                         : "+v"(cn[0]), "+v"(cn[1]), "+v"(qs[0]), "+v"(qs[1]), "+v"(qz[0]), "+v"(qz[1]) :: "memory");
-        else
-            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" : "+v"(cn[0]), "+v"(cn[1]) :: "memory");
-        cw[0] = cn[0];
-        cw[1] = cn[1];
+        end_of_step(ic<ODD ? 1 : 0>());
     };
 
-    load_qparams(0);
+    if (!I8) load_qparams(0);
     load_codes(0, cn);
     issue_a(0, lds_a0);
     issue_a(nk > 1 ? 1 : 0, lds_a1);
-    asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier"
-                 : "+v"(cn[0]), "+v"(cn[1]), "+v"(qs[0]), "+v"(qs[1]), "+v"(qz[0]), "+v"(qz[1]) :: "memory");
-    cw[0] = cn[0];
-    cw[1] = cn[1];
+    end_of_step(ic<1>());
     int kt = 0;
     for (; kt + 6 <= nk; kt += 6) {
         step(kt, ic<0>(), ic<0>());
@@ -246,10 +284,14 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         step(kt + 4, ic<1>(), ic<0>());
         step(kt + 5, ic<2>(), ic<1>());
     }
-    // nk is even (K is a multiple of 128) and kt a multiple of 6: 0, 2 or 4 steps remain
+    // kt is a multiple of 6 here, so the stage and parity phases restart at 0; 0..5 steps remain
+    // (an even number for int4 weights, whose K is a multiple of 128 = two steps)
     const int rem = nk - kt;
-    if (rem > 0) { step(kt, ic<0>(), ic<0>()); step(kt + 1, ic<1>(), ic<1>()); }
-    if (rem > 2) { step(kt + 2, ic<2>(), ic<0>()); step(kt + 3, ic<0>(), ic<1>()); }
+    if (rem > 0) step(kt, ic<0>(), ic<0>());
+    if (rem > 1) step(kt + 1, ic<1>(), ic<1>());
+    if (rem > 2) step(kt + 2, ic<2>(), ic<0>());
+    if (rem > 3) step(kt + 3, ic<0>(), ic<1>());
+    if (rem > 4) step(kt + 4, ic<1>(), ic<0>());
     // the clamped prefetches of the last two steps are still writing LDS: drain them
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
@@ -258,6 +300,8 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     for (int j = 0; j < 4; ++j) {
         const int m = m0 + j * 32 + r;
         if (m >= p.M) continue;
+        float sxm = 1.0f;
+        if constexpr (I8) sxm = p.sx[m];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
 #pragma unroll
@@ -267,11 +311,18 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    v[e] = acc[i][j][4 * q + e];
+                    if constexpr (I8) v[e] = ((float)acc[i][j][4 * q + e] * sxm) * p.sw[c + e];
+                    else v[e] = acc[i][j][4 * q + e];
                     if (p.bias) v[e] += lq_bf16_bits_to_f32(p.bias[c + e]);
                 }
                 u32x2_t o = {lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3])};
                 *reinterpret_cast<u32x2_t *>(p.y + (long long)m * p.N + c) = o;
+                if constexpr (I8) {
+                    if (p.acc_out) {
+                        i32x4_t a4 = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                        *reinterpret_cast<i32x4_t *>(p.acc_out + (long long)m * p.N + c) = a4;
+                    }
+                }
             }
         }
     }
@@ -283,6 +334,18 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
 // can fill the device two per CU.
 long long lq_gemm_fwd_direct_workgroups(int M, int N) { return (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN); }
 
+static int launch_direct(FwdParams p, bool i8, hipStream_t st, const char *who) {
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    const long long nwg = (long long)p.tiles_m * p.tiles_n;
+    if (nwg > 0x7FFFFFFFll) return lq_fail(LQ_ERR_BAD_ARG, "%s: problem too large", who);
+    // the 32-bit lane offsets of the activation and weight loads span 128 / 256 rows
+    if ((long long)BN * p.K * 2 >= (1ll << 32)) return lq_fail(LQ_ERR_BAD_ARG, "%s: K too large", who);
+    if (i8) hipLaunchKernelGGL(gemm_fwd_direct_kernel<true>, dim3((unsigned)nwg), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(gemm_fwd_direct_kernel<false>, dim3((unsigned)nwg), dim3(256), 0, st, p);
+    return lq_check_launch(who);
+}
+
 // Called by lq_a16w4_fwd (lq_gemm.hip) after argument validation: K % 128 == 0, N % 16 == 0, M > 16.
 int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
                               void *y, int M, int N, int K, hipStream_t st) {
@@ -291,12 +354,15 @@ int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scal
     p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.bias = (const unsigned short *)bias; p.y = (unsigned short *)y;
     p.M = M; p.N = N; p.K = K;
-    p.tiles_m = (M + BM - 1) / BM;
-    p.tiles_n = (N + BN - 1) / BN;
-    const long long nwg = (long long)p.tiles_m * p.tiles_n;
-    if (nwg > 0x7FFFFFFFll) return lq_fail(LQ_ERR_BAD_ARG, "lq_a16w4_fwd: problem too large");
-    // the 32-bit lane offsets of the A loads span 128 rows of K bf16
-    if ((long long)BM * K * 2 >= (1ll << 32)) return lq_fail(LQ_ERR_BAD_ARG, "lq_a16w4_fwd: K too large");
-    hipLaunchKernelGGL(gemm_fwd_direct_kernel, dim3((unsigned)nwg), dim3(256), 0, st, p);
-    return lq_check_launch("lq_a16w4_fwd");
+    return launch_direct(p, false, st, "lq_a16w4_fwd");
+}
+
+// Called by lq_a8w8_fwd (lq_gemm.hip) after argument validation: K % 128 == 0, N % 16 == 0.
+int lq_gemm_i8_direct_launch(const void *x8, const void *w8, const float *sx, const float *sw, const void *bias, void *y,
+                             int *acc_or_null, int M, int N, int K, hipStream_t st) {
+    FwdParams p = {};
+    p.x = (const unsigned char *)x8; p.w = (const unsigned char *)w8; p.sx = sx; p.sw = sw;
+    p.bias = (const unsigned short *)bias; p.y = (unsigned short *)y; p.acc_out = acc_or_null;
+    p.M = M; p.N = N; p.K = K;
+    return launch_direct(p, true, st, "lq_a8w8_fwd");
 }
