@@ -142,6 +142,28 @@ def bench_requant(device):
             "bytes": nbytes, "noise": "in-kernel Philox4x32-10"}
 
 
+def bench_latent(device):
+    """The two fused passes of the exact 4-bit-residual latent mode (lbit = 4) on the requantizer's shape."""
+    from latentq_llm_amd import ops
+    N, K = 8192, 2048
+    curve = (2, 0.125, 2, 0.25, 4)  # k1, b1, k2, b2, k3 of the default companding curve
+    sets = []
+    for i in range(8):
+        p, s, z = synth_w4(N, K, 40 + i, device)
+        res = torch.randint(-2 ** 31, 2 ** 31 - 1, (N * K // 8,), device=device, dtype=torch.int64).to(torch.int32)
+        lat = ops.latent_w4_reconstruct(p, s, z, res, (N, K), *curve)
+        sets.append((p, s, z, res, lat))
+    nbytes = N * K // 2 + N * K // 2 + N * K * 2 + 4 * N * K // GROUP
+    out = {"shape": [N, K], "bytes": nbytes}
+    for name, calls in [
+        ("reconstruct", [(lambda t=t: ops.latent_w4_reconstruct(t[0], t[1], t[2], t[3], (N, K), *curve)) for t in sets]),
+        ("requant", [(lambda t=t: ops.latent_w4_requant(t[4], t[1], t[2], t[3], (N, K), *curve)) for t in sets]),
+    ]:
+        sec = graph_time(calls)
+        out[name] = {"us": sec * 1e6, "GB/s": nbytes / sec / 1e9, "frac_hbm": nbytes / sec / PEAK_HBM}
+    return out
+
+
 def bench_gemv(device):
     from latentq_llm_amd import ops
     out = []
@@ -346,6 +368,7 @@ def main():
         del blk
         torch.cuda.empty_cache()
         line["requant"] = bench_requant(dev)
+        line["latent_lbit4"] = bench_latent(dev)
         line["gemv"] = bench_gemv(dev)
         line["a8w8"] = bench_a8w8(dev)
         line["hbm_copy"] = bench_copy(dev)

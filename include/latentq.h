@@ -143,6 +143,25 @@ int lq_residual_dequant(const int32_t *q, void *x_out, int64_t n_words, int mode
                         float b2, int k3, void *stream);
 
 /* ---------------------------------------------------------------------------
+ * Fused latent-weight passes of the A16W4 layer in its 4-bit-residual mode (lbit = 4), three-segment
+ * codec with the parameters of lq_residual_quant. Each is one pass instead of a chain of bf16
+ * tensor operations around the codec kernel, with the chain's rounding points kept (bit-identical).
+ *   lq_latent_w4_reconstruct: latent = bf16(bf16(value(nibble) * s) + bf16(bf16(q - z) * s))
+ *     replaces ResidualTensor.add(DeQfunc_4bit_g(...)), utils/quant.py:66-72, 826-837, 1066-1079.
+ *   lq_latent_w4_requant: Z = bf16(bf16(t / s) + z), q = rint(Z), residual nibble and carry from
+ *     bf16(Z - q), code = clamp(q + carry, 0, 15); replaces Qfunc_4bit_g_res + ResidualTensor.set_value,
+ *     utils/quant.py:45-63, 803-811.
+ * codes: native layout; residual: int32[N*K/8], first element in the top nibble; latent: bf16[N,K];
+ * all three 16-byte aligned. A NaN in the latent gives code 0 (the tensor-op chain leaves it undefined).
+ * ------------------------------------------------------------------------- */
+int lq_latent_w4_reconstruct(const void *codes, const void *scales, const void *zeros, const int32_t *residual,
+                             void *latent_out, int64_t N, int64_t K, int group, int k1, float b1, int k2, float b2,
+                             int k3, void *stream);
+int lq_latent_w4_requant(const void *latent, const void *scales, const void *zeros, void *codes_out,
+                         int32_t *residual_out, int64_t N, int64_t K, int group, int k1, float b1, int k2, float b2,
+                         int k3, void *stream);
+
+/* ---------------------------------------------------------------------------
  * Layout converters (device side).
  * GPTQ layout (reference PTQ/quant/quant_linear.py:343-389): qweight is
  * int32[K/8, N] with code(k, n) at bits 4*(k%8) of word [k/8, n].

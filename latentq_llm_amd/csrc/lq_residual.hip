@@ -11,41 +11,9 @@
 // here with fmaf. Layout of the work differs: a thread moves 16 bytes in and out instead of
 // eight 2-byte accesses.
 #include "lq_common.h"
+#include "lq_residual_codec.h"
 
 namespace {
-
-struct CodecParams {
-    float c1, c2, c3;  // forward slopes (quant) or inverse slopes (dequant)
-    float b1, b2;
-    int t1, t2;
-};
-
-__device__ __forceinline__ float level_3fold(float x, const CodecParams &p) {
-    const float S = fabsf(x);
-    float v = fmaf(S, 499.0f, 0.0f);
-    v -= roundf(v);
-    if (S < p.b1) return roundf(fmaf(x, p.c1, v));
-    float r;
-    if (S < p.b2) r = roundf(fmaf(S - p.b1, p.c2, v)) + (float)p.t1;
-    else r = roundf(fmaf(S - p.b2, p.c3, v)) + (float)p.t2;
-    return x < 0.0f ? -r : r;
-}
-
-__device__ __forceinline__ float level_uniform(float x) {
-    const float S = fabsf(x);
-    float v = fmaf(S, 499.0f, 0.0f);
-    v = roundf(v) - v;
-    return roundf(fmaf(x, 8.0f, v));
-}
-
-// float level -> (nibble, carry). Negative values below -8 saturate to nibble 0 like the
-// float->unsigned conversion of the reference's target.
-__device__ __forceinline__ unsigned nibble_of(float lv, bool &carry) {
-    carry = lv > 7.5f;
-    if (carry) return 1u;
-    const float t = lv + 8.0f;
-    return t > 0.0f ? ((unsigned)t & 0xFu) : 0u;
-}
 
 template <int MODE>  // 0: three-segment companding, 1: uniform with dither
 __global__ __launch_bounds__(256) void residual_quant_kernel(u32x4_t *__restrict__ x, unsigned *__restrict__ q,
@@ -81,19 +49,7 @@ __global__ __launch_bounds__(256) void residual_dequant_kernel(const unsigned *_
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
         const int s = (int)((word >> (28 - 4 * k)) & 0xFu) - 8;
-        if (MODE == 1) {
-            v[k] = (float)s * 0.125f;
-        } else if (s < -p.t2) {
-            v[k] = fmaf((float)(s + p.t2), p.c3, -p.b2);
-        } else if (s < -p.t1) {
-            v[k] = fmaf((float)(s + p.t1), p.c2, -p.b1);
-        } else if (s <= p.t1) {
-            v[k] = (float)s * p.c1;
-        } else if (s <= p.t2) {
-            v[k] = fmaf((float)(s - p.t1), p.c2, p.b1);
-        } else {
-            v[k] = fmaf((float)(s - p.t2), p.c3, p.b2);
-        }
+        v[k] = MODE == 1 ? (float)s * 0.125f : value_3fold(s, p);
     }
     u32x4_t out;
 #pragma unroll
@@ -120,12 +76,7 @@ extern "C" int lq_residual_quant(void *x_inout, int32_t *q_out, int64_t n_words,
     int rc = check("lq_residual_quant", x_inout, q_out, n_words, mode, k1, b1, k2, b2, k3);
     if (rc) return rc;
     CodecParams p = {};
-    if (mode == 0) {
-        p.c1 = (float)k1 / b1;
-        p.c2 = (float)k2 / (b2 - b1);
-        p.c3 = (float)((double)k3 / (0.5 - (double)b2));
-        p.b1 = b1; p.b2 = b2; p.t1 = k1; p.t2 = k1 + k2;
-    }
+    if (mode == 0) p = lq_codec_quant_params(k1, b1, k2, b2, k3);
     const unsigned blocks = (unsigned)((n_words + 255) / 256);
     if (mode == 0)
         hipLaunchKernelGGL(residual_quant_kernel<0>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (u32x4_t *)x_inout,
@@ -141,12 +92,7 @@ extern "C" int lq_residual_dequant(const int32_t *q, void *x_out, int64_t n_word
     int rc = check("lq_residual_dequant", x_out, q, n_words, mode, k1, b1, k2, b2, k3);
     if (rc) return rc;
     CodecParams p = {};
-    if (mode == 0) {
-        p.c1 = b1 / (float)k1;
-        p.c2 = (b2 - b1) / (float)k2;
-        p.c3 = (float)((0.5 - (double)b2) / (double)k3);
-        p.b1 = b1; p.b2 = b2; p.t1 = k1; p.t2 = k1 + k2;
-    }
+    if (mode == 0) p = lq_codec_dequant_params(k1, b1, k2, b2, k3);
     const unsigned blocks = (unsigned)((n_words + 255) / 256);
     if (mode == 0)
         hipLaunchKernelGGL(residual_dequant_kernel<0>, dim3(blocks), dim3(256), 0, (hipStream_t)stream,

@@ -206,3 +206,36 @@ def residual_dequant(q, mode: int, k1=0, b1=0.0, k2=0, b2=0.0, k3=0):
         _C.call("lq_residual_dequant", q.data_ptr(), x.data_ptr(), q.numel(), mode, k1, float(b1), k2, float(b2), k3,
                 _stream(q))
     return x
+
+
+def latent_w4_reconstruct(codes, scales, zeros, residual_int, shape, k1, b1, k2, b2, k3):
+    """Latent weight of an A16W4 layer with a 4-bit residual: dequantised codes + dequantised residual * scale,
+    with the bf16 rounding points of the reference's tensor-op chain. Returns bf16 [N, K]."""
+    N, K = shape
+    _codes_ok(codes, N, K)
+    _qparam_ok(scales, zeros, N, K)
+    _chk(residual_int, torch.int32, "residual_int")
+    if residual_int.numel() != N * K // 8:
+        raise ValueError("residual_int must hold N*K/8 words")
+    out = torch.empty((N, K), dtype=torch.bfloat16, device=codes.device)
+    with torch.cuda.device(codes.device):
+        _C.call("lq_latent_w4_reconstruct", codes.data_ptr(), scales.data_ptr(), zeros.data_ptr(), residual_int.data_ptr(),
+                out.data_ptr(), N, K, 128, int(k1), float(b1), int(k2), float(b2), int(k3), _stream(codes))
+    return out
+
+
+def latent_w4_requant(latent, scales, zeros, residual_int, shape, k1, b1, k2, b2, k3):
+    """Re-quantise a bf16 latent weight: returns the packed codes and overwrites residual_int (int32[N*K/8])."""
+    N, K = shape
+    _chk(latent, torch.bfloat16, "latent")
+    if latent.numel() != N * K:
+        raise ValueError("latent must hold N*K elements")
+    _qparam_ok(scales, zeros, N, K)
+    _chk(residual_int, torch.int32, "residual_int")
+    if residual_int.numel() != N * K // 8:
+        raise ValueError("residual_int must hold N*K/8 words")
+    codes = torch.empty(N * K // 2, dtype=torch.int8, device=latent.device)
+    with torch.cuda.device(latent.device):
+        _C.call("lq_latent_w4_requant", latent.data_ptr(), scales.data_ptr(), zeros.data_ptr(), codes.data_ptr(),
+                residual_int.data_ptr(), N, K, 128, int(k1), float(b1), int(k2), float(b2), int(k3), _stream(latent))
+    return codes

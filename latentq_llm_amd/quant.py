@@ -32,6 +32,10 @@ import torch.nn as nn
 from . import ops
 
 GROUPSIZE = 128  # utils/quant.py:44
+# lbit = 4 latent passes (codes + residual -> latent, latent -> codes + residual) as single HIP
+# kernels; False runs the reference's chain of tensor operations around the codec kernel instead
+# (same bits either way).
+FUSED_LATENT = True
 EXT_type = torch.bfloat16  # utils/quant.py:722
 
 # dW travels from the autograd Functions to the full-backward hook through this list
@@ -103,6 +107,17 @@ def Qfunc_4bit_g_res(tensor, residual_handle, qparam, groupsize=GROUPSIZE):
     scales, zeros, shape = qparam
     scales = scales.contiguous().reshape(-1, 1)
     zeros = zeros.contiguous().reshape(-1, 1)
+    if (FUSED_LATENT and isinstance(residual_handle, ResidualTensor) and groupsize == GROUPSIZE and tensor.is_cuda
+            and tensor.dtype == torch.bfloat16 and scales.dtype == torch.bfloat16 and zeros.dtype == torch.bfloat16
+            and residual_handle.residual_int.is_cuda):
+        # one HIP pass with the rounding points of the chain below (lq_latent_w4_requant)
+        p1, y1, p2, y2 = three_fold_curve_4bit(residual_handle.mu)
+        codes = ops.latent_w4_requant(tensor.data.contiguous(), scales, zeros, residual_handle.residual_int.view(-1),
+                                      tuple(shape), p1, y1, p2 - p1, y2, 8 - p2)
+        residual_handle.weight_scale = scales
+        residual_handle.lock_mu = residual_handle.mu
+        residual_handle.init = False
+        return codes
     t = tensor.data.view(-1, groupsize)
     Z = t / scales + zeros
     q = torch.round(Z)
@@ -885,6 +900,15 @@ class MyAdam(torch.optim.Adam):
             if p.wbit == 8:
                 return p.residual.add((p.data * p.qparam).to(dtype))
             if p.wbit == 4:
+                r = p.residual
+                scales, zeros, shape = _flat_qparam(p.qparam)
+                if (FUSED_LATENT and not r.init and dtype == torch.bfloat16 and p.data.is_cuda
+                        and scales.dtype == torch.bfloat16 and zeros.dtype == torch.bfloat16
+                        and r.weight_scale is not None and r.weight_scale.dtype == torch.bfloat16
+                        and r.weight_scale.data_ptr() == scales.data_ptr() and r.weight_scale.numel() == scales.numel()):
+                    p1, y1, p2, y2 = three_fold_curve_4bit(r.lock_mu)
+                    return ops.latent_w4_reconstruct(p.data.contiguous(), scales, zeros, r.residual_int.view(-1),
+                                                     tuple(shape), p1, y1, p2 - p1, y2, 8 - p2)
                 return p.residual.add(DeQfunc_4bit_g(p.data, p.qparam, dtype))
             raise AssertionError("wbit must be 4 or 8")
         return p.residual.data.to(dtype)

@@ -110,3 +110,36 @@ def a8w8_backward(dy, x8, clampv, w8, qscales):
     xf = x8.to(dy.dtype) * (clampv / 127.)
     wf = w8.to(dy.dtype) * qscales
     return dy.mm(wf), dy.t().mm(xf)
+
+
+@torch.no_grad()
+def latent_w4_reconstruct(packed, scales, zeros, residual_int, shape, curve):
+    """Latent weight in lbit=4 mode, the reference's chain on CPU tensors: DeQfunc_4bit_g
+    (utils/quant.py:66-72) + ResidualTensor.add (utils/quant.py:826-837) with the residual decoded
+    by the C restatement of the codec. curve = (p1, y1, p2, y2) of three_fold_curve_4bit."""
+    import numpy as np
+    from . import c_oracle as co
+    p1, y1, p2, y2 = curve
+    w = dequant_4bit_g(packed, scales, zeros, shape)                      # bf16
+    r_bits = co.residual_dequant(residual_int.numpy().view(np.uint32), 0, p1, y1, p2 - p1, y2, 8 - p2)
+    r = torch.from_numpy(r_bits.view(np.int16).copy()).view(torch.bfloat16)
+    r = (r.view(-1, 128) * scales.reshape(-1, 1)).to(torch.bfloat16)       # bf16 * bf16 -> bf16
+    return r.view(shape).add(w.view(shape))
+
+
+@torch.no_grad()
+def latent_w4_requant(latent, scales, zeros, shape, curve):
+    """Qfunc_4bit_g_res with a ResidualTensor handle (utils/quant.py:45-63, 803-811) on CPU tensors.
+    Returns (packed codes int8, residual words int32)."""
+    import numpy as np
+    from . import c_oracle as co
+    p1, y1, p2, y2 = curve
+    t = latent.view(-1, 128)
+    Z = t / scales.reshape(-1, 1) + zeros.reshape(-1, 1)
+    q = torch.round(Z)
+    f = (Z - q).to(torch.bfloat16).contiguous()
+    words, carry_bits = co.residual_quant(f.view(torch.int16).numpy().view(np.uint16), 0, p1, y1, p2 - p1, y2, 8 - p2)
+    carry = torch.from_numpy(carry_bits.view(np.int16).copy()).view(torch.bfloat16).view(shape)
+    q = q.view(shape) + carry
+    codes = compress(torch.clamp(q, 0, 15).to(torch.uint8))
+    return codes, torch.from_numpy(words.view(np.int32).copy())

@@ -1,0 +1,103 @@
+"""Fused lbit=4 latent passes (lq_latent_w4_reconstruct / lq_latent_w4_requant) through the C ABI,
+bit for bit against (a) the reference's chain of bf16 tensor operations run by torch on the CPU
+around the C restatement of the residual codec (oracle/torch_ref.py) and (b) this package's own
+unfused module path on the GPU, including whole optimizer steps."""
+import numpy as np
+import pytest
+import torch
+
+from tests.util import make_w4, randn_bf16
+
+pytestmark = pytest.mark.gpu
+
+CURVES = {0: (2, 0.125, 4, 0.25), 1: (2, 0.2666300266320331, 4, 0.375), 2: (2, 0.37272211741724515, 4, 0.4375),
+          3: (2, 0.4330623539159437, 4, 0.46875)}
+
+
+@pytest.fixture(scope="module")
+def ops(hip_lib):
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from latentq_llm_amd import ops as _ops
+    return _ops
+
+
+@pytest.mark.parametrize("mu", [0, 1, 2, 3])
+@pytest.mark.parametrize("N,K", [(8, 128), (40, 384), (256, 1024)])
+def test_reconstruct_matches_the_tensor_op_chain(ops, N, K, mu):
+    from oracle import torch_ref as tr
+    p1, y1, p2, y2 = CURVES[mu]
+    codes, packed, scales, zeros = make_w4(N, K, N + K + mu)
+    g = torch.Generator().manual_seed(mu + 1)
+    residual = torch.randint(-2 ** 31, 2 ** 31 - 1, (N * K // 8,), generator=g, dtype=torch.int64).to(torch.int32)
+    want = tr.latent_w4_reconstruct(packed, scales, zeros, residual, (N, K), CURVES[mu])
+    got = ops.latent_w4_reconstruct(packed.cuda(), scales.cuda(), zeros.cuda(), residual.cuda(), (N, K),
+                                    p1, y1, p2 - p1, y2, 8 - p2)
+    assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("mu", [0, 1, 2, 3])
+@pytest.mark.parametrize("N,K", [(8, 128), (40, 384), (256, 1024)])
+def test_requant_matches_the_tensor_op_chain(ops, N, K, mu):
+    from oracle import torch_ref as tr
+    p1, y1, p2, y2 = CURVES[mu]
+    codes, packed, scales, zeros = make_w4(N, K, N + K + mu)
+    # a latent that covers the whole code range, exact half-way points, carries and both clamps
+    w = tr.dequant_4bit_g(packed, scales, zeros, (N, K)).float()
+    s = scales.float().reshape(N, K // 128, 1).expand(N, K // 128, 128).reshape(N, K)
+    noise = torch.rand((N, K), generator=torch.Generator().manual_seed(3)) - 0.5
+    latent = w + noise * s * 1.2
+    latent.view(-1)[::37] = (w + 0.5 * s).view(-1)[::37]
+    latent.view(-1)[5::101] = (w + 40.0 * s).view(-1)[5::101]
+    latent.view(-1)[7::103] = (w - 40.0 * s).view(-1)[7::103]
+    latent = latent.to(torch.bfloat16)
+    want_codes, want_res = tr.latent_w4_requant(latent, scales, zeros, (N, K), CURVES[mu])
+    res = torch.empty(N * K // 8, dtype=torch.int32, device="cuda")
+    got = ops.latent_w4_requant(latent.cuda(), scales.cuda(), zeros.cuda(), res, (N, K), p1, y1, p2 - p1, y2, 8 - p2)
+    assert torch.equal(got.cpu().view(torch.uint8), want_codes.view(torch.uint8))
+    assert torch.equal(res.cpu(), want_res)
+    # and back: the reconstruction of what was just stored is close to the input (one residual step plus the
+    # bf16 rounding of the latent itself, both well below a quarter of a code step)
+    back = ops.latent_w4_reconstruct(got, scales.cuda(), zeros.cuda(), res, (N, K), p1, y1, p2 - p1, y2, 8 - p2)
+    inside = (latent.float() >= (0 - zeros.float().reshape(N, -1, 1).expand(N, K // 128, 128).reshape(N, K)) * s) & \
+             (latent.float() <= (15 - zeros.float().reshape(N, -1, 1).expand(N, K // 128, 128).reshape(N, K)) * s)
+    err = ((back.float().cpu() - latent.float()).abs() / s)[inside]
+    assert float(err.max()) <= 0.25, float(err.max())
+
+
+def _run_steps(Q, fused, steps=4):
+    Q.FUSED_LATENT = fused
+    torch.manual_seed(0)
+    N, K = 128, 256
+    codes, packed, scales, zeros = make_w4(N, K, 9)
+    layer = Q.QLinearA16W4(K, N, bias=False, lbit=4, gbit=16)
+    layer.zeros.data = zeros.clone()
+    layer.scales.data = scales.clone()
+    layer.weight.set_value(packed.clone(), [layer.scales, layer.zeros, layer.wshape])
+    layer.to("cuda")
+    layer.add_hook()
+    opt = Q.MyAdam([{"params": [layer.weight]}], lr=2e-3, betas=(0.9, 0.999), obit=16, mu_updata_f=20)
+    x = randn_bf16((64, K), 11).cuda().requires_grad_(True)
+    tgt = randn_bf16((64, N), 12).cuda()
+    for _ in range(steps):
+        y = layer(x)
+        ((y.float() - tgt.float()) ** 2).mean().backward()
+        opt.step()
+    return layer.weight.data.clone().cpu(), layer.weight.residual.residual_int.clone().cpu()
+
+
+def test_optimizer_steps_fused_equals_unfused(hip_lib, monkeypatch):
+    from latentq_llm_amd import ops as O
+    from latentq_llm_amd import quant as Q
+    calls = {"reconstruct": 0, "requant": 0}
+    rec, req = O.latent_w4_reconstruct, O.latent_w4_requant
+    monkeypatch.setattr(O, "latent_w4_reconstruct", lambda *a, **k: (calls.__setitem__("reconstruct", calls["reconstruct"] + 1), rec(*a, **k))[1])
+    monkeypatch.setattr(O, "latent_w4_requant", lambda *a, **k: (calls.__setitem__("requant", calls["requant"] + 1), req(*a, **k))[1])
+    try:
+        c1, r1 = _run_steps(Q, True)
+        assert calls == {"reconstruct": 3, "requant": 4}  # the first step has no stored residual yet
+        c0, r0 = _run_steps(Q, False)
+        assert calls == {"reconstruct": 3, "requant": 4}
+    finally:
+        Q.FUSED_LATENT = True
+    assert torch.equal(c1, c0) and torch.equal(r1, r0)
+    assert not torch.equal(c1, make_w4(128, 256, 9)[1])  # the steps did move the weights
