@@ -48,24 +48,27 @@ typedef const __attribute__((address_space(1))) void gbl_void;
 constexpr int kUnroll = 4;       // groups per batch (scale/zero batches are 4 x bf16 = 8 bytes)
 constexpr int kXRow = 1024 + 16;  // LDS bytes per staged token row: 4 groups x 256 B, padded against bank conflicts
 
-// MP = number of token rows staged per wave and batch (>= M).
-template <int WAVES, int MP>
+// MP = number of token rows staged per wave and batch (>= M). NT = 16-row weight tiles per
+// workgroup: every workgroup stages the activations of its K range again, so with many tokens two
+// tiles per workgroup halve that traffic (and share the activation-sum MFMAs).
+template <int WAVES, int MP, int NT>
 __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *__restrict__ x,
                                                           const unsigned char *__restrict__ codes,
                                                           const unsigned short *__restrict__ scales,
                                                           const unsigned short *__restrict__ zeros,
                                                           const unsigned short *__restrict__ bias,
                                                           unsigned short *__restrict__ y, int M, int N, int K) {
-    __shared__ float red[WAVES][4][64];
+    __shared__ float red[WAVES][NT][4][64];
     __shared__ __attribute__((aligned(16))) unsigned char xs[WAVES][MP][kXRow];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // scalar: uniform control flow
     const int n = lane & 15, kq = lane >> 4;
-    const int row = blockIdx.x * 16 + n;  // weight row of this lane's B fragment
+    const int row = blockIdx.x * (16 * NT) + n;  // weight row of this lane's B fragment in tile 0 (tile j: + 16 j)
     const int G = K / LQ_GROUP;
 
     // load layout of the codes: lane 4*r + c -> row r of this block, 16-byte chunk c of the group
-    const unsigned char *wrow = codes + (long long)(blockIdx.x * 16 + (lane >> 2)) * (K / 2) + (lane & 3) * 16;
+    const unsigned char *wrow = codes + (long long)(blockIdx.x * (16 * NT) + (lane >> 2)) * (K / 2) + (lane & 3) * 16;
+    const long long tile_stride = 16ll * (K / 2);  // bytes between the same row of consecutive tiles
     const int bperm_src = (4 * n + kq) * 4;  // ds_bpermute: take from lane 4*n + kq
     const int bcast_src = n * 4;             // ds_bpermute: take from lane n (kq = 0)
     const unsigned short *srow = scales + (long long)row * G;
@@ -75,7 +78,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
     const unsigned char *xfrag = &xs[wave][n < M ? n : M - 1][kq * 64];
 
     const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    f32x4_t acc[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     for (int g0 = wave * kUnroll; g0 < G; g0 += WAVES * kUnroll) {
         const bool full = g0 + kUnroll <= G;  // a short tail batch re-reads the last group with zero scale
@@ -92,82 +97,104 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
                                                      (lds_void *)&xs[wave][m][0], 16, 0, 0);
         }
         // ---- codes, scales, zeros
-        u32x4_t wv[kUnroll];
-        float sc[kUnroll], zz[kUnroll];
-        u32x2_t sraw = {0u, 0u}, zraw = {0u, 0u};
+        u32x4_t wv[NT][kUnroll];
+        float sc[NT][kUnroll], zz[NT][kUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const int g = g0 + u < G ? g0 + u : G - 1;
-            wv[u] = *reinterpret_cast<const u32x4_t *>(wrow + g * 64);
-        }
-        if (full) {
-            if (kq == 0) {
-                sraw = *reinterpret_cast<const u32x2_t *>(srow + g0);
-                zraw = *reinterpret_cast<const u32x2_t *>(zrow + g0);
-            }
-            unsigned s01 = (unsigned)__builtin_amdgcn_ds_bpermute(bcast_src, (int)sraw[0]);
-            unsigned s23 = (unsigned)__builtin_amdgcn_ds_bpermute(bcast_src, (int)sraw[1]);
-            unsigned z01 = (unsigned)__builtin_amdgcn_ds_bpermute(bcast_src, (int)zraw[0]);
-            unsigned z23 = (unsigned)__builtin_amdgcn_ds_bpermute(bcast_src, (int)zraw[1]);
-            sc[0] = lq_bf16_lo(s01); sc[1] = lq_bf16_hi(s01); sc[2] = lq_bf16_lo(s23); sc[3] = lq_bf16_hi(s23);
-            zz[0] = 128.0f + lq_bf16_lo(z01); zz[1] = 128.0f + lq_bf16_hi(z01);
-            zz[2] = 128.0f + lq_bf16_lo(z23); zz[3] = 128.0f + lq_bf16_hi(z23);
-        } else {
+        for (int j = 0; j < NT; ++j)
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) {
-                const bool live = g0 + u < G;
-                const int g = live ? g0 + u : G - 1;
-                sc[u] = live ? lq_bf16_bits_to_f32(srow[g]) : 0.0f;
-                zz[u] = 128.0f + lq_bf16_bits_to_f32(zrow[g]);
+                const int g = g0 + u < G ? g0 + u : G - 1;
+                wv[j][u] = *reinterpret_cast<const u32x4_t *>(wrow + j * tile_stride + g * 64);
+            }
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const unsigned short *sr = srow + (long long)j * 16 * G, *zr = zrow + (long long)j * 16 * G;
+            if (full) {
+                u32x2_t sraw = {0u, 0u}, zraw = {0u, 0u};
+                if (kq == 0) {
+                    sraw = *reinterpret_cast<const u32x2_t *>(sr + g0);
+                    zraw = *reinterpret_cast<const u32x2_t *>(zr + g0);
+                }
+                unsigned s01 = (unsigned)__builtin_amdgcn_ds_bpermute(bcast_src, (int)sraw[0]);
+                unsigned s23 = (unsigned)__builtin_amdgcn_ds_bpermute(bcast_src, (int)sraw[1]);
+                unsigned z01 = (unsigned)__builtin_amdgcn_ds_bpermute(bcast_src, (int)zraw[0]);
+                unsigned z23 = (unsigned)__builtin_amdgcn_ds_bpermute(bcast_src, (int)zraw[1]);
+                sc[j][0] = lq_bf16_lo(s01); sc[j][1] = lq_bf16_hi(s01); sc[j][2] = lq_bf16_lo(s23); sc[j][3] = lq_bf16_hi(s23);
+                zz[j][0] = 128.0f + lq_bf16_lo(z01); zz[j][1] = 128.0f + lq_bf16_hi(z01);
+                zz[j][2] = 128.0f + lq_bf16_lo(z23); zz[j][3] = 128.0f + lq_bf16_hi(z23);
+            } else {
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) {
+                    const bool live = g0 + u < G;
+                    const int g = live ? g0 + u : G - 1;
+                    sc[j][u] = live ? lq_bf16_bits_to_f32(sr[g]) : 0.0f;
+                    zz[j][u] = 128.0f + lq_bf16_bits_to_f32(zr[g]);
+                }
             }
         }
         // ---- codes to the MFMA lane layout
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
+        for (int j = 0; j < NT; ++j)
 #pragma unroll
-            for (int t = 0; t < 4; ++t) wv[u][t] = (unsigned)__builtin_amdgcn_ds_bpermute(bperm_src, (int)wv[u][t]);
+            for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    wv[j][u][t] = (unsigned)__builtin_amdgcn_ds_bpermute(bperm_src, (int)wv[j][u][t]);
         // ---- MFMAs, step index outermost so that consecutive MFMAs feed different accumulators
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the staged rows have landed in LDS
-        f32x4_t P[kUnroll], S[kUnroll];
+        f32x4_t P[NT][kUnroll], S[kUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) P[u] = S[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int u = 0; u < kUnroll; ++u) {
+            S[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < NT; ++j) P[j][u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) {
-                unsigned b[4], a[4];
-                unpack_word_128q(wv[u][t], b);
+                unsigned a[4];
                 const u32x4_t xv = *reinterpret_cast<const u32x4_t *>(xfrag + u * 256 + t * 16);
                 permute_x(xv, a);
                 const u32x4_t av = {a[0], a[1], a[2], a[3]};
-                const u32x4_t bv = {b[0], b[1], b[2], b[3]};
-                P[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
-                                                               __builtin_bit_cast(bf16x8_t, bv), P[u], 0, 0, 0);
                 S[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
                                                                __builtin_bit_cast(bf16x8_t, ones), S[u], 0, 0, 0);
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    unsigned b[4];
+                    unpack_word_128q(wv[j][u][t], b);
+                    const u32x4_t bv = {b[0], b[1], b[2], b[3]};
+                    P[j][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                                      __builtin_bit_cast(bf16x8_t, bv), P[j][u], 0, 0, 0);
+                }
             }
         }
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
+        for (int j = 0; j < NT; ++j)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) acc[r] = fmaf(sc[u], fmaf(-zz[u], S[u][r], P[u][r]), acc[r]);
+            for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[j][r] = fmaf(sc[j][u], fmaf(-zz[j][u], S[u][r], P[j][u][r]), acc[j][r]);
         // the next batch overwrites the staged rows: all fragment reads above must have returned
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
 
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][r][lane] = acc[r];
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[wave][j][r][lane] = acc[j][r];
     __syncthreads();
-    if (wave == 0) {
-        // lane holds D[m = 4*kq + r][n]
-        const float b = bias ? lq_bf16_bits_to_f32(bias[row]) : 0.0f;
+    if (wave < NT) {
+        // wave j finishes tile j; lane holds D[m = 4*kq + r][n]
+        const int orow = row + 16 * wave;
+        const float b = bias ? lq_bf16_bits_to_f32(bias[orow]) : 0.0f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             float v = 0.f;
 #pragma unroll
-            for (int w = 0; w < WAVES; ++w) v += red[w][r][lane];
+            for (int w = 0; w < WAVES; ++w) v += red[w][wave][r][lane];
             const int m = 4 * kq + r;
-            if (m < M) y[(long long)m * N + row] = lq_f32_to_bf16_bits(v + b);
+            if (m < M) y[(long long)m * N + orow] = lq_f32_to_bf16_bits(v + b);
         }
     }
 }
@@ -177,24 +204,28 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
 int lq_gemv_a16w4_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
                          void *y, int M, int N, int K, hipStream_t st) {
     // N % 16 == 0, K % 128 == 0 and 1 <= M <= 16 are guaranteed by the caller.
-    const int blocks = N / 16;
     const int G = K / LQ_GROUP;
     // One batch of 4 groups per wave when possible: all of a wave's loads are then in flight at once.
     // With 16 staged token rows a wave needs 16.25 KB of LDS, which caps the workgroup at 8 waves.
-#define LQ_GEMV_LAUNCH(W, MP)                                                                                     \
-    hipLaunchKernelGGL((gemv_kernel<W, MP>), dim3(blocks), dim3(64 * W), 0, st, (const unsigned short *)x,         \
+#define LQ_GEMV_LAUNCH(W, MP, NT)                                                                                  \
+    hipLaunchKernelGGL((gemv_kernel<W, MP, NT>), dim3(N / (16 * NT)), dim3(64 * W), 0, st, (const unsigned short *)x, \
                        (const unsigned char *)codes, (const unsigned short *)scales, (const unsigned short *)zeros, \
                        (const unsigned short *)bias, (unsigned short *)y, M, N, K)
     const int want = (G + 3) / 4;  // waves for one batch each
     if (M <= 4) {
-        if (want <= 2) LQ_GEMV_LAUNCH(2, 4);
-        else if (want <= 4) LQ_GEMV_LAUNCH(4, 4);
-        else if (want <= 8) LQ_GEMV_LAUNCH(8, 4);
-        else LQ_GEMV_LAUNCH(16, 4);
+        if (want <= 2) LQ_GEMV_LAUNCH(2, 4, 1);
+        else if (want <= 4) LQ_GEMV_LAUNCH(4, 4, 1);
+        else if (want <= 8) LQ_GEMV_LAUNCH(8, 4, 1);
+        else LQ_GEMV_LAUNCH(16, 4, 1);
+    } else if (N % 32 == 0 && N >= 32 * 256) {
+        // many tokens and enough rows for one 32-row workgroup per CU: half the activation traffic
+        // (4 waves = 65 KB of staged activations: two workgroups per CU, all of them resident at once)
+        if (want <= 2) LQ_GEMV_LAUNCH(2, 16, 2);
+        else LQ_GEMV_LAUNCH(4, 16, 2);
     } else {
-        if (want <= 2) LQ_GEMV_LAUNCH(2, 16);
-        else if (want <= 4) LQ_GEMV_LAUNCH(4, 16);
-        else LQ_GEMV_LAUNCH(8, 16);
+        if (want <= 2) LQ_GEMV_LAUNCH(2, 16, 1);
+        else if (want <= 4) LQ_GEMV_LAUNCH(4, 16, 1);
+        else LQ_GEMV_LAUNCH(8, 16, 1);
     }
 #undef LQ_GEMV_LAUNCH
     return lq_check_launch("lq_a16w4_fwd(gemv)");
