@@ -237,6 +237,14 @@ def profile_target(device, which, launches=10):
             p, s, z = synth_w4(N, K, 10 + i, device)
             g = (torch.randn(N, K, device=device) * 1e-3).to(torch.bfloat16)
             o.requant_sr(p, s, z, g, 1e-4, (N, K), seed=7, offset=i)
+    elif which == "latent":
+        N, K = 8192, 2048
+        curve = (2, 0.125, 2, 0.25, 4)
+        for i in range(launches):
+            p, s, z = synth_w4(N, K, 40 + i, device)
+            res = torch.randint(-2 ** 31, 2 ** 31 - 1, (N * K // 8,), device=device, dtype=torch.int64).to(torch.int32)
+            lat = o.latent_w4_reconstruct(p, s, z, res, (N, K), *curve)
+            o.latent_w4_requant(lat, s, z, res, (N, K), *curve)
     elif which == "gemv":
         for (N, K) in [(4096, 4096), (11008, 4096), (4096, 11008)]:
             for M in (1, 4, 16):
@@ -306,7 +314,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-mlp", action="store_true", help="skip the side measurements (requant, GEMV, A8W8)")
-    ap.add_argument("--profile-target", choices=["gemm", "requant", "gemv", "a8w8"],
+    ap.add_argument("--profile-target", choices=["gemm", "requant", "gemv", "a8w8", "latent"],
                     help="run only a short fixed launch sequence of one kernel family (for rocprofv3), print nothing")
     args = ap.parse_args()
     if args.gpus != 1:
