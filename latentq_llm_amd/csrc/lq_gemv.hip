@@ -140,41 +140,39 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
                     wv[j][u][t] = (unsigned)__builtin_amdgcn_ds_bpermute(bperm_src, (int)wv[j][u][t]);
-        // ---- MFMAs, step index outermost so that consecutive MFMAs feed different accumulators
+        // ---- MFMAs
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the staged rows have landed in LDS
-        f32x4_t P[NT][kUnroll], S[kUnroll];
+        // One group at a time: a single pair of MFMA accumulators (plus one per extra tile) is live,
+        // which keeps the kernel at <= 80 registers (6 waves per SIMD, three 8-wave workgroups per
+        // CU); the unpacking between two MFMAs on the same accumulator covers their latency.
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            S[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            f32x4_t P[NT], S = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int j = 0; j < NT; ++j) P[j][u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-        }
+            for (int j = 0; j < NT; ++j) P[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
+            for (int t = 0; t < 4; ++t) {
                 unsigned a[4];
                 const u32x4_t xv = *reinterpret_cast<const u32x4_t *>(xfrag + u * 256 + t * 16);
                 permute_x(xv, a);
                 const u32x4_t av = {a[0], a[1], a[2], a[3]};
-                S[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
-                                                               __builtin_bit_cast(bf16x8_t, ones), S[u], 0, 0, 0);
+                S = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                            __builtin_bit_cast(bf16x8_t, ones), S, 0, 0, 0);
 #pragma unroll
                 for (int j = 0; j < NT; ++j) {
                     unsigned b[4];
                     unpack_word_128q(wv[j][u][t], b);
                     const u32x4_t bv = {b[0], b[1], b[2], b[3]};
-                    P[j][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
-                                                                      __builtin_bit_cast(bf16x8_t, bv), P[j][u], 0, 0, 0);
+                    P[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                                   __builtin_bit_cast(bf16x8_t, bv), P[j], 0, 0, 0);
                 }
             }
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[j][r] = fmaf(sc[j][u], fmaf(-zz[j][u], S[r], P[j][r]), acc[j][r]);
+            __builtin_amdgcn_sched_barrier(0);  // keeps the next group's unpacking from being hoisted (registers)
         }
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) acc[j][r] = fmaf(sc[j][u], fmaf(-zz[j][u], S[u][r], P[j][u][r]), acc[j][r]);
         // the next batch overwrites the staged rows: all fragment reads above must have returned
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
@@ -201,32 +199,58 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
 
 }  // namespace
 
+namespace {
+
+struct GemvArgs {
+    const void *x, *codes, *scales, *zeros, *bias;
+    void *y;
+    int M, N, K;
+    hipStream_t st;
+};
+
+template <int W, int MP, int NT>
+void launch_one(const GemvArgs &a) {
+    hipLaunchKernelGGL((gemv_kernel<W, MP, NT>), dim3(a.N / (16 * NT)), dim3(64 * W), 0, a.st, (const unsigned short *)a.x,
+                       (const unsigned char *)a.codes, (const unsigned short *)a.scales, (const unsigned short *)a.zeros,
+                       (const unsigned short *)a.bias, (unsigned short *)a.y, a.M, a.N, a.K);
+}
+
+// Waves per workgroup: as many as there are batches, up to the cap, in powers of two. More waves
+// mean more of the matrix in flight at once, which matters more than an even split of the batches
+// (K = 11008 = 22 batches: 16 waves, 6 of them with two batches, beat 11 waves x 2).
+int pick_waves(int batches, int max_waves) {
+    int w = 2;
+    while (w < batches && w < max_waves) w *= 2;
+    return w;
+}
+
+template <int MP, int NT, int MAXW>
+void launch_waves(int w, const GemvArgs &a) {
+    switch (w) {
+        case 2: launch_one<2, MP, NT>(a); break;
+        case 4: launch_one<4, MP, NT>(a); break;
+        case 8: if constexpr (MAXW >= 8) launch_one<8, MP, NT>(a); break;
+        default: launch_one<MAXW, MP, NT>(a); break;
+    }
+}
+
+}  // namespace
+
 int lq_gemv_a16w4_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
                          void *y, int M, int N, int K, hipStream_t st) {
     // N % 16 == 0, K % 128 == 0 and 1 <= M <= 16 are guaranteed by the caller.
-    const int G = K / LQ_GROUP;
-    // One batch of 4 groups per wave when possible: all of a wave's loads are then in flight at once.
-    // With 16 staged token rows a wave needs 16.25 KB of LDS, which caps the workgroup at 8 waves.
-#define LQ_GEMV_LAUNCH(W, MP, NT)                                                                                  \
-    hipLaunchKernelGGL((gemv_kernel<W, MP, NT>), dim3(N / (16 * NT)), dim3(64 * W), 0, st, (const unsigned short *)x, \
-                       (const unsigned char *)codes, (const unsigned short *)scales, (const unsigned short *)zeros, \
-                       (const unsigned short *)bias, (unsigned short *)y, M, N, K)
-    const int want = (G + 3) / 4;  // waves for one batch each
+    const GemvArgs a = {x, codes, scales, zeros, bias, y, M, N, K, st};
+    const int batches = (K / LQ_GROUP + 3) / 4;  // one batch of 4 groups per wave when possible: all of a
+                                                 // wave's loads are then in flight at once
     if (M <= 4) {
-        if (want <= 2) LQ_GEMV_LAUNCH(2, 4, 1);
-        else if (want <= 4) LQ_GEMV_LAUNCH(4, 4, 1);
-        else if (want <= 8) LQ_GEMV_LAUNCH(8, 4, 1);
-        else LQ_GEMV_LAUNCH(16, 4, 1);
+        launch_waves<4, 1, 16>(pick_waves(batches, 16), a);
     } else if (N % 32 == 0 && N >= 32 * 256) {
-        // many tokens and enough rows for one 32-row workgroup per CU: half the activation traffic
-        // (4 waves = 65 KB of staged activations: two workgroups per CU, all of them resident at once)
-        if (want <= 2) LQ_GEMV_LAUNCH(2, 16, 2);
-        else LQ_GEMV_LAUNCH(4, 16, 2);
+        // many tokens and enough rows for one 32-row workgroup per CU: half the activation traffic;
+        // 4 waves = 65 KB of staged activations: two workgroups per CU, all of them resident at once
+        launch_waves<16, 2, 4>(pick_waves(batches, 4), a);
     } else {
-        if (want <= 2) LQ_GEMV_LAUNCH(2, 16, 1);
-        else if (want <= 4) LQ_GEMV_LAUNCH(4, 16, 1);
-        else LQ_GEMV_LAUNCH(8, 16, 1);
+        // 16 staged token rows cost a wave 16.25 KB of LDS, which caps the workgroup at 8 waves
+        launch_waves<16, 1, 8>(pick_waves(batches, 8), a);
     }
-#undef LQ_GEMV_LAUNCH
     return lq_check_launch("lq_a16w4_fwd(gemv)");
 }
