@@ -33,9 +33,17 @@
 // the exact (q - z)*s once; for integer zeros this equals the reference's bf16(bf16(q-z)*s).
 //
 // Pipeline: A tiles are loaded two steps ahead into three LDS stages, codes one step ahead into
-// registers, scales/zeros once per 128-k group. One s_barrier per step, issued without a fence;
-// the LDS-direct loads are inline assembly with explicit s_waitcnt so that they stay in flight
-// across barriers and the compiler's wait insertion never sees them.
+// registers, scales/zeros four groups at a time (8 bytes per row every 8 steps). One s_barrier per
+// step, issued without a fence, three quarters of the way through the step; the last quarter
+// already prepares the first operands of the next step, so the MFMA stream never drains. The
+// global loads are inline assembly with explicit s_waitcnt so that they stay in flight across
+// barriers and the compiler's wait insertion never sees them; they are spread over the step, one
+// kind per half-slice.
+//
+// The chip is power-limited on this kernel (the shader clock sits near 1.35 GHz while it runs,
+// against 2.1 GHz for a loop of MFMAs on constant operands), so what the loop does besides MFMAs
+// costs throughput even where it overlaps them in time: the forms of the loads above are chosen to
+// keep the bytes moved between L2 and the CU near the bytes used.
 #include "lq_common.h"
 
 #include <type_traits>
@@ -112,14 +120,15 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         a_off[i] = (unsigned)((long long)(gr - m0) * lda + chunk * 16);
     }
     const unsigned char *a_base = p.x + (long long)m0 * lda;
-    auto issue_a = [&](int kt, unsigned char *la) {
+    auto issue_a_one = [&](int kt, unsigned char *la, int i) {
         const unsigned char *src = a_base + (long long)kt * ROWB;
+        const unsigned lds_addr = (unsigned)reinterpret_cast<size_t>((lds_void *)(la + (i * 256 + wave * 64) * 16));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :: "s"(lds_addr), "v"(a_off[i]), "s"(src) : "memory");
+    };
+    auto issue_a = [&](int kt, unsigned char *la) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const unsigned lds_addr = (unsigned)reinterpret_cast<size_t>((lds_void *)(la + (i * 256 + wave * 64) * 16));
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                         :: "s"(lds_addr), "v"(a_off[i]), "s"(src) : "memory");
-        }
+        for (int i = 0; i < 4; ++i) issue_a_one(kt, la, i);
     };
 
     // ---- A fragments: row 32j + r, chunk (4h + t) ^ ((r >> 1) & 7)
@@ -161,11 +170,13 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     // its own (it could only wait for everything, LDS-direct loads included); the single
     // s_waitcnt at the end of a step is tied to the loaded registers instead.
     u32x4_t cw[2][NB], cn[2][NB];  // weights of the current and of the next step (int4 codes or int8)
-    unsigned qs[2], qz[2];  // raw bf16 scale / zero of the next group
+    // Raw bf16 scales / zeros of four consecutive groups of the lane's two rows (one 8-byte load per
+    // row every 8 steps: a 2-byte load per group would pull a whole cache line through L1 each time).
+    // The 8-byte loads need 4-byte aligned rows: the launcher requires an even number of groups per row.
+    u32x2_t qs[2], qz[2];
     float s[2], nzs[2];
-    auto load_codes = [&](int kt, u32x4_t (*c)[NB]) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
+    auto load_codes_one = [&](int kt, u32x4_t (*c)[NB], int i) {
+        {
             asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(c[i][0]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
             if constexpr (I8) {
                 asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:16" : "=v"(c[i][1]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
@@ -174,64 +185,116 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
             }
         }
     };
+    auto load_codes = [&](int kt, u32x4_t (*c)[NB]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) load_codes_one(kt, c, i);
+    };
+    // Called on the even step two steps before group g starts; loads when g opens a quad.
+    auto load_qparams_one = [&](int g, int i) {
+        if ((g & 3) != 0) return;
+        asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "=v"(qs[i]) : "v"(q_off[i]), "s"(s_rsrc), "s"(g * 2));
+        asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "=v"(qz[i]) : "v"(q_off[i]), "s"(z_rsrc), "s"(g * 2));
+    };
     auto load_qparams = [&](int g) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            asm volatile("buffer_load_ushort %0, %1, %2, %3 offen" : "=v"(qs[i]) : "v"(q_off[i]), "s"(s_rsrc), "s"(g * 2));
-            asm volatile("buffer_load_ushort %0, %1, %2, %3 offen" : "=v"(qz[i]) : "v"(q_off[i]), "s"(z_rsrc), "s"(g * 2));
-        }
+        for (int i = 0; i < 2; ++i) load_qparams_one(g, i);
     };
-    auto use_qparams = [&]() {
+    auto use_qparams = [&](int g) {
+        const int shift = (g & 3) * 16;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            s[i] = __uint_as_float(qs[i] << 16);
-            nzs[i] = -(__uint_as_float(qz[i] << 16) * s[i]);
+            const unsigned long long s4 = ((unsigned long long)qs[i][1] << 32) | qs[i][0];
+            const unsigned long long z4 = ((unsigned long long)qz[i][1] << 32) | qz[i][0];
+            s[i] = __uint_as_float((unsigned)(s4 >> shift) << 16);
+            nzs[i] = -(__uint_as_float((unsigned)(z4 >> shift) << 16) * s[i]);
         }
     };
     auto read_a = [&](const unsigned char *la, int t, u32x4_t *af) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) af[j] = *reinterpret_cast<const u32x4_t *>(la + j * 4096 + a_frag[t]);
     };
-    auto deq = [&](int t, u32x4_t *bf) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            if constexpr (I8) {
-                bf[i] = cw[i][t];  // 16 int8 of the lane's row: already the MFMA operand
-                continue;
-            }
+    auto deq_one = [&](const u32x4_t (*c)[NB], int t, u32x4_t *bf, int i) {
+        if constexpr (I8) {
+            bf[i] = c[i][t];  // 16 int8 of the lane's row: already the MFMA operand
+        } else {
             float f[8];
-            lq_dequant_word_f32(cw[i][0][t], s[i], nzs[i], f);
+            lq_dequant_word_f32(c[i][0][t], s[i], nzs[i], f);
             bf[i] = u32x4_t{lq_pack_bf16(f[0], f[1]), lq_pack_bf16(f[2], f[3]), lq_pack_bf16(f[4], f[5]),
                             lq_pack_bf16(f[6], f[7])};
         }
     };
-    auto mfma = [&](const u32x4_t *af, const u32x4_t *bf) {
+    auto mfma_half = [&](const u32x4_t *af, const u32x4_t *bf, int i) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if constexpr (I8)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf[i]),
-                                                                     __builtin_bit_cast(i32x4_t, af[j]), acc[i][j], 0, 0, 0);
-                else
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[i]),
-                                                                       __builtin_bit_cast(bf16x8_t, af[j]), acc[i][j], 0, 0, 0);
+        for (int j = 0; j < 4; ++j)
+            if constexpr (I8)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf[i]),
+                                                                 __builtin_bit_cast(i32x4_t, af[j]), acc[i][j], 0, 0, 0);
+            else
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[i]),
+                                                                   __builtin_bit_cast(bf16x8_t, af[j]), acc[i][j], 0, 0, 0);
     };
 
-    // End of a step (and of the prologue): everything this wave loaded for the next step has
-    // arrived (all but the 4 newest loads, the LDS-direct loads of the tile after it), its fragment
-    // reads have returned: meet the other waves, then make the next step's weights current. The
-    // wait is tied to the registers the assembly loads wrote.
-    auto end_of_step = [&](auto with_qparams) {
+    // The one synchronisation point of a step (and the end of the prologue): everything this wave
+    // loaded has arrived except the NEWEST newest loads, its fragment reads have returned: meet the
+    // other waves. The wait is tied to the registers the assembly loads wrote.
+    auto wait_and_meet = [&](auto newest, auto with_qparams) {
+        constexpr int NEWEST = decltype(newest)::value;
+        (void)cn; (void)qs; (void)qz;  // named outside the constexpr branches so that the lambda captures them
         if constexpr (I8) {
-            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier"
+            asm volatile("s_waitcnt vmcnt(%8) lgkmcnt(0)\n\ts_barrier"
                          : "+v"(cn[0][0]), "+v"(cn[0][1]), "+v"(cn[0][2]), "+v"(cn[0][3]), "+v"(cn[1][0]), "+v"(cn[1][1]),
-                           "+v"(cn[1][2]), "+v"(cn[1][3]) :: "memory");
+                           "+v"(cn[1][2]), "+v"(cn[1][3]) : "n"(NEWEST) : "memory");
         } else if constexpr (decltype(with_qparams)::value != 0) {
-            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier"
-                         : "+v"(cn[0][0]), "+v"(cn[1][0]), "+v"(qs[0]), "+v"(qs[1]), "+v"(qz[0]), "+v"(qz[1]) :: "memory");
+            asm volatile("s_waitcnt vmcnt(%6) lgkmcnt(0)\n\ts_barrier"
+                         : "+v"(cn[0][0]), "+v"(cn[1][0]), "+v"(qs[0]), "+v"(qs[1]), "+v"(qz[0]), "+v"(qz[1]) : "n"(NEWEST) : "memory");
         } else {
-            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" : "+v"(cn[0][0]), "+v"(cn[1][0]) :: "memory");
+            asm volatile("s_waitcnt vmcnt(%2) lgkmcnt(0)\n\ts_barrier" : "+v"(cn[0][0]), "+v"(cn[1][0]) : "n"(NEWEST) : "memory");
+        }
+    };
+
+    // Operands of the first reduction slice of the step about to run; slice 3 of every step
+    // prepares them for the step after it, so the MFMA stream continues across the step boundary.
+    u32x4_t af[2][4], bf[2][2];
+
+    // One reduction step on stage AI with the codes in cw, cut into 8 half-slices of 4 MFMAs (one
+    // column tile x four row tiles of one reduction slice). A half-slice also issues the fragment
+    // reads and the dequantisation its counterpart in the next slice needs, and at most one kind of
+    // global load: a burst of loads would hold the wave at the memory pipeline's queue with its
+    // MFMAs behind it. Load order within a step: next step's codes (half-slices 0, 1), on even steps
+    // the next group's scale and zero (2, 3), the LDS-direct loads of the tile two steps ahead
+    // (4..7). Before half-slice 6 the wave waits for all but the two newest loads, which covers tile
+    // kt+1 and the codes of step kt+1, and meets the other waves; slice 3 then reads the first
+    // fragments of tile kt+1 and dequantises the first words of step kt+1 (on odd steps with the
+    // next group's scale and zero). That barrier also orders this step's reads of stage AI before
+    // the next step's loads into it.
+    auto step = [&](int kt, auto ai, auto odd) {
+        constexpr int AI = decltype(ai)::value;
+        constexpr bool ODD = decltype(odd)::value != 0;
+        const unsigned char *la = abuf(ic<AI>());
+        const unsigned char *la_after = abuf(ic<(AI + 1) % 3>());
+        unsigned char *la_load = abuf(ic<(AI + 2) % 3>());
+        const int kt_codes = kt + 1 < nk ? kt + 1 : kt;
+        const int kt_a = kt + 2 < nk ? kt + 2 : nk - 1;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                if (t == 3 && i == 0) {
+                    wait_and_meet(ic<2>(), ic<ODD ? 0 : 1>());
+                    if (!I8 && ODD) use_qparams((kt + 1) >> 1);
+                }
+                const unsigned char *src = t < 3 ? la : la_after;
+                const int tn = (t + 1) & 3;
+                af[tn & 1][2 * i] = *reinterpret_cast<const u32x4_t *>(src + (2 * i) * 4096 + a_frag[tn]);
+                af[tn & 1][2 * i + 1] = *reinterpret_cast<const u32x4_t *>(src + (2 * i + 1) * 4096 + a_frag[tn]);
+                if (t < 3) deq_one(cw, tn, bf[tn & 1], i);
+                else deq_one(cn, 0, bf[0], i);
+                if (t == 0) load_codes_one(kt_codes, cn, i);
+                if (t == 1 && !I8 && !ODD) load_qparams_one((kt_codes + 1) >> 1 < groups_per_row ? (kt_codes + 1) >> 1 : groups_per_row - 1, i);
+                if (t >= 2) issue_a_one(kt_a, la_load, 2 * (t - 2) + i);
+                mfma_half(af[t & 1], bf[t & 1], i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
 #pragma unroll
         for (int i = 0; i < 2; ++i)
@@ -239,42 +302,20 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
             for (int b = 0; b < NB; ++b) cw[i][b] = cn[i][b];
     };
 
-    // One reduction step on stage AI with the codes in cw. Even steps start a quantisation group
-    // (its scale and zero were fetched during the previous, odd step); odd steps fetch the next
-    // group's. Within the step, the fragment reads and the dequantisation of slice t+1 are issued
-    // together with the MFMAs of slice t.
-    auto step = [&](int kt, auto ai, auto odd) {
-        constexpr int AI = decltype(ai)::value;
-        constexpr bool ODD = decltype(odd)::value != 0;
-        const unsigned char *la = abuf(ic<AI>());
-        u32x4_t af[2][4], bf[2][2];
-        if (!I8 && !ODD) use_qparams();
-        read_a(la, 0, af[0]);
-        if (!I8 && ODD) load_qparams(kt + 1 < nk ? (kt + 1) >> 1 : kt >> 1);
-        load_codes(kt + 1 < nk ? kt + 1 : kt, cn);
-        issue_a(kt + 2 < nk ? kt + 2 : nk - 1, abuf(ic<(AI + 2) % 3>()));
-        deq(0, bf[0]);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            if (t < 3) {
-                read_a(la, t + 1, af[(t + 1) & 1]);
-                deq(t + 1, bf[(t + 1) & 1]);
-            }
-            mfma(af[t & 1], bf[t & 1]);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        // Everything this wave loaded for step kt+1 has arrived (all but the 4 newest loads, the
-        // LDS-direct loads of tile kt+2) and its fragment reads of tile kt have returned: meet the
-        // other waves.
-        end_of_step(ic<ODD ? 1 : 0>());
-    };
-
     if (!I8) load_qparams(0);
     load_codes(0, cn);
     issue_a(0, lds_a0);
     issue_a(nk > 1 ? 1 : 0, lds_a1);
-    end_of_step(ic<1>());
+    wait_and_meet(ic<4>(), ic<1>());
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) cw[i][b] = cn[i][b];
+    if (!I8) use_qparams(0);
+    read_a(lds_a0, 0, af[0]);
+    deq_one(cw, 0, bf[0], 0);
+    deq_one(cw, 0, bf[0], 1);
+    __builtin_amdgcn_sched_barrier(0);
     int kt = 0;
     for (; kt + 6 <= nk; kt += 6) {
         step(kt, ic<0>(), ic<0>());
@@ -346,7 +387,7 @@ static int launch_direct(FwdParams p, bool i8, hipStream_t st, const char *who) 
     return lq_check_launch(who);
 }
 
-// Called by lq_a16w4_fwd (lq_gemm.hip) after argument validation: K % 128 == 0, N % 16 == 0, M > 16.
+// Called by lq_a16w4_fwd (lq_gemm.hip) after argument validation: K % 256 == 0, N % 16 == 0, M > 16.
 int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
                               void *y, int M, int N, int K, hipStream_t st) {
     FwdParams p = {};
