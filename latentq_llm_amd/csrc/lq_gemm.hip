@@ -549,7 +549,7 @@ extern "C" int lq_a16w4_fwd(const void *x, const void *codes, const void *scales
     // its tiles can occupy every CU twice; otherwise the staged 256 x 128 kernel, whose producer
     // waves hide more latency with a single workgroup per CU, is faster.
     // the weights-direct kernel loads scales and zeros four groups at a time: rows must be 4-byte aligned
-    if (lq_gemm_fwd_direct_workgroups((int)M, (int)N) >= 2ll * lq_device_cu_count() && (K / LQ_GROUP) % 2 == 0)
+    if (lq_gemm_fwd_direct_workgroups((int)M, (int)N) >= 1ll * lq_device_cu_count() && (K / LQ_GROUP) % 2 == 0)
         return lq_gemm_fwd_direct_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
     GemmParams p = {};
     p.a = x; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;

@@ -76,7 +76,11 @@ template <bool I8>
 __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     constexpr int ESZ = I8 ? 1 : 2;          // bytes per A element
     constexpr int WROW = I8 ? 128 : 32;      // bytes of one weight row consumed per step
-    constexpr int NB = I8 ? 4 : 1;           // 16-byte weight loads per lane, column tile and step
+    // 16-byte weight loads per lane and column tile in one batch: int8, the 4 pieces of one step;
+    // int4, the pieces of two consecutive steps (steps 2j and 2j+1 are 64 contiguous bytes of a
+    // row across the two lane halves: fetched together they pull their cache line through L1 twice
+    // instead of four times)
+    constexpr int NB = I8 ? 4 : 2;
     __shared__ __attribute__((aligned(16))) unsigned char lds_a0[STAGE];
     __shared__ __attribute__((aligned(16))) unsigned char lds_a1[STAGE];
     __shared__ __attribute__((aligned(16))) unsigned char lds_a2[STAGE];
@@ -169,7 +173,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     // All global loads of the loop are inline assembly: the compiler then inserts no vmcnt waits of
     // its own (it could only wait for everything, LDS-direct loads included); the single
     // s_waitcnt at the end of a step is tied to the loaded registers instead.
-    u32x4_t cw[2][NB], cn[2][NB];  // weights of the current and of the next step (int4 codes or int8)
+    u32x4_t cw[2][NB], cn[2][NB];  // weights of the current and of the next batch (int4 codes or int8)
     // Raw bf16 scales / zeros of four consecutive groups of the lane's two rows (one 8-byte load per
     // row every 8 steps: a 2-byte load per group would pull a whole cache line through L1 each time).
     // The 8-byte loads need 4-byte aligned rows: the launcher requires an even number of groups per row.
@@ -178,7 +182,9 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     auto load_codes_one = [&](int kt, u32x4_t (*c)[NB], int i) {
         {
             asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(c[i][0]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
-            if constexpr (I8) {
+            if constexpr (!I8) {
+                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:32" : "=v"(c[i][1]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
+            } else {
                 asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:16" : "=v"(c[i][1]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
                 asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:32" : "=v"(c[i][2]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
                 asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:48" : "=v"(c[i][3]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
@@ -213,12 +219,13 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) af[j] = *reinterpret_cast<const u32x4_t *>(la + j * 4096 + a_frag[t]);
     };
-    auto deq_one = [&](const u32x4_t (*c)[NB], int t, u32x4_t *bf, int i) {
+    // par = which step of the batch (int4 only)
+    auto deq_one = [&](const u32x4_t (*c)[NB], int par, int t, u32x4_t *bf, int i) {
         if constexpr (I8) {
             bf[i] = c[i][t];  // 16 int8 of the lane's row: already the MFMA operand
         } else {
             float f[8];
-            lq_dequant_word_f32(c[i][0][t], s[i], nzs[i], f);
+            lq_dequant_word_f32(c[i][par][t], s[i], nzs[i], f);
             bf[i] = u32x4_t{lq_pack_bf16(f[0], f[1]), lq_pack_bf16(f[2], f[3]), lq_pack_bf16(f[4], f[5]),
                             lq_pack_bf16(f[6], f[7])};
         }
@@ -245,10 +252,12 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
                          : "+v"(cn[0][0]), "+v"(cn[0][1]), "+v"(cn[0][2]), "+v"(cn[0][3]), "+v"(cn[1][0]), "+v"(cn[1][1]),
                            "+v"(cn[1][2]), "+v"(cn[1][3]) : "n"(NEWEST) : "memory");
         } else if constexpr (decltype(with_qparams)::value != 0) {
-            asm volatile("s_waitcnt vmcnt(%6) lgkmcnt(0)\n\ts_barrier"
-                         : "+v"(cn[0][0]), "+v"(cn[1][0]), "+v"(qs[0]), "+v"(qs[1]), "+v"(qz[0]), "+v"(qz[1]) : "n"(NEWEST) : "memory");
+            asm volatile("s_waitcnt vmcnt(%8) lgkmcnt(0)\n\ts_barrier"
+                         : "+v"(cn[0][0]), "+v"(cn[0][1]), "+v"(cn[1][0]), "+v"(cn[1][1]), "+v"(qs[0]), "+v"(qs[1]), "+v"(qz[0]),
+                           "+v"(qz[1]) : "n"(NEWEST) : "memory");
         } else {
-            asm volatile("s_waitcnt vmcnt(%2) lgkmcnt(0)\n\ts_barrier" : "+v"(cn[0][0]), "+v"(cn[1][0]) : "n"(NEWEST) : "memory");
+            asm volatile("s_waitcnt vmcnt(%4) lgkmcnt(0)\n\ts_barrier"
+                         : "+v"(cn[0][0]), "+v"(cn[0][1]), "+v"(cn[1][0]), "+v"(cn[1][1]) : "n"(NEWEST) : "memory");
         }
     };
 
@@ -273,7 +282,8 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         const unsigned char *la = abuf(ic<AI>());
         const unsigned char *la_after = abuf(ic<(AI + 1) % 3>());
         unsigned char *la_load = abuf(ic<(AI + 2) % 3>());
-        const int kt_codes = kt + 1 < nk ? kt + 1 : kt;
+        // int8: the next step's weights every step; int4: the next pair of steps on even steps
+        const int kt_codes = I8 ? (kt + 1 < nk ? kt + 1 : kt) : (kt + 2 < nk ? kt + 2 : kt);
         const int kt_a = kt + 2 < nk ? kt + 2 : nk - 1;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -287,19 +297,22 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
                 const int tn = (t + 1) & 3;
                 af[tn & 1][2 * i] = *reinterpret_cast<const u32x4_t *>(src + (2 * i) * 4096 + a_frag[tn]);
                 af[tn & 1][2 * i + 1] = *reinterpret_cast<const u32x4_t *>(src + (2 * i + 1) * 4096 + a_frag[tn]);
-                if (t < 3) deq_one(cw, tn, bf[tn & 1], i);
-                else deq_one(cn, 0, bf[0], i);
-                if (t == 0) load_codes_one(kt_codes, cn, i);
-                if (t == 1 && !I8 && !ODD) load_qparams_one((kt_codes + 1) >> 1 < groups_per_row ? (kt_codes + 1) >> 1 : groups_per_row - 1, i);
+                if (t < 3) deq_one(cw, ODD ? 1 : 0, tn, bf[tn & 1], i);
+                else if (I8 || ODD) deq_one(cn, 0, 0, bf[0], i);
+                else deq_one(cw, 1, 0, bf[0], i);
+                if (t == 0 && (I8 || !ODD)) load_codes_one(kt_codes, cn, i);
+                if (t == 1 && !I8 && !ODD) load_qparams_one((kt + 2) >> 1 < groups_per_row ? (kt + 2) >> 1 : groups_per_row - 1, i);
                 if (t >= 2) issue_a_one(kt_a, la_load, 2 * (t - 2) + i);
                 mfma_half(af[t & 1], bf[t & 1], i);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        if (I8 || ODD) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int b = 0; b < NB; ++b) cw[i][b] = cn[i][b];
+                for (int b = 0; b < NB; ++b) cw[i][b] = cn[i][b];
+        }
     };
 
     if (!I8) load_qparams(0);
@@ -313,8 +326,8 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         for (int b = 0; b < NB; ++b) cw[i][b] = cn[i][b];
     if (!I8) use_qparams(0);
     read_a(lds_a0, 0, af[0]);
-    deq_one(cw, 0, bf[0], 0);
-    deq_one(cw, 0, bf[0], 1);
+    deq_one(cw, 0, 0, bf[0], 0);
+    deq_one(cw, 0, 0, bf[0], 1);
     __builtin_amdgcn_sched_barrier(0);
     int kt = 0;
     for (; kt + 6 <= nk; kt += 6) {
