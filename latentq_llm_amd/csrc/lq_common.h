@@ -53,15 +53,25 @@ __device__ __forceinline__ float lq_ubyte1(unsigned x) { float r; asm("v_cvt_f32
 __device__ __forceinline__ float lq_ubyte2(unsigned x) { float r; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(x)); return r; }
 __device__ __forceinline__ float lq_ubyte3(unsigned x) { float r; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(x)); return r; }
 
+// Two adjacent bytes holding 0..15 -> two floats q/512, one instruction (v_cvt_pk_f32_fp8): read
+// as OCP FP8 E4M3, the bit patterns 0..15 are exactly q * 2^-9 (the first normal binade continues
+// the subnormals linearly). hi = false: bytes 0 and 1 of x, true: bytes 2 and 3.
+typedef float lq_f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ lq_f32x2_t lq_nibbles_lo(unsigned x) { return __builtin_amdgcn_cvt_pk_f32_fp8((int)x, false); }
+__device__ __forceinline__ lq_f32x2_t lq_nibbles_hi(unsigned x) { return __builtin_amdgcn_cvt_pk_f32_fp8((int)x, true); }
+
 // 8 codes of a native word -> 8 floats in k order, f = (q - z) * s rounded once:
-// nzs = -(z*s) is exact for bf16 z and s, and fma(q, s, nzs) rounds the exact (q - z) * s.
-__device__ __forceinline__ void lq_dequant_word_f32(unsigned word, float s, float nzs, float f[8]) {
+// nzs = -(z*s) is exact for bf16 z and s, s512 = 512*s is exact, and fma(q/512, s512, nzs) rounds
+// the exact (q - z) * s (scales of 2^118 and more, for which 512*s overflows, are not supported).
+__device__ __forceinline__ void lq_dequant_word_f32(unsigned word, float s512, float nzs, float f[8]) {
     const unsigned lo4 = word & 0x0F0F0F0Fu;         // odd k
     const unsigned hi4 = (word >> 4) & 0x0F0F0F0Fu;  // even k
-    f[0] = fmaf(lq_ubyte0(hi4), s, nzs); f[1] = fmaf(lq_ubyte0(lo4), s, nzs);
-    f[2] = fmaf(lq_ubyte1(hi4), s, nzs); f[3] = fmaf(lq_ubyte1(lo4), s, nzs);
-    f[4] = fmaf(lq_ubyte2(hi4), s, nzs); f[5] = fmaf(lq_ubyte2(lo4), s, nzs);
-    f[6] = fmaf(lq_ubyte3(hi4), s, nzs); f[7] = fmaf(lq_ubyte3(lo4), s, nzs);
+    const lq_f32x2_t e0 = lq_nibbles_lo(hi4), e1 = lq_nibbles_hi(hi4);  // k = 0, 2 and 4, 6
+    const lq_f32x2_t o0 = lq_nibbles_lo(lo4), o1 = lq_nibbles_hi(lo4);  // k = 1, 3 and 5, 7
+    f[0] = fmaf(e0[0], s512, nzs); f[1] = fmaf(o0[0], s512, nzs);
+    f[2] = fmaf(e0[1], s512, nzs); f[3] = fmaf(o0[1], s512, nzs);
+    f[4] = fmaf(e1[0], s512, nzs); f[5] = fmaf(o1[0], s512, nzs);
+    f[6] = fmaf(e1[1], s512, nzs); f[7] = fmaf(o1[1], s512, nzs);
 }
 
 // ---- Philox4x32-10 ---------------------------------------------------------

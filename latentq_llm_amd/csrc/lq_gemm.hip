@@ -79,23 +79,6 @@ __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
 __device__ __forceinline__ int swz_dx_piece(int row) { return ((row & 3) << 1) | (row & 1); }
 __device__ __forceinline__ int swz_dx_half(int row) { return (row >> 1) & 1; }
 
-// byte N of a dword as float, one instruction each
-__device__ __forceinline__ float ubyte0(unsigned x) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(x)); return r; }
-__device__ __forceinline__ float ubyte1(unsigned x) { float r; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(x)); return r; }
-__device__ __forceinline__ float ubyte2(unsigned x) { float r; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(x)); return r; }
-__device__ __forceinline__ float ubyte3(unsigned x) { float r; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(x)); return r; }
-
-// 8 codes of a native word -> 8 floats in k order, f = (q - z) * s exactly rounded once:
-// nzs = -(z*s) is exact for integer zeros, and fma(q, s, nzs) rounds the exact product (q-z)*s.
-__device__ __forceinline__ void dequant_word_f32(unsigned word, float s, float nzs, float f[8]) {
-    const unsigned lo4 = word & 0x0F0F0F0Fu;         // odd k
-    const unsigned hi4 = (word >> 4) & 0x0F0F0F0Fu;  // even k
-    f[0] = fmaf(ubyte0(hi4), s, nzs); f[1] = fmaf(ubyte0(lo4), s, nzs);
-    f[2] = fmaf(ubyte1(hi4), s, nzs); f[3] = fmaf(ubyte1(lo4), s, nzs);
-    f[4] = fmaf(ubyte2(hi4), s, nzs); f[5] = fmaf(ubyte2(lo4), s, nzs);
-    f[6] = fmaf(ubyte3(hi4), s, nzs); f[7] = fmaf(ubyte3(lo4), s, nzs);
-}
-
 template <int MODE, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
     constexpr int NT = 64 * WM * WN;           // threads per role
@@ -249,10 +232,11 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             } else if constexpr (MODE == MODE_W4_FWD) {
                 const float s = lq_bf16_bits_to_f32(S.s[0]);
                 const float nzs = -(lq_bf16_bits_to_f32(S.z[0]) * s);
+                const float s512 = s * 512.0f;  // the codes come out of the conversion as q/512
 #pragma unroll
                 for (int w = 0; w < NW; ++w) {
                     float f[8];
-                    dequant_word_f32(S.w[w], s, nzs, f);
+                    lq_dequant_word_f32(S.w[w], s512, nzs, f);
                     const int ch = b_w0 + w;
                     u32x4_t v = {lq_pack_bf16(f[0], f[1]), lq_pack_bf16(f[2], f[3]), lq_pack_bf16(f[4], f[5]),
                                  lq_pack_bf16(f[6], f[7])};
@@ -261,10 +245,11 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             } else {
                 const float s = lq_bf16_bits_to_f32(S.s[0]);
                 const float nzs = -(lq_bf16_bits_to_f32(S.z[0]) * s);
+                const float s512 = s * 512.0f;  // the codes come out of the conversion as q/512
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
                     float f[8];
-                    dequant_word_f32(S.w[w], s, nzs, f);
+                    lq_dequant_word_f32(S.w[w], s512, nzs, f);
                     u32x4_t v = {lq_pack_bf16(f[0], f[1]), lq_pack_bf16(f[2], f[3]), lq_pack_bf16(f[4], f[5]),
                                  lq_pack_bf16(f[6], f[7])};
                     const int c32 = b_w0 * 2 + (w >> 1);  // 32-byte piece of the 256-byte row

@@ -211,8 +211,9 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         for (int i = 0; i < 2; ++i) {
             const unsigned long long s4 = ((unsigned long long)qs[i][1] << 32) | qs[i][0];
             const unsigned long long z4 = ((unsigned long long)qz[i][1] << 32) | qz[i][0];
-            s[i] = __uint_as_float((unsigned)(s4 >> shift) << 16);
-            nzs[i] = -(__uint_as_float((unsigned)(z4 >> shift) << 16) * s[i]);
+            const float sc = __uint_as_float((unsigned)(s4 >> shift) << 16);
+            nzs[i] = -(__uint_as_float((unsigned)(z4 >> shift) << 16) * sc);
+            s[i] = sc * 512.0f;  // the codes come out of the conversion as q/512
         }
     };
     auto read_a = [&](const unsigned char *la, int t, u32x4_t *af) {
