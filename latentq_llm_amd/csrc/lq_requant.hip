@@ -39,19 +39,17 @@ __device__ __forceinline__ unsigned requant_word_fast(unsigned codes, const unsi
     const float nzs = -(z * s);
     const unsigned lo4 = codes & 0x0F0F0F0Fu;         // odd elements
     const unsigned hi4 = (codes >> 4) & 0x0F0F0F0Fu;  // even elements
-    float qf[8];
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        qf[2 * b] = (float)((hi4 >> (8 * b)) & 0xFFu);
-        qf[2 * b + 1] = (float)((lo4 >> (8 * b)) & 0xFFu);
-    }
+    // the codes as q/512, two per conversion; s512 = 512*s is exact (s <= 2^40 here)
+    const lq_f32x2_t e0 = lq_nibbles_lo(hi4), e1 = lq_nibbles_hi(hi4), o0 = lq_nibbles_lo(lo4), o1 = lq_nibbles_hi(lo4);
+    const float qf[8] = {e0[0], o0[0], e0[1], o0[1], e1[0], o1[0], e1[1], o1[1]};
+    const float s512 = s * 512.0f;
     unsigned out = 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        // (q - z) * s as fma(q, s, -(z*s)): z*s and q*s are exact (8-bit significands), the sum has at
+        // (q - z) * s as fma(q/512, 512*s, -(z*s)): z*s and q*s are exact (8-bit significands), the sum has at
         // most 16 significant bits, so the fma returns (q - z) * s exactly; then the bf16 rounding of
         // the dequantised weight, two elements per v_cvt_pk_bf16_f32
-        const unsigned pk = lq_pack_bf16(fmaf(qf[2 * i], s, nzs), fmaf(qf[2 * i + 1], s, nzs));
+        const unsigned pk = lq_pack_bf16(fmaf(qf[2 * i], s512, nzs), fmaf(qf[2 * i + 1], s512, nzs));
         float t[2] = {fmaf(-lr, lq_bf16_lo(gp[i]), lq_bf16_lo(pk)), fmaf(-lr, lq_bf16_hi(gp[i]), lq_bf16_hi(pk))};
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
