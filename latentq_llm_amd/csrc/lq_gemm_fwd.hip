@@ -296,8 +296,9 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
                 }
                 const unsigned char *src = t < 3 ? la : la_after;
                 const int tn = (t + 1) & 3;
-                af[tn & 1][2 * i] = *reinterpret_cast<const u32x4_t *>(src + (2 * i) * 4096 + a_frag[tn]);
-                af[tn & 1][2 * i + 1] = *reinterpret_cast<const u32x4_t *>(src + (2 * i + 1) * 4096 + a_frag[tn]);
+                // all four fragments of the next slice in the first half: a full slice of MFMAs covers
+                // their LDS latency
+                if (i == 0) read_a(src, tn, af[tn & 1]);
                 if (t < 3) deq_one(cw, ODD ? 1 : 0, tn, bf[tn & 1], i);
                 else if (I8 || ODD) deq_one(cn, 0, 0, bf[0], i);
                 else deq_one(cw, 1, 0, bf[0], i);
