@@ -26,8 +26,8 @@
 //     4h + t of the 128-byte tile row. Chunk c of row m sits at position c ^ ((m >> 1) & 7),
 //     which makes the 16-lane fragment reads conflict-free; the swizzle costs nothing because an
 //     LDS-direct load lets each lane choose which global chunk lands in its (fixed) LDS slot.
-//   * D = Wfrag x Xfrag^T: D[i][j] has i = n, j = m, so a lane owns 4 consecutive n of one m
-//     and the epilogue stores 8-byte bf16 quads.
+//   * D = Wfrag x Xfrag^T: D[i][j] has i = n, j = m, so a lane owns 4 consecutive n of one m;
+//     the epilogue regroups them through LDS into 16-byte pieces of full output rows.
 //
 // Dequantisation is bf16(fma(q, s, -(z*s))): z*s and q*s are exact in fp32, so the fma rounds
 // the exact (q - z)*s once; for integer zeros this equals the reference's bf16(bf16(q-z)*s).
@@ -351,35 +351,64 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     // the clamped prefetches of the last two steps are still writing LDS: drain them
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    // ---- epilogue: acc[i][j][q]: column c0 + 64*wave + 32i + 8*(q/4) + 4h + q%4, row m0 + 32j + r
+    // ---- epilogue: acc[i][j][q]: column c0 + 64*wave + 32i + 8*(q/4) + 4h + q%4, row m0 + 32j + r.
+    // A lane holds 4 consecutive columns of one row: stored straight from the registers, an
+    // instruction would touch 32 rows with 16 bytes each. Instead every wave passes its block
+    // through LDS, 32 rows (one j) at a time, and stores 16 bytes per lane with 8 lanes on the 128
+    // contiguous bytes of a row: full cache lines. The stages are free once every wave has left the
+    // loop and its loads have landed; a wave's staging area is private (waves 0,1 in stage 0, waves
+    // 2,3 in stage 1), row pitch 144 bytes.
+    __syncthreads();
+    constexpr int EP = 144;
+    unsigned char *ep = ((wave & 2) ? lds_a1 : lds_a0) + (wave & 1) * (32 * EP);
+    const int ep_row = lane >> 3, ep_chunk = lane & 7;
+    const int c_lane = c0 + wave * 64 + ep_chunk * 8;  // first of the 8 columns this lane stores
+    float bias_v[2][4][4], sw_v[2][4][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int c = c0 + wave * 64 + i * 32 + 8 * q + 4 * h;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const bool in = c + e < p.N;
+                bias_v[i][q][e] = (p.bias && in) ? lq_bf16_bits_to_f32(p.bias[c + e]) : 0.0f;
+                if constexpr (I8) sw_v[i][q][e] = in ? p.sw[c + e] : 0.0f;
+            }
+        }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int m = m0 + j * 32 + r;
-        if (m >= p.M) continue;
         float sxm = 1.0f;
-        if constexpr (I8) sxm = p.sx[m];
+        if constexpr (I8) sxm = m < p.M ? p.sx[m] : 0.0f;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int c = c0 + wave * 64 + i * 32 + 8 * q + 4 * h;
-                if (c >= p.N) continue;  // N is a multiple of 4: a quad is all-in or all-out
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    if constexpr (I8) v[e] = ((float)acc[i][j][4 * q + e] * sxm) * p.sw[c + e];
+                    if constexpr (I8) v[e] = ((float)acc[i][j][4 * q + e] * sxm) * sw_v[i][q][e];
                     else v[e] = acc[i][j][4 * q + e];
-                    if (p.bias) v[e] += lq_bf16_bits_to_f32(p.bias[c + e]);
+                    if (p.bias) v[e] += bias_v[i][q][e];
                 }
                 u32x2_t o = {lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3])};
-                *reinterpret_cast<u32x2_t *>(p.y + (long long)m * p.N + c) = o;
+                *reinterpret_cast<u32x2_t *>(ep + r * EP + (i * 32 + 8 * q + 4 * h) * 2) = o;
                 if constexpr (I8) {
-                    if (p.acc_out) {
+                    const int c = c0 + wave * 64 + i * 32 + 8 * q + 4 * h;
+                    if (p.acc_out && m < p.M && c < p.N) {
                         i32x4_t a4 = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
                         *reinterpret_cast<i32x4_t *>(p.acc_out + (long long)m * p.N + c) = a4;
                     }
                 }
             }
+        }
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int row = it * 8 + ep_row;
+            const u32x4_t o = *reinterpret_cast<const u32x4_t *>(ep + row * EP + ep_chunk * 16);
+            const int mm = m0 + j * 32 + row;
+            if (mm < p.M && c_lane < p.N) *reinterpret_cast<u32x4_t *>(p.y + (long long)mm * p.N + c_lane) = o;
         }
     }
 }
