@@ -20,7 +20,8 @@
 //
 // The MFMA is issued with the weight fragment as the first operand and the activation
 // fragment as the second, so that D[i][j] has i = output column (n), j = row (m): a
-// lane then owns 4 consecutive n for one m and the epilogue stores 8-byte bf16 quads.
+// lane then owns 4 consecutive n for one m; the epilogue regroups them through LDS into 16-byte
+// pieces of full output rows.
 //
 // Wave specialisation. A workgroup has 2 x WM x WN waves, two per SIMD.
 //   * The first WM x WN ("math") waves issue the MFMAs. They also fetch the A tiles, but with
@@ -429,37 +430,69 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
 
     // ---- epilogue -----------------------------------------------------------
     // acc[i][j][r]: column c = c0 + wn*TN + i*32 + 8*(r/4) + 4*(lane/32) + r%4, row m = m0 + wm*TM + j*32 + lane%32.
+    // A lane holds 4 consecutive columns of one row; stored straight from the registers an
+    // instruction would touch 32 rows with 16 bytes each. Every math wave passes its block through
+    // LDS instead, 32 rows (one j) at a time, and stores 16 bytes per lane with TN/8 lanes on the
+    // contiguous bytes of a row. The B buffers are free here (the weight waves wrote their last
+    // tile before the final barrier, and no load is in flight into them); a wave's staging area
+    // is private, row pitch TN*2 + 16 bytes.
     unsigned short *out = (unsigned short *)p.c;
+    constexpr int EP = TN * 2 + 16;
+    constexpr int EP_WAVE = 32 * EP;
+    constexpr int EP_PER_BUF = B_BYTES / EP_WAVE;
+    static_assert(WM * WN <= 2 * EP_PER_BUF, "epilogue staging does not fit the B buffers");
+    unsigned char *ep = (wave >= EP_PER_BUF ? lds_b1 : lds_b0) + (wave % EP_PER_BUF) * EP_WAVE;
+    constexpr int LPR = TN / 8;        // lanes per staged row (16 bytes each)
+    constexpr int RPI = 64 / LPR;      // rows per store instruction
+    const int ep_row = lane / LPR, ep_chunk = lane % LPR;
+    const int c_lane = c0 + wn * TN + ep_chunk * 8;
+    float bias_v[FN][4][4], sw_v[FN][4][4];
+#pragma unroll
+    for (int i = 0; i < FN; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int c = c0 + wn * TN + i * 32 + 8 * q + 4 * kh;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const bool in = c + r < p.C;
+                bias_v[i][q][r] = (p.bias && in) ? lq_bf16_bits_to_f32(p.bias[c + r]) : 0.0f;
+                if (MODE == MODE_I8) sw_v[i][q][r] = in ? p.sw[c + r] : 0.0f;
+            }
+        }
 #pragma unroll
     for (int j = 0; j < FM; ++j) {
         const int m = m0 + wm * TM + j * 32 + frag_row;
-        if (m >= p.M) continue;
         float sxm = 1.0f;
-        if (MODE == MODE_I8) sxm = p.sx[m];
+        if (MODE == MODE_I8) sxm = m < p.M ? p.sx[m] : 0.0f;
 #pragma unroll
         for (int i = 0; i < FN; ++i) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int c = c0 + wn * TN + i * 32 + 8 * q + 4 * kh;
-                if (c >= p.C) continue;  // C is a multiple of 4: a quad is all-in or all-out
                 float v[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    if (MODE == MODE_I8) {
-                        v[r] = ((float)acc[i][j][4 * q + r] * sxm) * p.sw[c + r];
-                    } else {
-                        v[r] = acc[i][j][4 * q + r];
-                    }
-                    if (p.bias) v[r] += lq_bf16_bits_to_f32(p.bias[c + r]);
+                    if (MODE == MODE_I8) v[r] = ((float)acc[i][j][4 * q + r] * sxm) * sw_v[i][q][r];
+                    else v[r] = acc[i][j][4 * q + r];
+                    if (p.bias) v[r] += bias_v[i][q][r];
                 }
                 u32x2_t o = {lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3])};
-                *reinterpret_cast<u32x2_t *>(out + (long long)m * p.C + c) = o;
+                *reinterpret_cast<u32x2_t *>(ep + frag_row * EP + (i * 32 + 8 * q + 4 * kh) * 2) = o;
                 if (MODE == MODE_I8 && p.acc_out) {
-                    i32x4_t a4 = {(int)acc[i][j][4 * q], (int)acc[i][j][4 * q + 1], (int)acc[i][j][4 * q + 2],
-                                  (int)acc[i][j][4 * q + 3]};
-                    *reinterpret_cast<i32x4_t *>(p.acc_out + (long long)m * p.C + c) = a4;
+                    const int c = c0 + wn * TN + i * 32 + 8 * q + 4 * kh;
+                    if (m < p.M && c < p.C) {
+                        i32x4_t a4 = {(int)acc[i][j][4 * q], (int)acc[i][j][4 * q + 1], (int)acc[i][j][4 * q + 2],
+                                      (int)acc[i][j][4 * q + 3]};
+                        *reinterpret_cast<i32x4_t *>(p.acc_out + (long long)m * p.C + c) = a4;
+                    }
                 }
             }
+        }
+#pragma unroll
+        for (int it = 0; it < 32 / RPI; ++it) {
+            const int row = it * RPI + ep_row;
+            const u32x4_t o = *reinterpret_cast<const u32x4_t *>(ep + row * EP + ep_chunk * 16);
+            const int mm = m0 + wm * TM + j * 32 + row;
+            if (mm < p.M && c_lane < p.C) *reinterpret_cast<u32x4_t *>(out + (long long)mm * p.C + c_lane) = o;
         }
     }
 }
