@@ -113,8 +113,8 @@ MLP_FLOP = 6 * 2 * TOKENS * HID * FFN  # 1 108.1 GFLOP
 # each scaled by what the same counter reads for the 256 MiB calibration copy of the same run
 # (FETCH_SIZE reads half the bytes fetched: factor 2.000; WRITE_SIZE factor 1.000).
 PMC_GEMM_MB = {
-    "fwd_gate_up": (221.77, 45.16), "fwd_down": (190.62, 16.78),
-    "dx_gate_up": (195.82, 16.78), "dx_down": (280.18, 45.10),
+    "fwd_gate_up": (223.79, 45.09), "fwd_down": (190.65, 16.78),
+    "dx_gate_up": (198.20, 16.78), "dx_down": (280.47, 45.09),
 }
 PMC_LAUNCHES = {"fwd_gate_up": 2, "fwd_down": 1, "dx_gate_up": 2, "dx_down": 1}  # per MLP step
 
@@ -357,7 +357,7 @@ def main():
     tot = 2 * kern["fwd_gate_up"]["us"] + kern["fwd_down"]["us"] + 2 * kern["dx_gate_up"]["us"] + kern["dx_down"]["us"]
     avg_us = tot / 6
     achieved = 2 * TOKENS * HID * FFN / (avg_us * 1e-6) / 1e12
-    roofline = {"bound": "mfma", "kernel": "A16W4 dequant-GEMM: gemm_fwd_direct_kernel (forward gate/up), gemm_kernel<0> (forward down), gemm_kernel<1> (dX)",
+    roofline = {"bound": "mfma", "kernel": "A16W4 dequant-GEMM: gemm_fwd_direct_kernel (forward), gemm_kernel<1> (dX)",
                 "achieved": achieved, "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": achieved * 1e12 / PEAK_BF16,
                 "avg_launch_us": avg_us, "flop_per_launch": 2 * TOKENS * HID * FFN, "traffic": gemm_traffic_bytes(),
                 "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated on a copy)"}
