@@ -167,8 +167,11 @@ def _fwd_case(ops, co, M, N, K, seed, with_bias):
 
 @pytest.mark.parametrize("M,N,K,bias", [(17, 16, 128, False), (33, 48, 256, True), (128, 128, 128, False),
                                         (129, 256, 384, True), (300, 272, 512, False), (1024, 3072, 768, True),
-                                        # ragged in M and N and large enough for the weights-direct kernel
-                                        (4100, 4112, 128, True), (3000, 6160, 384, False)])
+                                        # ragged in M and N on large grids: odd group counts (staged kernel) ...
+                                        (4100, 4112, 128, True), (3000, 6160, 384, False),
+                                        # ... and even ones (weights-direct kernel): 4, 12 and 20 steps, i.e. one
+                                        # partial quad of scales, one and a half, and two and a half
+                                        (4100, 4112, 256, True), (3000, 6160, 768, False), (2100, 4112, 1280, True)])
 def test_a16w4_fwd_gemm(ops, co, M, N, K, bias):
     _fwd_case(ops, co, M, N, K, seed=M + N + K, with_bias=bias)
 
@@ -188,6 +191,18 @@ def test_a16w4_fwd_identity_is_exact_dequant(ops, co):
     got = ops.a16w4_forward(dev(x), dev(packed), dev(scales), dev(zeros), (N, K))
     want = co.dequant(packed.numpy(), bits(scales), bits(zeros), N, K)  # [N, K]
     assert np.array_equal(bits(got).T, want)
+
+
+def test_a16w4_fwd_identity_is_exact_dequant_direct_kernel(ops, co):
+    """The same on a grid of 16 x 16 tiles, which runs the weights-direct kernel (half-integer zeros
+    included: q - z stays exact in bf16, so the reference's two roundings and the kernel's one agree)."""
+    N, K = 4096, 2048
+    codes, packed, scales, zeros = make_w4(N, K, 22)
+    zeros.view(-1)[::7] = 7.5
+    x = torch.eye(K, dtype=torch.bfloat16)
+    got = ops.a16w4_forward(dev(x), dev(packed), dev(scales), dev(zeros), (N, K))
+    want = co.dequant(packed.numpy(), bits(scales), bits(zeros), N, K)  # [N, K]
+    assert int((bits(got).T != want).sum()) == 0
 
 
 def test_a16w4_fwd_integer_exact(ops, co):
