@@ -47,12 +47,6 @@ __device__ __forceinline__ unsigned short lq_f32_to_bf16_bits(float a) {
 // consecutive k: code j sits at bit 4*(j^1)  (even index = high nibble of its byte).
 __device__ __forceinline__ unsigned lq_code(unsigned word, int j) { return (word >> (4 * (j ^ 1))) & 0xFu; }
 
-// byte N of a dword as float, one instruction each (v_cvt_f32_ubyteN)
-__device__ __forceinline__ float lq_ubyte0(unsigned x) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(x)); return r; }
-__device__ __forceinline__ float lq_ubyte1(unsigned x) { float r; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(x)); return r; }
-__device__ __forceinline__ float lq_ubyte2(unsigned x) { float r; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(x)); return r; }
-__device__ __forceinline__ float lq_ubyte3(unsigned x) { float r; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(x)); return r; }
-
 // Two adjacent bytes holding 0..15 -> two floats q/512, one instruction (v_cvt_pk_f32_fp8): read
 // as OCP FP8 E4M3, the bit patterns 0..15 are exactly q * 2^-9 (the first normal binade continues
 // the subnormals linearly). hi = false: bytes 0 and 1 of x, true: bytes 2 and 3.
