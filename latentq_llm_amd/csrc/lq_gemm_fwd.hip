@@ -172,7 +172,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
 
     // All global loads of the loop are inline assembly: the compiler then inserts no vmcnt waits of
     // its own (it could only wait for everything, LDS-direct loads included); the single
-    // s_waitcnt at the end of a step is tied to the loaded registers instead.
+    // s_waitcnt of a step is tied to the loaded registers instead.
     u32x4_t cw[2][NB], cn[2][NB];  // weights of the current and of the next batch (int4 codes or int8)
     // Raw bf16 scales / zeros of four consecutive groups of the lane's two rows (one 8-byte load per
     // row every 8 steps: a 2-byte load per group would pull a whole cache line through L1 each time).
