@@ -194,6 +194,11 @@ def bench_a8w8(device):
         sec = event_time(lambda: ops.a8w8_forward(x8, w8, sx, sw), 20)
         out.append({"M": M, "N": N, "K": K, "us": sec * 1e6, "TOP/s": 2 * M * N * K / sec / 1e12,
                     "frac_mfma_i8": 2 * M * N * K / sec / PEAK_I8})
+    # the activation quantiser in front of the GEMM (bf16 -> int8, clamp value on the device)
+    x = torch.randn(M, 8192, device=device).to(torch.bfloat16)
+    clampv = x.float().abs().max().reshape(1)
+    sec = event_time(lambda: ops.act_quant_i8(x, clampv), 20)
+    out.append({"act_quant": [M, 8192], "us": sec * 1e6, "GB/s": 3 * x.numel() / sec / 1e9})
     return out
 
 
