@@ -301,14 +301,20 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
     // lane offset) so that the compiler's wait-count insertion does not see an LDS write it cannot
     // tell apart from the fragment reads and park a vmcnt(0) in front of them: the explicit
     // s_waitcnt before each barrier is the only ordering these loads need.
-    auto issue_a = [&](int kt, unsigned char *la) {
+    static_assert(APT % 4 == 0, "A loads are issued in four parts per tile");
+    // part q (0..3) of a tile's loads: APT/4 of them
+    auto issue_a_part = [&](int kt, unsigned char *la, int q) {
         const unsigned char *src = a_base + (long long)kt * ROWB;
 #pragma unroll
-        for (int i = 0; i < APT; ++i) {
+        for (int i = q * (APT / 4); i < (q + 1) * (APT / 4); ++i) {
             const unsigned lds_addr = (unsigned)reinterpret_cast<size_t>((lds_void *)(la + (i * NT + wave * 64) * 16));
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                          :: "s"(lds_addr), "v"(a_off[i]), "s"(src) : "memory");
         }
+    };
+    auto issue_a = [&](int kt, unsigned char *la) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) issue_a_part(kt, la, q);
     };
 
     using acc_t = typename std::conditional<MODE == MODE_I8, i32x16_t, f32x16_t>::type;
@@ -384,30 +390,39 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             }
     };
 
-    // Tile kt: A in buffer kt%3, B in buffer kt%2. Start the first fragment reads, put the A loads
-    // of tile kt+2 in flight behind them (into the buffer tile kt-1 just left), then 4 MFMA steps
-    // with double-buffered fragments,
-    // then wait until this wave's part of tile kt+1 has landed (all but the newest APT loads)
-    // and its fragment reads have returned, and meet the other waves.
+    // Tile kt: A in buffer kt%3, B in buffer kt%2; the fragments of its first reduction slice are
+    // already in af[0] / bf[0]. Four slices of FN*FM MFMAs; each also reads the fragments of the
+    // next slice and issues a quarter of the A loads of tile kt+2 (into the buffer tile kt-1 left;
+    // one burst of them would hold the wave at the memory pipeline's queue with its MFMAs behind
+    // it). The tile's one synchronisation point sits before the last slice: this wave's part of
+    // tile kt+1 has landed (all but the 3/4 of tile kt+2's loads issued since), its fragment reads of
+    // tile kt have all returned, the weight waves have published B tile kt+1. The last slice then
+    // already reads the first fragments of tile kt+1, so the MFMA stream does not drain at the
+    // tile boundary. After the barrier nobody reads tile kt's buffers any more, which is what
+    // lets the weight waves overwrite its B buffer and the next tile's loads its A buffer.
+    u32x4_t af[2][FM], bf[2][FN];
     auto tile_step = [&](int kt, auto ai, auto bi) {
         constexpr int AI = decltype(ai)::value, BI = decltype(bi)::value;
         const unsigned char *la = abuf(ic<AI>()), *lb = bbuf(ic<BI>());
-        u32x4_t af[2][FM], bf[2][FN];
-        read_frags(la, lb, 0, af[0], bf[0]);
-        read_frags(la, lb, 1, af[1], bf[1]);
-        issue_a(kt + 2 < nk ? kt + 2 : nk - 1, abuf(ic<(AI + 2) % 3>()));
-        mfma_step(af[0], bf[0]);
-        read_frags(la, lb, 2, af[0], bf[0]);
-        mfma_step(af[1], bf[1]);
-        read_frags(la, lb, 3, af[1], bf[1]);
-        mfma_step(af[0], bf[0]);
-        mfma_step(af[1], bf[1]);
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(APT) : "memory");
+        const unsigned char *la_next = abuf(ic<(AI + 1) % 3>()), *lb_next = bbuf(ic<BI ^ 1>());
+        unsigned char *la_load = abuf(ic<(AI + 2) % 3>());
+        const int kt_a = kt + 2 < nk ? kt + 2 : nk - 1;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            if (t == 3) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(3 * APT / 4) : "memory");
+            if (t < 3) read_frags(la, lb, t + 1, af[(t + 1) & 1], bf[(t + 1) & 1]);
+            else read_frags(la_next, lb_next, 0, af[0], bf[0]);
+            issue_a_part(kt_a, la_load, t);
+            mfma_step(af[t & 1], bf[t & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     };
 
     issue_a(0, lds_a0);
     issue_a(nk > 1 ? 1 : 0, lds_a1);
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(APT) : "memory");
+    read_frags(lds_a0, lds_b0, 0, af[0], bf[0]);
+    __builtin_amdgcn_sched_barrier(0);
     int kt = 0;
     for (; kt + 6 <= nk; kt += 6) {
         tile_step(kt, ic<0>(), ic<0>());
