@@ -113,8 +113,8 @@ MLP_FLOP = 6 * 2 * TOKENS * HID * FFN  # 1 108.1 GFLOP
 # each scaled by what the same counter reads for the 256 MiB calibration copy of the same run
 # (FETCH_SIZE reads half the bytes fetched: factor 2.000; WRITE_SIZE factor 1.000).
 PMC_GEMM_MB = {
-    "fwd_gate_up": (223.79, 45.09), "fwd_down": (190.65, 16.78),
-    "dx_gate_up": (198.20, 16.78), "dx_down": (280.47, 45.09),
+    "fwd_gate_up": (224.16, 45.09), "fwd_down": (190.66, 16.78),
+    "dx_gate_up": (191.95, 16.78), "dx_down": (279.10, 45.09),
 }
 PMC_LAUNCHES = {"fwd_gate_up": 2, "fwd_down": 1, "dx_gate_up": 2, "dx_down": 1}  # per MLP step
 
