@@ -202,6 +202,36 @@ def bench_a8w8(device):
     return out
 
 
+def bench_adam8(device):
+    """One Adam step on uint8 block-wise moments over 8192 x 2048 elements: the fused kernel and, for
+    scale, the chain of tensor operations it replaces (latentq_llm_amd.quant with FUSED_ADAM8 off)."""
+    from latentq_llm_amd import ops, quant as q
+    n, block = 8192 * 2048, 2048
+    nblk = n // block
+    grad = (torch.randn(n, device=device) * 1e-3).to(torch.bfloat16)
+    param = (torch.randn(n, device=device) * 0.02).to(torch.bfloat16)
+    s1 = torch.randint(0, 256, (n,), device=device, dtype=torch.uint8)
+    s2 = torch.randint(0, 256, (n,), device=device, dtype=torch.uint8)
+    sc1 = torch.full((nblk, 1), 1e-5, device=device); mx1 = torch.full((nblk, 1), 1.3e-3, device=device)
+    sc2 = torch.full((nblk, 1), 1e-5, device=device); mx2 = torch.full((nblk, 1), 2.6e-3, device=device)
+    sec = event_time(lambda: ops.adam8_update(grad, s1, s2, sc1, mx1, sc2, mx2, 0.9, 0.95, 1e-8, 1e-3, param=param), 20)
+    nbytes = 10 * n + 32 * nblk
+
+    def chain():
+        m = q.DeQfunc_8bit_opt(s1, [sc1, mx1]).to(grad.dtype)
+        t = q.DeQfunc_8bit_opt(s2, [sc2, mx2])
+        v = (t * t).to(grad.dtype)
+        m.mul_(0.9).add_(grad, alpha=0.1)
+        v.mul_(0.95).addcmul_(grad, grad, value=0.05)
+        d = v.sqrt_().add_(1e-8)
+        param.addcdiv_(m, d, value=-1e-3)
+        q.Qfunc_8bit_opt(m.float(), blocksize=nblk)
+        q.Qfunc_8bit_opt(d.float(), blocksize=nblk)
+    sec_chain = event_time(chain, 5, warm=2)
+    return {"elements": n, "block": block, "bytes": nbytes, "us": sec * 1e6, "GB/s": nbytes / sec / 1e9,
+            "frac_hbm": nbytes / sec / PEAK_HBM, "tensor_op_chain_us": sec_chain * 1e6}
+
+
 def bench_copy(device):
     """Plain streaming copy (lq_calib_copy) over buffers larger than the last-level cache: the
     HBM rate this device sustains for read + write traffic, for comparison with the 8 TB/s peak."""
@@ -384,6 +414,7 @@ def main():
         line["latent_lbit4"] = bench_latent(dev)
         line["gemv"] = bench_gemv(dev)
         line["a8w8"] = bench_a8w8(dev)
+        line["adam8"] = bench_adam8(dev)
         line["hbm_copy"] = bench_copy(dev)
     line["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
     print(json.dumps(line))

@@ -162,6 +162,25 @@ int lq_latent_w4_requant(const void *latent, const void *scales, const void *zer
                          int k3, void *stream);
 
 /* ---------------------------------------------------------------------------
+ * One Adam step on 8-bit block-wise moments, the chain of tensor operations of
+ * MyAdam.update_step (reference utils/quant.py:1081-1134) with Qfunc_8bit_opt /
+ * DeQfunc_8bit_opt (:22-41) as a single pass with the chain's rounding points kept:
+ *   m = bf16(max1 - q1*scale1), v = bf16((max2 - q2*scale2)^2),
+ *   m = bf16(bf16(m*beta1) + (1-beta1)*g), v = bf16(bf16(v*beta2) + (1-beta2)*g*g),
+ *   d = bf16(bf16(sqrt(v)) + eps), param = bf16(param - step_size*(m/d))   (or direction = bf16(m/d)),
+ *   then m and d re-quantised per block: max = max(x), scale = (max - min(x))/255 + 1e-10,
+ *   q = clamp(rint((max - x)/scale), 0, 255).
+ * grad, param, direction: bf16[n], 16-byte aligned; exactly one of param (updated in place) and
+ * direction (written) is non-null. state1/state2: uint8[n], 8-byte aligned, updated in place;
+ * scale1/max1/scale2/max2: fp32[n/block_elems], updated in place (the reference's qmap1/absmax1/
+ * qmap2/absmax2). block_elems is 2048 or 128 and divides n. Weight decay and the periodic
+ * update of the residual codec's range are not part of this call.
+ * ------------------------------------------------------------------------- */
+int lq_adam8_update(const void *grad, void *param_or_null, void *direction_or_null, uint8_t *state1, uint8_t *state2,
+                    float *scale1, float *max1, float *scale2, float *max2, int64_t n, int block_elems, double beta1,
+                    double beta2, double eps, double step_size, void *stream);
+
+/* ---------------------------------------------------------------------------
  * Layout converters (device side).
  * GPTQ layout (reference PTQ/quant/quant_linear.py:343-389): qweight is
  * int32[K/8, N] with code(k, n) at bits 4*(k%8) of word [k/8, n].

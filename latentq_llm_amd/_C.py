@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "liblatentq_hip.so")
 
 ABI_VERSION = 1
 
-_vp, _i64, _i32, _u64, _f32 = C.c_void_p, C.c_int64, C.c_int, C.c_uint64, C.c_float
+_vp, _i64, _i32, _u64, _f32, _f64 = C.c_void_p, C.c_int64, C.c_int, C.c_uint64, C.c_float, C.c_double
 
 # name -> argtypes; every function returns int except lq_last_error.
 SIGNATURES = {
@@ -32,6 +32,7 @@ SIGNATURES = {
     "lq_calib_copy": [_vp, _vp, _i64, _vp],
     "lq_latent_w4_reconstruct": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],
     "lq_latent_w4_requant": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],
+    "lq_adam8_update": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _f64, _f64, _f64, _f64, _vp],
 }
 
 _lib = None

@@ -1,0 +1,176 @@
+// Fused Adam step on 8-bit block-wise moments for gfx950.
+//
+// The reference's optimizer (utils/quant.py:1081-1134 with Qfunc_8bit_opt / DeQfunc_8bit_opt,
+// :22-41) keeps both moments as uint8 with one fp32 (scale, max) pair per block of 2048 (or 128)
+// elements, the second one as sqrt(v) + eps, and runs one step as a chain of ~25 elementwise
+// tensor operations per parameter:
+//     m  = bf16(max1 - q1 * scale1)                      s2 = max2 - q2 * scale2,  v = bf16(s2 * s2)
+//     m  = bf16(m * beta1);  m = bf16(m + (1 - beta1) * g)
+//     v  = bf16(v * beta2);  v = bf16(v + (1 - beta2) * g * g)
+//     d  = bf16(sqrt(v));    d = bf16(d + eps)
+//     p  = bf16(p - step * (m / d))                      (or, for the stochastic-rounding
+//                                                         requantizer, direction = bf16(m / d))
+//     per block: max = max(x), scale = (max - min(x)) * (1/255) + 1e-10,
+//                q = clamp(rint((max - x) / scale), 0, 255)        for x = m and for x = d
+// Every tensor operation computes in fp32 and rounds its result to the tensor's type; an
+// operation of the form a + alpha * b is a fused multiply-add inside the tensor library's
+// kernels. This kernel is that chain in one pass with the same rounding points, so its results
+// equal the chain's bit for bit: 8 elements per thread (16 bytes of gradient and parameter, 8
+// bytes of each moment), the block's minimum and maximum found by a reduction over the BS/8
+// threads of the block, 6 bytes read and 4 written per element instead of ~120.
+#include "lq_common.h"
+
+namespace {
+
+__device__ __forceinline__ float bf16r(float v) { return lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(v)); }
+
+struct Adam8Params {
+    const u32x4_t *grad;     // bf16
+    u32x4_t *param;          // bf16, updated in place, or null
+    u32x4_t *direction;      // bf16 m / d, or null
+    u32x2_t *state1, *state2;  // uint8 moments, updated in place
+    float *scale1, *max1, *scale2, *max2;  // per block, updated in place
+    long long n_threads;     // elements / 8
+    float beta1, one_minus_beta1, beta2, one_minus_beta2, eps, neg_step;
+};
+
+// minimum and maximum over the W threads that share a block (W = 16: one 16-lane row of the
+// wave, by cross-lane shuffles; W = 256: the whole workgroup, through LDS)
+template <int W>
+__device__ __forceinline__ void block_minmax(float &lo, float &hi, float (*red)[2]) {
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        lo = fminf(lo, __shfl_xor(lo, off, 64));
+        hi = fmaxf(hi, __shfl_xor(hi, off, 64));
+    }
+    if constexpr (W == 256) {
+#pragma unroll
+        for (int off = 16; off < 64; off <<= 1) {
+            lo = fminf(lo, __shfl_xor(lo, off, 64));
+            hi = fmaxf(hi, __shfl_xor(hi, off, 64));
+        }
+        const int wave = threadIdx.x >> 6;
+        __syncthreads();  // the previous use of red has been read
+        if ((threadIdx.x & 63) == 0) { red[wave][0] = lo; red[wave][1] = hi; }
+        __syncthreads();
+        lo = fminf(fminf(red[0][0], red[1][0]), fminf(red[2][0], red[3][0]));
+        hi = fmaxf(fmaxf(red[0][1], red[1][1]), fmaxf(red[2][1], red[3][1]));
+    }
+}
+
+// x[8] -> uint8 codes with the block's (scale, max); returns them packed, 8 bytes
+__device__ __forceinline__ u32x2_t quantize8(const float x[8], float scale, float hi) {
+    unsigned w[2] = {0u, 0u};
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        float q = rintf((hi - x[k]) / scale);
+        q = fminf(fmaxf(q, 0.0f), 255.0f);
+        w[k >> 2] |= ((unsigned)q & 0xFFu) << (8 * (k & 3));
+    }
+    return u32x2_t{w[0], w[1]};
+}
+
+template <int BS>
+__global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
+    constexpr int W = BS / 8;  // threads per block of the moments
+    __shared__ float red[4][2];
+    const long long T = (long long)blockIdx.x * 256 + threadIdx.x;
+    const bool live = T < a.n_threads;  // n is a multiple of BS: a block is all-live or all-dead
+    const long long Tc = live ? T : 0;
+    const long long blk = Tc / W;
+    const u32x4_t g4 = a.grad[Tc];
+    const u32x2_t q1 = a.state1[Tc], q2 = a.state2[Tc];
+    const float sc1 = a.scale1[blk], mx1 = a.max1[blk], sc2 = a.scale2[blk], mx2 = a.max2[blk];
+    u32x4_t p4 = {0u, 0u, 0u, 0u};
+    if (a.param) p4 = a.param[Tc];
+
+    float m[8], d[8], out[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const float g = (k & 1) ? lq_bf16_hi(g4[k >> 1]) : lq_bf16_lo(g4[k >> 1]);
+        const float c1 = (float)((q1[k >> 2] >> (8 * (k & 3))) & 0xFFu);
+        const float c2 = (float)((q2[k >> 2] >> (8 * (k & 3))) & 0xFFu);
+        float mk = bf16r(mx1 - c1 * sc1);
+        const float s2 = mx2 - c2 * sc2;
+        float vk = bf16r(s2 * s2);
+        mk = bf16r(mk * a.beta1);
+        mk = bf16r(fmaf(a.one_minus_beta1, g, mk));
+        vk = bf16r(vk * a.beta2);
+        vk = bf16r(fmaf(a.one_minus_beta2 * g, g, vk));
+        float dk = bf16r(__builtin_sqrtf(vk));
+        dk = bf16r(dk + a.eps);
+        m[k] = mk;
+        d[k] = dk;
+        const float ratio = mk / dk;
+        if (a.param) {
+            const float p = (k & 1) ? lq_bf16_hi(p4[k >> 1]) : lq_bf16_lo(p4[k >> 1]);
+            out[k] = fmaf(a.neg_step, ratio, p);
+        } else {
+            out[k] = ratio;
+        }
+    }
+    if (live) {
+        const u32x4_t o = {lq_pack_bf16(out[0], out[1]), lq_pack_bf16(out[2], out[3]), lq_pack_bf16(out[4], out[5]),
+                           lq_pack_bf16(out[6], out[7])};
+        if (a.param) a.param[T] = o;
+        else a.direction[T] = o;
+    }
+
+    // the moments back to uint8 with the block's new (scale, max)
+    float lo1 = m[0], hi1 = m[0], lo2 = d[0], hi2 = d[0];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) {
+        lo1 = fminf(lo1, m[k]); hi1 = fmaxf(hi1, m[k]);
+        lo2 = fminf(lo2, d[k]); hi2 = fmaxf(hi2, d[k]);
+    }
+    block_minmax<W>(lo1, hi1, red);
+    block_minmax<W>(lo2, hi2, red);
+    const float inv255 = 1.0f / 255.0f;  // the tensor library divides by a scalar as a multiplication by its reciprocal
+    const float ns1 = (hi1 - lo1) * inv255 + 1e-10f;
+    const float ns2 = (hi2 - lo2) * inv255 + 1e-10f;
+    if (live) {
+        a.state1[T] = quantize8(m, ns1, hi1);
+        a.state2[T] = quantize8(d, ns2, hi2);
+        if (T % W == 0) {
+            a.scale1[blk] = ns1; a.max1[blk] = hi1;
+            a.scale2[blk] = ns2; a.max2[blk] = hi2;
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int lq_adam8_update(const void *grad, void *param_or_null, void *direction_or_null, uint8_t *state1,
+                               uint8_t *state2, float *scale1, float *max1, float *scale2, float *max2, int64_t n,
+                               int block_elems, double beta1, double beta2, double eps, double step_size, void *stream) {
+    LQ_REQUIRE(grad && state1 && state2 && scale1 && max1 && scale2 && max2, "lq_adam8_update: null pointer argument");
+    LQ_REQUIRE((param_or_null != nullptr) != (direction_or_null != nullptr),
+               "lq_adam8_update: exactly one of param and direction must be given");
+    LQ_REQUIRE(block_elems == 2048 || block_elems == 128, "lq_adam8_update: block must be 2048 or 128 elements, got %d",
+               block_elems);
+    LQ_REQUIRE(n > 0 && n % block_elems == 0, "lq_adam8_update: n=%lld must be a positive multiple of the block (%d)",
+               (long long)n, block_elems);
+    LQ_REQUIRE(n / 8 / 256 < 0x7FFFFFFFll, "lq_adam8_update: tensor too large");
+    LQ_REQUIRE(lq_aligned(grad, 16) && lq_aligned(state1, 8) && lq_aligned(state2, 8) &&
+                   (!param_or_null || lq_aligned(param_or_null, 16)) &&
+                   (!direction_or_null || lq_aligned(direction_or_null, 16)) && lq_aligned(scale1, 4) &&
+                   lq_aligned(max1, 4) && lq_aligned(scale2, 4) && lq_aligned(max2, 4),
+               "lq_adam8_update: grad, param, direction must be 16-byte, the moments 8-byte aligned");
+    Adam8Params a;
+    a.grad = (const u32x4_t *)grad;
+    a.param = (u32x4_t *)param_or_null;
+    a.direction = (u32x4_t *)direction_or_null;
+    a.state1 = (u32x2_t *)state1; a.state2 = (u32x2_t *)state2;
+    a.scale1 = scale1; a.max1 = max1; a.scale2 = scale2; a.max2 = max2;
+    a.n_threads = n / 8;
+    // the optimizer computes its scalars in double precision and the tensor library's kernels take them as fp32
+    a.beta1 = (float)beta1; a.one_minus_beta1 = (float)(1.0 - beta1);
+    a.beta2 = (float)beta2; a.one_minus_beta2 = (float)(1.0 - beta2);
+    a.eps = (float)eps; a.neg_step = (float)(-step_size);
+    const unsigned blocks = (unsigned)((a.n_threads + 255) / 256);
+    if (block_elems == 2048)
+        hipLaunchKernelGGL(adam8_update_kernel<2048>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+    else
+        hipLaunchKernelGGL(adam8_update_kernel<128>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+    return lq_check_launch("lq_adam8_update");
+}

@@ -167,6 +167,37 @@ def act_quant_i8(x, clampv):
     return out
 
 
+def adam8_update(grad, state1, state2, scale1, max1, scale2, max2, beta1, beta2, eps, step_size, param=None,
+                 direction=None):
+    """One Adam step on uint8 block-wise moments (all updated in place). Either ``param`` (bf16, updated in
+    place: param -= step_size * m / d) or ``direction`` (bf16, receives m / d) is given."""
+    _chk(grad, torch.bfloat16, "grad")
+    n = grad.numel()
+    for t, name in ((state1, "state1"), (state2, "state2")):
+        _chk(t, torch.uint8, name)
+        if t.numel() != n:
+            raise ValueError(f"{name} must hold as many elements as grad")
+    nblk = scale1.numel()
+    if nblk == 0 or n % nblk:
+        raise ValueError("the number of blocks must divide the number of elements")
+    for t, name in ((scale1, "scale1"), (max1, "max1"), (scale2, "scale2"), (max2, "max2")):
+        _chk(t, torch.float32, name)
+        if t.numel() != nblk:
+            raise ValueError(f"{name} must hold one value per block")
+    if (param is None) == (direction is None):
+        raise ValueError("give exactly one of param and direction")
+    out = param if param is not None else direction
+    _chk(out, torch.bfloat16, "param" if param is not None else "direction")
+    if out.numel() != n:
+        raise ValueError("param / direction must hold as many elements as grad")
+    with torch.cuda.device(grad.device):
+        _C.call("lq_adam8_update", grad.data_ptr(), param.data_ptr() if param is not None else None,
+                direction.data_ptr() if direction is not None else None, state1.data_ptr(), state2.data_ptr(),
+                scale1.data_ptr(), max1.data_ptr(), scale2.data_ptr(), max2.data_ptr(), n, n // nblk,
+                float(beta1), float(beta2), float(eps), float(step_size), _stream(grad))
+    return out
+
+
 def repack_gptq_to_native(qweight, shape):
     N, K = shape
     _chk(qweight, torch.int32, "qweight")

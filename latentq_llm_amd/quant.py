@@ -36,6 +36,9 @@ GROUPSIZE = 128  # utils/quant.py:44
 # kernels; False runs the reference's chain of tensor operations around the codec kernel instead
 # (same bits either way).
 FUSED_LATENT = True
+# The Adam step on uint8 moments (dequantise both moments, update them, apply the update, re-quantise
+# them per block) as one HIP kernel; False runs the chain of tensor operations (same bits either way).
+FUSED_ADAM8 = True
 EXT_type = torch.bfloat16  # utils/quant.py:722
 
 # dW travels from the autograd Functions to the full-backward hook through this list
@@ -928,6 +931,26 @@ class MyAdam(torch.optim.Adam):
             pdata = p.data
 
         q8 = state["state1"].dtype == torch.uint8
+        mu_step = (state["step"] + 1 > 250 and (state["step"] + 1) % self.mu_updata_f == (self.mu_updata_f - 1)
+                   and isinstance(getattr(p, 'residual', None), ResidualTensor))
+        if (FUSED_ADAM8 and q8 and config["weight_decay"] == 0 and not mu_step and grad.is_cuda
+                and grad.dtype == torch.bfloat16 and grad.is_contiguous()
+                and all(state[k].device == grad.device and state[k].is_contiguous()
+                        for k in ("state1", "state2", "qmap1", "absmax1", "qmap2", "absmax2"))
+                and p.numel() // len(state["absmax1"]) in (2048, 128)
+                and (sr_mode or (pdata.dtype == torch.bfloat16 and pdata.is_contiguous()))):
+            # the whole chain below as one kernel (moments, their block parameters and pdata updated in place)
+            beta1, beta2 = config["betas"]
+            state["step"] += 1
+            bias_correction1 = 1 - beta1 ** state["step"]
+            bias_correction2 = 1 - beta2 ** state["step"]
+            step_size = config["lr"] * math.sqrt(bias_correction2) / bias_correction1
+            direction = torch.empty_like(grad) if sr_mode else None
+            ops.adam8_update(grad, state["state1"], state["state2"], state["qmap1"], state["absmax1"], state["qmap2"],
+                             state["absmax2"], beta1, beta2, group["eps"], step_size,
+                             param=None if sr_mode else pdata, direction=direction)
+            self._requantise(p, pdata, direction if sr_mode else None, step_size, is_q, sr_mode)
+            return
         if q8:
             exp_avg = DeQfunc_8bit_opt(state["state1"].to(grad.device), [state["qmap1"], state["absmax1"]]).to(grad.dtype)
             s2 = DeQfunc_8bit_opt(state["state2"].to(grad.device), [state["qmap2"], state["absmax2"]])
@@ -972,6 +995,11 @@ class MyAdam(torch.optim.Adam):
             state["state1"] = exp_avg
             state["state2"] = exp_avg_sq  # holds sqrt(v) + eps after the in-place ops above, as in the reference
 
+        self._requantise(p, pdata, direction if sr_mode else None, step_size, is_q, sr_mode)
+
+    def _requantise(self, p, pdata, direction, step_size, is_q, sr_mode):
+        """Back from the updated latent weight (or, in stochastic-rounding mode, from the update
+        direction) to codes, and the gradient released (utils/quant.py:1139-1148)."""
         if is_q:
             if sr_mode:
                 scales, zeros, shape = _flat_qparam(p.qparam)

@@ -143,3 +143,43 @@ def latent_w4_requant(latent, scales, zeros, shape, curve):
     q = q.view(shape) + carry
     codes = compress(torch.clamp(q, 0, 15).to(torch.uint8))
     return codes, torch.from_numpy(words.view(np.int32).copy())
+
+
+@torch.no_grad()
+def quant_8bit_opt(tensor, nblocks):
+    """utils/quant.py:22-33 — block-wise asymmetric uint8 quantiser of an optimizer moment
+    (the reference's ``blocksize`` argument is the NUMBER of blocks)."""
+    shape = tensor.shape
+    blocks = tensor.reshape(nblocks, -1)
+    lo, hi = torch.aminmax(blocks, dim=1, keepdim=True)
+    scale = (hi - lo) / 255 + 1e-10
+    q = torch.clamp(torch.round((hi - blocks) / scale), 0, 255)
+    return q.to(torch.uint8).reshape(shape), scale, hi
+
+
+@torch.no_grad()
+def dequant_8bit_opt(q, scale, hi):
+    """utils/quant.py:35-41."""
+    return (hi - q.reshape(scale.shape[0], -1).to(torch.float32) * scale).reshape(q.shape)
+
+
+@torch.no_grad()
+def adam8_step(grad, state1, scale1, max1, state2, scale2, max2, beta1, beta2, eps, step_size, param=None):
+    """utils/quant.py:1081-1134 for uint8 moments and no weight decay: returns the updated parameter
+    (or, with param=None, the update direction bf16(m / d) that the stochastic-rounding requantizer
+    takes) and the re-quantised moments (state1, scale1, max1, state2, scale2, max2)."""
+    nblk = scale1.shape[0]
+    exp_avg = dequant_8bit_opt(state1, scale1, max1).to(grad.dtype)
+    s2 = dequant_8bit_opt(state2, scale2, max2)
+    exp_avg_sq = (s2 * s2).to(grad.dtype)
+    exp_avg.mul_(beta1).add_(grad, alpha=1 - beta1)
+    exp_avg_sq.mul_(beta2).addcmul_(grad, grad, value=1 - beta2)
+    exp_avg_sqrt = exp_avg_sq.sqrt_()
+    denom = exp_avg_sqrt.add_(eps)
+    if param is not None:
+        out = param.clone().addcdiv_(exp_avg, denom, value=-step_size)
+    else:
+        out = (exp_avg / denom).to(torch.bfloat16)
+    q1, sc1, mx1 = quant_8bit_opt(exp_avg.float(), nblk)
+    q2, sc2, mx2 = quant_8bit_opt(exp_avg_sqrt.float(), nblk)
+    return out, (q1, sc1, mx1, q2, sc2, mx2)

@@ -54,6 +54,12 @@ def test_bad_arguments_are_rejected_without_a_gpu(hip_lib):
     assert lib.lq_latent_w4_reconstruct(p, p, p, res, p, 8, 128, 128, 2, 0.3, 2, 0.25, 4, None) == -1
     assert b"b1 < b2" in lib.lq_last_error()
     assert lib.lq_calib_copy(p, p, 10, None) == -1
+    assert lib.lq_adam8_update(p, p, p, p, p, p, p, p, p, 2048, 2048, 0.9, 0.95, 1e-8, 1e-3, None) == -1
+    assert b"exactly one of param and direction" in lib.lq_last_error()
+    assert lib.lq_adam8_update(p, p, None, p, p, p, p, p, p, 2048, 512, 0.9, 0.95, 1e-8, 1e-3, None) == -1
+    assert b"2048 or 128" in lib.lq_last_error()
+    assert lib.lq_adam8_update(p, p, None, p, p, p, p, p, p, 3000, 2048, 0.9, 0.95, 1e-8, 1e-3, None) == -1
+    assert b"multiple of the block" in lib.lq_last_error()
     with pytest.raises(_C.LatentQError, match="lq_a16w4_dequant"):
         _C.call("lq_a16w4_dequant", None, None, None, None, 1, 128, 128, None)
 
