@@ -228,8 +228,18 @@ def bench_adam8(device):
         q.Qfunc_8bit_opt(m.float(), blocksize=nblk)
         q.Qfunc_8bit_opt(d.float(), blocksize=nblk)
     sec_chain = event_time(chain, 5, warm=2)
+    # the whole optimizer step of an lbit = 4 layer as one kernel: codes + residual words in and out
+    N, K = 8192, 2048
+    codes, scales, zeros = synth_w4(N, K, 7, device)
+    res = torch.randint(-2**31, 2**31 - 1, (n // 8,), device=device, dtype=torch.int64).to(torch.int32)
+    curve = (2, 0.1875, 3, 0.375, 3)
+    sec_step = event_time(lambda: ops.adam8_latent_w4_step(grad, codes, res, scales.view(-1), zeros.view(-1), (N, K), s1, s2,
+                                                           sc1, mx1, sc2, mx2, curve, curve, 0.9, 0.95, 1e-8, 1e-3), 20)
+    step_bytes = 6 * n + 32 * nblk + 4 * n // 128
     return {"elements": n, "block": block, "bytes": nbytes, "us": sec * 1e6, "GB/s": nbytes / sec / 1e9,
-            "frac_hbm": nbytes / sec / PEAK_HBM, "tensor_op_chain_us": sec_chain * 1e6}
+            "frac_hbm": nbytes / sec / PEAK_HBM, "tensor_op_chain_us": sec_chain * 1e6,
+            "latent_w4_step": {"bytes": step_bytes, "us": sec_step * 1e6, "GB/s": step_bytes / sec_step / 1e9,
+                               "frac_hbm": step_bytes / sec_step / PEAK_HBM}}
 
 
 def bench_copy(device):

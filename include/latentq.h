@@ -180,6 +180,21 @@ int lq_adam8_update(const void *grad, void *param_or_null, void *direction_or_nu
                     float *scale1, float *max1, float *scale2, float *max2, int64_t n, int block_elems, double beta1,
                     double beta2, double eps, double step_size, void *stream);
 
+/* The same step for an A16W4 layer in its exact 4-bit-residual mode (lbit = 4), with the two passes
+ * around it folded in: the parameter is rebuilt from codes and residual words exactly as
+ * lq_latent_w4_reconstruct does (curve dk1..dk3: the one the residual was stored with), updated,
+ * and re-quantised exactly as lq_latent_w4_requant does (curve qk1..qk3: the current one). One call
+ * replaces ResidualTensor.add(DeQfunc_4bit_g(...)), the Adam chain and Qfunc_4bit_g_res of
+ * MyAdam.update_step (utils/quant.py:1066-1144). codes (native layout, N*K/2 bytes) and residual
+ * (int32[N*K/8]) are updated in place and need 4-byte alignment; the rest as lq_adam8_update
+ * with n = N*K.
+ */
+int lq_adam8_latent_w4_step(const void *grad, void *codes, int32_t *residual, const void *scales, const void *zeros,
+                            uint8_t *state1, uint8_t *state2, float *scale1, float *max1, float *scale2, float *max2,
+                            int64_t N, int64_t K, int group, int block_elems, int dk1, float db1, int dk2, float db2,
+                            int dk3, int qk1, float qb1, int qk2, float qb2, int qk3, double beta1, double beta2,
+                            double eps, double step_size, void *stream);
+
 /* ---------------------------------------------------------------------------
  * Layout converters (device side).
  * GPTQ layout (reference PTQ/quant/quant_linear.py:343-389): qweight is

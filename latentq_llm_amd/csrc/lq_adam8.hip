@@ -18,11 +18,18 @@
 // equal the chain's bit for bit: 8 elements per thread (16 bytes of gradient and parameter, 8
 // bytes of each moment), the block's minimum and maximum found by a reduction over the BS/8
 // threads of the block, 6 bytes read and 4 written per element instead of ~120.
-#include "lq_common.h"
+//
+// In its latent mode the kernel also takes over the two passes around the step in the exact
+// 4-bit-residual mode of the A16W4 layer: the parameter is rebuilt from codes and residual words
+// (as lq_latent_w4_reconstruct does) and the updated value goes straight back to codes and
+// residual words (as lq_latent_w4_requant does); a thread's 8 elements are one code word and one
+// residual word. The whole optimizer step of a layer is then one pass over 4 + 4 bytes of codes
+// and residual, 16 of gradient and 16 of moments per 8 elements.
+#include "lq_latent_math.h"
 
 namespace {
 
-__device__ __forceinline__ float bf16r(float v) { return lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(v)); }
+__device__ __forceinline__ float bf16r(float v) { return lq_bf16r(v); }
 
 struct Adam8Params {
     const u32x4_t *grad;     // bf16
@@ -32,6 +39,10 @@ struct Adam8Params {
     float *scale1, *max1, *scale2, *max2;  // per block, updated in place
     long long n_threads;     // elements / 8
     float beta1, one_minus_beta1, beta2, one_minus_beta2, eps, neg_step;
+    // latent mode: the parameter lives as codes + residual words (one of each per thread)
+    unsigned *codes, *residual;
+    const unsigned short *wscales, *wzeros;  // per group of 128 elements
+    CodecParams dequant_curve, quant_curve;
 };
 
 // minimum and maximum over the W threads that share a block (W = 16: one 16-lane row of the
@@ -70,7 +81,7 @@ __device__ __forceinline__ u32x2_t quantize8(const float x[8], float scale, floa
     return u32x2_t{w[0], w[1]};
 }
 
-template <int BS>
+template <int BS, bool LATENT>
 __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
     constexpr int W = BS / 8;  // threads per block of the moments
     __shared__ float red[4][2];
@@ -82,7 +93,16 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
     const u32x2_t q1 = a.state1[Tc], q2 = a.state2[Tc];
     const float sc1 = a.scale1[blk], mx1 = a.max1[blk], sc2 = a.scale2[blk], mx2 = a.max2[blk];
     u32x4_t p4 = {0u, 0u, 0u, 0u};
-    if (a.param) p4 = a.param[Tc];
+    unsigned cword = 0, rword = 0;
+    float ws = 0.0f, wz = 0.0f;
+    if constexpr (LATENT) {
+        cword = a.codes[Tc];
+        rword = a.residual[Tc];
+        ws = lq_bf16_bits_to_f32(a.wscales[Tc >> 4]);
+        wz = lq_bf16_bits_to_f32(a.wzeros[Tc >> 4]);
+    } else if (a.param) {
+        p4 = a.param[Tc];
+    }
 
     float m[8], d[8], out[8];
 #pragma unroll
@@ -102,14 +122,33 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
         m[k] = mk;
         d[k] = dk;
         const float ratio = mk / dk;
-        if (a.param) {
+        if constexpr (LATENT) {
+            const int nib = (int)((rword >> (28 - 4 * k)) & 0xFu) - 8;
+            const float p = bf16r(lq_latent_value(lq_code(cword, k), nib, ws, wz, a.dequant_curve));
+            out[k] = bf16r(fmaf(a.neg_step, ratio, p));
+        } else if (a.param) {
             const float p = (k & 1) ? lq_bf16_hi(p4[k >> 1]) : lq_bf16_lo(p4[k >> 1]);
             out[k] = fmaf(a.neg_step, ratio, p);
         } else {
             out[k] = ratio;
         }
     }
-    if (live) {
+    if constexpr (LATENT) {
+        const bool fast = (ws >= 0x1p-40f) && (ws <= 0x1p40f);
+        const float wr = 1.0f / ws;
+        unsigned cnew = 0, rnew = 0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            unsigned nib, code;
+            lq_latent_requant_elem(out[k], ws, wz, wr, fast, a.quant_curve, nib, code);
+            rnew = (rnew << 4) | nib;
+            cnew |= code << (4 * (k ^ 1));
+        }
+        if (live) {
+            a.codes[T] = cnew;
+            a.residual[T] = rnew;
+        }
+    } else if (live) {
         const u32x4_t o = {lq_pack_bf16(out[0], out[1]), lq_pack_bf16(out[2], out[3]), lq_pack_bf16(out[4], out[5]),
                            lq_pack_bf16(out[6], out[7])};
         if (a.param) a.param[T] = o;
@@ -140,37 +179,82 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
 
 }  // namespace
 
+static int adam8_check(const char *who, const void *grad, const void *state1, const void *state2, const void *scale1,
+                       const void *max1, const void *scale2, const void *max2, int64_t n, int block_elems) {
+    LQ_REQUIRE(grad && state1 && state2 && scale1 && max1 && scale2 && max2, "%s: null pointer argument", who);
+    LQ_REQUIRE(block_elems == 2048 || block_elems == 128, "%s: block must be 2048 or 128 elements, got %d", who, block_elems);
+    LQ_REQUIRE(n > 0 && n % block_elems == 0, "%s: n=%lld must be a positive multiple of the block (%d)", who, (long long)n,
+               block_elems);
+    LQ_REQUIRE(n / 8 / 256 < 0x7FFFFFFFll, "%s: tensor too large", who);
+    LQ_REQUIRE(lq_aligned(grad, 16) && lq_aligned(state1, 8) && lq_aligned(state2, 8) && lq_aligned(scale1, 4) &&
+                   lq_aligned(max1, 4) && lq_aligned(scale2, 4) && lq_aligned(max2, 4),
+               "%s: grad must be 16-byte, the moments 8-byte aligned", who);
+    return LQ_OK;
+}
+
+static void adam8_scalars(Adam8Params &a, double beta1, double beta2, double eps, double step_size) {
+    // the optimizer computes its scalars in double precision and the tensor library's kernels take them as fp32
+    a.beta1 = (float)beta1; a.one_minus_beta1 = (float)(1.0 - beta1);
+    a.beta2 = (float)beta2; a.one_minus_beta2 = (float)(1.0 - beta2);
+    a.eps = (float)eps; a.neg_step = (float)(-step_size);
+}
+
 extern "C" int lq_adam8_update(const void *grad, void *param_or_null, void *direction_or_null, uint8_t *state1,
                                uint8_t *state2, float *scale1, float *max1, float *scale2, float *max2, int64_t n,
                                int block_elems, double beta1, double beta2, double eps, double step_size, void *stream) {
-    LQ_REQUIRE(grad && state1 && state2 && scale1 && max1 && scale2 && max2, "lq_adam8_update: null pointer argument");
+    int rc = adam8_check("lq_adam8_update", grad, state1, state2, scale1, max1, scale2, max2, n, block_elems);
+    if (rc) return rc;
     LQ_REQUIRE((param_or_null != nullptr) != (direction_or_null != nullptr),
                "lq_adam8_update: exactly one of param and direction must be given");
-    LQ_REQUIRE(block_elems == 2048 || block_elems == 128, "lq_adam8_update: block must be 2048 or 128 elements, got %d",
-               block_elems);
-    LQ_REQUIRE(n > 0 && n % block_elems == 0, "lq_adam8_update: n=%lld must be a positive multiple of the block (%d)",
-               (long long)n, block_elems);
-    LQ_REQUIRE(n / 8 / 256 < 0x7FFFFFFFll, "lq_adam8_update: tensor too large");
-    LQ_REQUIRE(lq_aligned(grad, 16) && lq_aligned(state1, 8) && lq_aligned(state2, 8) &&
-                   (!param_or_null || lq_aligned(param_or_null, 16)) &&
-                   (!direction_or_null || lq_aligned(direction_or_null, 16)) && lq_aligned(scale1, 4) &&
-                   lq_aligned(max1, 4) && lq_aligned(scale2, 4) && lq_aligned(max2, 4),
-               "lq_adam8_update: grad, param, direction must be 16-byte, the moments 8-byte aligned");
-    Adam8Params a;
+    LQ_REQUIRE((!param_or_null || lq_aligned(param_or_null, 16)) && (!direction_or_null || lq_aligned(direction_or_null, 16)),
+               "lq_adam8_update: param and direction must be 16-byte aligned");
+    Adam8Params a = {};
     a.grad = (const u32x4_t *)grad;
     a.param = (u32x4_t *)param_or_null;
     a.direction = (u32x4_t *)direction_or_null;
     a.state1 = (u32x2_t *)state1; a.state2 = (u32x2_t *)state2;
     a.scale1 = scale1; a.max1 = max1; a.scale2 = scale2; a.max2 = max2;
     a.n_threads = n / 8;
-    // the optimizer computes its scalars in double precision and the tensor library's kernels take them as fp32
-    a.beta1 = (float)beta1; a.one_minus_beta1 = (float)(1.0 - beta1);
-    a.beta2 = (float)beta2; a.one_minus_beta2 = (float)(1.0 - beta2);
-    a.eps = (float)eps; a.neg_step = (float)(-step_size);
+    adam8_scalars(a, beta1, beta2, eps, step_size);
     const unsigned blocks = (unsigned)((a.n_threads + 255) / 256);
     if (block_elems == 2048)
-        hipLaunchKernelGGL(adam8_update_kernel<2048>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+        hipLaunchKernelGGL((adam8_update_kernel<2048, false>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
     else
-        hipLaunchKernelGGL(adam8_update_kernel<128>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+        hipLaunchKernelGGL((adam8_update_kernel<128, false>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
     return lq_check_launch("lq_adam8_update");
+}
+
+extern "C" int lq_adam8_latent_w4_step(const void *grad, void *codes, int32_t *residual, const void *scales,
+                                       const void *zeros, uint8_t *state1, uint8_t *state2, float *scale1, float *max1,
+                                       float *scale2, float *max2, int64_t N, int64_t K, int group, int block_elems,
+                                       int dk1, float db1, int dk2, float db2, int dk3, int qk1, float qb1, int qk2,
+                                       float qb2, int qk3, double beta1, double beta2, double eps, double step_size,
+                                       void *stream) {
+    LQ_REQUIRE(N > 0 && K > 0 && K % LQ_GROUP == 0, "lq_adam8_latent_w4_step: need N > 0, K a positive multiple of %d",
+               LQ_GROUP);
+    LQ_REQUIRE(group == LQ_GROUP, "lq_adam8_latent_w4_step: group must be %d", LQ_GROUP);
+    const int64_t n = N * K;
+    int rc = adam8_check("lq_adam8_latent_w4_step", grad, state1, state2, scale1, max1, scale2, max2, n, block_elems);
+    if (rc) return rc;
+    LQ_REQUIRE(codes && residual && scales && zeros, "lq_adam8_latent_w4_step: null pointer argument");
+    LQ_REQUIRE(lq_aligned(codes, 4) && lq_aligned(residual, 4), "lq_adam8_latent_w4_step: codes and residual must be 4-byte aligned");
+    LQ_REQUIRE(dk1 > 0 && dk2 > 0 && dk3 > 0 && db1 > 0.0f && db2 > db1 && db2 < 0.5f && qk1 > 0 && qk2 > 0 && qk3 > 0 &&
+                   qb1 > 0.0f && qb2 > qb1 && qb2 < 0.5f,
+               "lq_adam8_latent_w4_step: need k1,k2,k3 > 0 and 0 < b1 < b2 < 0.5 for both curves");
+    Adam8Params a = {};
+    a.grad = (const u32x4_t *)grad;
+    a.state1 = (u32x2_t *)state1; a.state2 = (u32x2_t *)state2;
+    a.scale1 = scale1; a.max1 = max1; a.scale2 = scale2; a.max2 = max2;
+    a.n_threads = n / 8;
+    a.codes = (unsigned *)codes; a.residual = (unsigned *)residual;
+    a.wscales = (const unsigned short *)scales; a.wzeros = (const unsigned short *)zeros;
+    a.dequant_curve = lq_codec_dequant_params(dk1, db1, dk2, db2, dk3);
+    a.quant_curve = lq_codec_quant_params(qk1, qb1, qk2, qb2, qk3);
+    adam8_scalars(a, beta1, beta2, eps, step_size);
+    const unsigned blocks = (unsigned)((a.n_threads + 255) / 256);
+    if (block_elems == 2048)
+        hipLaunchKernelGGL((adam8_update_kernel<2048, true>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+    else
+        hipLaunchKernelGGL((adam8_update_kernel<128, true>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+    return lq_check_launch("lq_adam8_latent_w4_step");
 }

@@ -13,12 +13,9 @@
 //   reconstruct:  w = bf16(bf16(q - z) * s);  r = bf16(bf16(value(nibble)) * s);  latent = bf16(r + w)
 //   requant:      Z = bf16(bf16(t / s) + z);  q = rint(Z);  f = bf16(Z - q)
 //                 (nibble, carry) = codec(f);  code = clamp(bf16(q + carry), 0, 15)
-#include "lq_common.h"
-#include "lq_residual_codec.h"
+#include "lq_latent_math.h"
 
 namespace {
-
-__device__ __forceinline__ float bf16r(float v) { return lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(v)); }
 
 // A thread owns 32 consecutive elements of one quantisation group: 16 bytes of codes, 16 bytes of
 // residual words, 64 bytes of latent; one scale and zero per thread.
@@ -38,10 +35,8 @@ __global__ __launch_bounds__(256) void latent_reconstruct_kernel(const u32x4_t *
         float v[8];
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            const float wq = bf16r(bf16r((float)lq_code(cw[i], k) - z) * s);
             const int nib = (int)((rw[i] >> (28 - 4 * k)) & 0xFu) - 8;
-            const float r = bf16r(bf16r(value_3fold(nib, p)) * s);
-            v[k] = r + wq;
+            v[k] = lq_latent_value(lq_code(cw[i], k), nib, s, z, p);
         }
         latent[L * 4 + i] = u32x4_t{lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3]), lq_pack_bf16(v[4], v[5]),
                                     lq_pack_bf16(v[6], v[7])};
@@ -60,10 +55,6 @@ __global__ __launch_bounds__(256) void latent_requant_kernel(const u32x4_t *__re
     for (int i = 0; i < 4; ++i) in[i] = latent[L * 4 + i];
     const float s = lq_bf16_bits_to_f32(scales[L >> 2]);
     const float z = lq_bf16_bits_to_f32(zeros[L >> 2]);
-    // t / s, correctly rounded. For 2^-40 <= s <= 2^40 the quotient comes from the correctly rounded
-    // reciprocal (q0 = t*r, e = t - q0*s exactly, q = q0 + e*r: three operations instead of a
-    // division sequence); |t| is clamped to 2^60 first, which keeps t*r finite and changes nothing
-    // downstream (any |Z| >= 2^20 is an integer in bf16: zero residual, saturated code).
     const bool fast = (s >= 0x1p-40f) && (s <= 0x1p40f);
     const float r = 1.0f / s;
     u32x4_t cout, rout;
@@ -73,23 +64,10 @@ __global__ __launch_bounds__(256) void latent_requant_kernel(const u32x4_t *__re
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             const float t = (k & 1) ? lq_bf16_hi(in[i][k >> 1]) : lq_bf16_lo(in[i][k >> 1]);
-            float quo;
-            if (fast && t == t) {
-                const float tc = __builtin_amdgcn_fmed3f(t, -0x1p60f, 0x1p60f);
-                const float q0 = tc * r;
-                quo = fmaf(fmaf(-q0, s, tc), r, q0);
-            } else {
-                quo = t / s;
-            }
-            const float Z = bf16r(bf16r(quo) + z);
-            const float q = rintf(Z);  // round half to even, as torch.round
-            const float f = bf16r(Z - q);
-            bool carry;
-            const unsigned nib = nibble_of(level_3fold(f, p), carry);
+            unsigned nib, code;
+            lq_latent_requant_elem(t, s, z, r, fast, p, nib, code);
             rword = (rword << 4) | nib;
-            float c = bf16r(q + (carry ? 1.0f : 0.0f));
-            c = fminf(fmaxf(c, 0.0f), 15.0f);
-            cword |= ((unsigned)c & 0xFu) << (4 * (k ^ 1));
+            cword |= code << (4 * (k ^ 1));
         }
         cout[i] = cword;
         rout[i] = rword;

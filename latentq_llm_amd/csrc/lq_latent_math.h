@@ -1,0 +1,41 @@
+// Per-element arithmetic of the lbit = 4 latent weight (codes + 4-bit residual), shared by the
+// latent passes (lq_latent.hip) and the fused optimizer step (lq_adam8.hip). Every line is one
+// tensor operation of the reference's chains (utils/quant.py:45-72, 803-837) with its bf16 rounding.
+#pragma once
+#include "lq_common.h"
+#include "lq_residual_codec.h"
+
+__device__ __forceinline__ float lq_bf16r(float v) { return lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(v)); }
+
+// latent = bf16(bf16(bf16(value(nibble)) * s) + bf16(bf16(q - z) * s)); the caller applies the last rounding
+__device__ __forceinline__ float lq_latent_value(unsigned code, int nib, float s, float z, const CodecParams &pd) {
+    const float wq = lq_bf16r(lq_bf16r((float)code - z) * s);
+    const float r = lq_bf16r(lq_bf16r(value_3fold(nib, pd)) * s);
+    return r + wq;
+}
+
+// One element of the re-quantiser: Z = bf16(bf16(t / s) + z), q = rint(Z), residual nibble and
+// carry from bf16(Z - q), code = clamp(bf16(q + carry), 0, 15).
+// t / s is correctly rounded: for 2^-40 <= s <= 2^40 (fast) the quotient comes from the correctly
+// rounded reciprocal r (q0 = t*r, e = t - q0*s exactly, q = q0 + e*r: three operations instead of a
+// division sequence); |t| is clamped to 2^60 first, which keeps t*r finite and changes nothing
+// downstream (any |Z| >= 2^20 is an integer in bf16: zero residual, saturated code).
+__device__ __forceinline__ void lq_latent_requant_elem(float t, float s, float z, float r, bool fast, const CodecParams &pq,
+                                                       unsigned &nib, unsigned &code) {
+    float quo;
+    if (fast && t == t) {
+        const float tc = __builtin_amdgcn_fmed3f(t, -0x1p60f, 0x1p60f);
+        const float q0 = tc * r;
+        quo = fmaf(fmaf(-q0, s, tc), r, q0);
+    } else {
+        quo = t / s;
+    }
+    const float Z = lq_bf16r(lq_bf16r(quo) + z);
+    const float q = rintf(Z);  // round half to even, as torch.round
+    const float f = lq_bf16r(Z - q);
+    bool carry;
+    nib = nibble_of(level_3fold(f, pq), carry);
+    float c = lq_bf16r(q + (carry ? 1.0f : 0.0f));
+    c = fminf(fmaxf(c, 0.0f), 15.0f);
+    code = (unsigned)c & 0xFu;
+}

@@ -198,6 +198,44 @@ def adam8_update(grad, state1, state2, scale1, max1, scale2, max2, beta1, beta2,
     return out
 
 
+def adam8_latent_w4_step(grad, codes, residual_int, scales, zeros, shape, state1, state2, scale1, max1, scale2, max2,
+                         dequant_curve, quant_curve, beta1, beta2, eps, step_size):
+    """The Adam step of an lbit = 4 layer in one pass: codes (packed, N*K/2 bytes), residual_int
+    (int32[N*K/8]) and the uint8 moments with their block parameters are all updated in place.
+    The curves are (k1, b1, k2, b2, k3) tuples: the one the residual was stored with and the
+    current one."""
+    N, K = shape
+    _chk(grad, torch.bfloat16, "grad")
+    if grad.numel() != N * K:
+        raise ValueError("grad must hold N*K elements")
+    _codes_ok(codes, N, K)
+    _qparam_ok(scales, zeros, N, K)
+    _chk(residual_int, torch.int32, "residual_int")
+    if residual_int.numel() != N * K // 8:
+        raise ValueError("residual_int must hold N*K/8 words")
+    n = N * K
+    for t, name in ((state1, "state1"), (state2, "state2")):
+        _chk(t, torch.uint8, name)
+        if t.numel() != n:
+            raise ValueError(f"{name} must hold N*K elements")
+    nblk = scale1.numel()
+    if nblk == 0 or n % nblk:
+        raise ValueError("the number of blocks must divide the number of elements")
+    for t, name in ((scale1, "scale1"), (max1, "max1"), (scale2, "scale2"), (max2, "max2")):
+        _chk(t, torch.float32, name)
+        if t.numel() != nblk:
+            raise ValueError(f"{name} must hold one value per block")
+    d, q = dequant_curve, quant_curve
+    with torch.cuda.device(grad.device):
+        _C.call("lq_adam8_latent_w4_step", grad.data_ptr(), codes.data_ptr(), residual_int.data_ptr(), scales.data_ptr(),
+                zeros.data_ptr(), state1.data_ptr(), state2.data_ptr(), scale1.data_ptr(), max1.data_ptr(),
+                scale2.data_ptr(), max2.data_ptr(), N, K, 128, n // nblk,
+                int(d[0]), float(d[1]), int(d[2]), float(d[3]), int(d[4]),
+                int(q[0]), float(q[1]), int(q[2]), float(q[3]), int(q[4]),
+                float(beta1), float(beta2), float(eps), float(step_size), _stream(grad))
+    return codes
+
+
 def repack_gptq_to_native(qweight, shape):
     N, K = shape
     _chk(qweight, torch.int32, "qweight")

@@ -923,22 +923,24 @@ class MyAdam(torch.optim.Adam):
         grad = p.grad
         is_q = isinstance(p, QuantTensor)
         sr_mode = is_q and p.wbit == 4 and p.residual is None
+        if is_q and isinstance(grad, GradientQTensor):
+            grad = grad.get_value()
+        q8 = state["state1"].dtype == torch.uint8
+        mu_step = (state["step"] + 1 > 250 and (state["step"] + 1) % self.mu_updata_f == (self.mu_updata_f - 1)
+                   and isinstance(getattr(p, 'residual', None), ResidualTensor))
+        adam8_ok = (FUSED_ADAM8 and q8 and config["weight_decay"] == 0 and not mu_step and grad.is_cuda
+                    and grad.dtype == torch.bfloat16 and grad.is_contiguous()
+                    and all(state[k].device == grad.device and state[k].is_contiguous()
+                            for k in ("state1", "state2", "qmap1", "absmax1", "qmap2", "absmax2"))
+                    and p.numel() // len(state["absmax1"]) in (2048, 128))
+        if adam8_ok and FUSED_LATENT and is_q and not sr_mode and self._fused_latent_step(group, p, state, config, grad):
+            return
         if is_q:
-            if isinstance(grad, GradientQTensor):
-                grad = grad.get_value()
             pdata = None if sr_mode else self._latent(p, grad.dtype)
         else:
             pdata = p.data
 
-        q8 = state["state1"].dtype == torch.uint8
-        mu_step = (state["step"] + 1 > 250 and (state["step"] + 1) % self.mu_updata_f == (self.mu_updata_f - 1)
-                   and isinstance(getattr(p, 'residual', None), ResidualTensor))
-        if (FUSED_ADAM8 and q8 and config["weight_decay"] == 0 and not mu_step and grad.is_cuda
-                and grad.dtype == torch.bfloat16 and grad.is_contiguous()
-                and all(state[k].device == grad.device and state[k].is_contiguous()
-                        for k in ("state1", "state2", "qmap1", "absmax1", "qmap2", "absmax2"))
-                and p.numel() // len(state["absmax1"]) in (2048, 128)
-                and (sr_mode or (pdata.dtype == torch.bfloat16 and pdata.is_contiguous()))):
+        if adam8_ok and (sr_mode or (pdata.dtype == torch.bfloat16 and pdata.is_contiguous())):
             # the whole chain below as one kernel (moments, their block parameters and pdata updated in place)
             beta1, beta2 = config["betas"]
             state["step"] += 1
@@ -996,6 +998,36 @@ class MyAdam(torch.optim.Adam):
             state["state2"] = exp_avg_sq  # holds sqrt(v) + eps after the in-place ops above, as in the reference
 
         self._requantise(p, pdata, direction if sr_mode else None, step_size, is_q, sr_mode)
+
+    def _fused_latent_step(self, group, p, state, config, grad):
+        """The whole step of an lbit = 4 layer (latent from codes + residual, Adam on uint8 moments,
+        back to codes + residual) as one kernel, when every piece is in the form the kernel takes;
+        returns False to let the separate passes run."""
+        r = p.residual
+        if not (p.wbit == 4 and isinstance(r, ResidualTensor) and not r.init and p.data.is_cuda
+                and p.data.is_contiguous() and r.residual_int.is_cuda and r.residual_int.is_contiguous()):
+            return False
+        scales, zeros, shape = _flat_qparam(p.qparam)
+        if not (scales.dtype == torch.bfloat16 and zeros.dtype == torch.bfloat16 and scales.is_contiguous()
+                and zeros.is_contiguous() and r.weight_scale is not None and r.weight_scale.dtype == torch.bfloat16
+                and r.weight_scale.data_ptr() == scales.data_ptr() and r.weight_scale.numel() == scales.numel()):
+            return False
+        beta1, beta2 = config["betas"]
+        state["step"] += 1
+        step_size = config["lr"] * math.sqrt(1 - beta2 ** state["step"]) / (1 - beta1 ** state["step"])
+        p1, y1, p2, y2 = three_fold_curve_4bit(r.lock_mu)
+        q1, z1, q2, z2 = three_fold_curve_4bit(r.mu)
+        ops.adam8_latent_w4_step(grad, p.data, r.residual_int.view(-1), scales, zeros, tuple(shape), state["state1"],
+                                 state["state2"], state["qmap1"], state["absmax1"], state["qmap2"], state["absmax2"],
+                                 (p1, y1, p2 - p1, y2, 8 - p2), (q1, z1, q2 - q1, z2, 8 - q2), beta1, beta2,
+                                 group["eps"], step_size)
+        r.weight_scale = scales.contiguous().reshape(-1, 1)
+        r.lock_mu = r.mu
+        if isinstance(p.grad, GradientQTensor):
+            p.grad.zero()
+        else:
+            p.grad = None
+        return True
 
     def _requantise(self, p, pdata, direction, step_size, is_q, sr_mode):
         """Back from the updated latent weight (or, in stochastic-rounding mode, from the update

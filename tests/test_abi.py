@@ -60,6 +60,9 @@ def test_bad_arguments_are_rejected_without_a_gpu(hip_lib):
     assert b"2048 or 128" in lib.lq_last_error()
     assert lib.lq_adam8_update(p, p, None, p, p, p, p, p, p, 3000, 2048, 0.9, 0.95, 1e-8, 1e-3, None) == -1
     assert b"multiple of the block" in lib.lq_last_error()
+    assert lib.lq_adam8_latent_w4_step(p, p, res, p, p, p, p, p, p, p, p, 16, 128, 128, 2048, 2, 0.125, 2, 0.25, 4,
+                                       2, 0.3, 2, 0.25, 4, 0.9, 0.95, 1e-8, 1e-3, None) == -1
+    assert b"b1 < b2" in lib.lq_last_error()
     with pytest.raises(_C.LatentQError, match="lq_a16w4_dequant"):
         _C.call("lq_a16w4_dequant", None, None, None, None, 1, 128, 128, None)
 

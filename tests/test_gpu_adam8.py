@@ -106,25 +106,31 @@ def _run_module_steps(Q, fused, lbit, steps=5):
         opt.step()
     st = opt.state[layer.weight]
     assert st["state1"].dtype == torch.uint8
-    return (layer.weight.data.clone().cpu(), st["state1"].clone().cpu(), st["state2"].clone().cpu(),
+    res = getattr(layer.weight, "residual", None)
+    res_words = res.residual_int.clone().cpu() if res is not None and hasattr(res, "residual_int") else torch.zeros(1)
+    return (layer.weight.data.clone().cpu(), res_words, st["state1"].clone().cpu(), st["state2"].clone().cpu(),
             st["qmap1"].clone().cpu(), st["absmax1"].clone().cpu(), st["qmap2"].clone().cpu(), st["absmax2"].clone().cpu())
 
 
 @pytest.mark.parametrize("lbit", [4, 0])
 def test_optimizer_steps_with_fused_adam8_equal_the_chain(ops, monkeypatch, lbit):
     """Whole optimizer steps of the module path (latent mode lbit=4 and the stochastic-rounding mode
-    lbit=0): codes, moments and block parameters identical with the fused kernel on and off, and
-    the fused kernel is what ran."""
+    lbit=0): codes, moments and block parameters identical with the fused kernels on and off, and
+    the fused kernels are what ran: in latent mode the single-kernel step from the second step on
+    (the first has no stored residual yet), otherwise the Adam kernel."""
     from latentq_llm_amd import ops as O
     from latentq_llm_amd import quant as Q
-    calls = {"n": 0}
-    real = O.adam8_update
-    monkeypatch.setattr(O, "adam8_update", lambda *a, **k: (calls.__setitem__("n", calls["n"] + 1), real(*a, **k))[1])
+    calls = {"adam": 0, "step": 0}
+    real_adam, real_step = O.adam8_update, O.adam8_latent_w4_step
+    monkeypatch.setattr(O, "adam8_update", lambda *a, **k: (calls.__setitem__("adam", calls["adam"] + 1), real_adam(*a, **k))[1])
+    monkeypatch.setattr(O, "adam8_latent_w4_step",
+                        lambda *a, **k: (calls.__setitem__("step", calls["step"] + 1), real_step(*a, **k))[1])
+    expect = {"adam": 1, "step": 4} if lbit == 4 else {"adam": 5, "step": 0}
     try:
         a = _run_module_steps(Q, True, lbit)
-        assert calls["n"] == 5
+        assert calls == expect
         b = _run_module_steps(Q, False, lbit)
-        assert calls["n"] == 5
+        assert calls == expect
     finally:
         Q.FUSED_ADAM8 = True
     for x, y in zip(a, b):
@@ -161,3 +167,40 @@ def test_fused_adam8_against_the_cpu_oracle(ops):
         # carry on from the oracle's state so that differences do not accumulate
         dst = [t.clone().to(dev) for t in st]
         dp = p.clone().to(dev)
+
+
+@pytest.mark.parametrize("N,K,block", [(64, 2048, 2048), (257, 384, 128), (1024, 4096, 2048)])
+def test_single_kernel_latent_step_equals_the_three_passes(ops, N, K, block):
+    """lq_adam8_latent_w4_step against lq_latent_w4_reconstruct -> lq_adam8_update -> lq_latent_w4_requant,
+    with different curves for the stored residual and for the new one (as after an update of the
+    codec's range), over several steps: codes, residual words, moments and block parameters identical."""
+    from latentq_llm_amd import quant as q
+    from tests.util import make_w4
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(N + K)
+    n = N * K
+    nblk = n // block
+    codes, packed, scales, zeros = make_w4(N, K, 5)
+    scales, zeros = scales.to(dev).view(-1), zeros.to(dev).view(-1)
+    res = torch.randint(-2**31, 2**31 - 1, (n // 8,), generator=g, dtype=torch.int64).to(torch.int32).to(dev)
+    a = {"codes": packed.clone().to(dev), "res": res.clone(), **fresh_state(n, nblk, dev)}
+    b = {"codes": packed.clone().to(dev), "res": res.clone(), **fresh_state(n, nblk, dev)}
+
+    def curve(mu):
+        p1, y1, p2, y2 = q.three_fold_curve_4bit(mu)
+        return (p1, y1, p2 - p1, y2, 8 - p2)
+    curves = [curve(0), curve(1), curve(1), curve(2), curve(0)]
+    for step in range(1, 5):
+        grad = (torch.randn(n, generator=g) * 10.0 ** torch.randint(-5, -1, (n,), generator=g).float()).to(torch.bfloat16).to(dev)
+        step_size = 2e-3 * math.sqrt(1 - 0.95 ** step) / (1 - 0.9 ** step)
+        dq, qq = curves[step - 1], curves[step]
+        latent = ops.latent_w4_reconstruct(a["codes"], scales, zeros, a["res"], (N, K), *dq)
+        ops.adam8_update(grad, a["state1"], a["state2"], a["qmap1"], a["absmax1"], a["qmap2"], a["absmax2"],
+                         0.9, 0.95, 1e-8, step_size, param=latent.view(-1))
+        a["codes"] = ops.latent_w4_requant(latent, scales, zeros, a["res"], (N, K), *qq)
+        ops.adam8_latent_w4_step(grad, b["codes"], b["res"], scales, zeros, (N, K), b["state1"], b["state2"], b["qmap1"],
+                                 b["absmax1"], b["qmap2"], b["absmax2"], dq, qq, 0.9, 0.95, 1e-8, step_size)
+        torch.cuda.synchronize()
+        for name in a:
+            assert torch.equal(a[name].view(-1), b[name].view(-1)), f"step {step}: {name} differs"
+    assert not torch.equal(b["codes"].cpu(), packed)
