@@ -290,6 +290,22 @@ def profile_target(device, which, launches=10):
             res = torch.randint(-2 ** 31, 2 ** 31 - 1, (N * K // 8,), device=device, dtype=torch.int64).to(torch.int32)
             lat = o.latent_w4_reconstruct(p, s, z, res, (N, K), *curve)
             o.latent_w4_requant(lat, s, z, res, (N, K), *curve)
+    elif which == "adam8":
+        N, K = 8192, 2048
+        n, nblk = N * K, N * K // 2048
+        curve = (2, 0.1875, 3, 0.375, 3)
+        for i in range(launches):
+            # fresh buffers per launch, so that every launch reads its operands from HBM
+            p, s, z = synth_w4(N, K, 60 + i, device)
+            res = torch.randint(-2 ** 31, 2 ** 31 - 1, (n // 8,), device=device, dtype=torch.int64).to(torch.int32)
+            grad = (torch.randn(n, device=device) * 1e-3).to(torch.bfloat16)
+            param = (torch.randn(n, device=device) * 0.02).to(torch.bfloat16)
+            s1 = torch.randint(0, 256, (n,), device=device, dtype=torch.uint8)
+            s2 = torch.randint(0, 256, (n,), device=device, dtype=torch.uint8)
+            q = [torch.full((nblk, 1), v, device=device) for v in (1e-5, 1.3e-3, 1e-5, 2.6e-3)]
+            o.adam8_update(grad, s1, s2, q[0], q[1], q[2], q[3], 0.9, 0.95, 1e-8, 1e-3, param=param)
+            o.adam8_latent_w4_step(grad, p, res, s.view(-1), z.view(-1), (N, K), s1, s2, q[0], q[1], q[2], q[3], curve, curve,
+                                   0.9, 0.95, 1e-8, 1e-3)
     elif which == "gemv":
         for (N, K) in [(4096, 4096), (11008, 4096), (4096, 11008)]:
             for M in (1, 4, 16):
@@ -359,7 +375,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-mlp", action="store_true", help="skip the side measurements (requant, GEMV, A8W8)")
-    ap.add_argument("--profile-target", choices=["gemm", "requant", "gemv", "a8w8", "latent"],
+    ap.add_argument("--profile-target", choices=["gemm", "requant", "gemv", "a8w8", "latent", "adam8"],
                     help="run only a short fixed launch sequence of one kernel family (for rocprofv3), print nothing")
     args = ap.parse_args()
     if args.gpus != 1:
