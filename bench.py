@@ -242,6 +242,24 @@ def bench_adam8(device):
                                "frac_hbm": step_bytes / sec_step / PEAK_HBM}}
 
 
+def bench_dw(device):
+    """dW = dY^T X of the two MLP shapes (not part of `value`): the vendor GEMM on the strided view, as
+    the reference calls it, against the transposed-copy form the drop-in modules use."""
+    from latentq_llm_amd import ops
+    out = []
+    for (N, K) in [(FFN, HID), (HID, FFN)]:
+        dy = torch.randn(TOKENS, N, device=device).to(torch.bfloat16)
+        x = torch.randn(TOKENS, K, device=device).to(torch.bfloat16)
+        flop = 2 * TOKENS * N * K
+        t_ref = event_time(lambda: dy.t().mm(x), 20)
+        t_tr = event_time(lambda: ops.transpose_bf16(dy), 20)
+        t_new = event_time(lambda: ops.weight_grad(dy, x), 20)
+        out.append({"N": N, "K": K, "strided_mm_us": t_ref * 1e6, "strided_mm_TFLOP/s": flop / t_ref / 1e12,
+                    "transpose_us": t_tr * 1e6, "transpose_GB/s": 4 * TOKENS * N / t_tr / 1e9,
+                    "weight_grad_us": t_new * 1e6, "weight_grad_TFLOP/s": flop / t_new / 1e12})
+    return out
+
+
 def bench_copy(device):
     """Plain streaming copy (lq_calib_copy) over buffers larger than the last-level cache: the
     HBM rate this device sustains for read + write traffic, for comparison with the 8 TB/s peak."""
@@ -441,6 +459,7 @@ def main():
         line["gemv"] = bench_gemv(dev)
         line["a8w8"] = bench_a8w8(dev)
         line["adam8"] = bench_adam8(dev)
+        line["dw"] = bench_dw(dev)
         line["hbm_copy"] = bench_copy(dev)
     line["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
     print(json.dumps(line))

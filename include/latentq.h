@@ -206,6 +206,14 @@ int lq_repack_native_to_gptq(const void *codes_native, int32_t *qweight_gptq, in
                              void *stream);
 
 /* ---------------------------------------------------------------------------
+ * dst[c][r] = src[r][c] for a row-major bf16 [R, C] matrix (R, C multiples of 8, both buffers
+ * 16-byte aligned, not overlapping). Used for the weight gradient dW = dY^T X of
+ * QLinearFunctionW4.backward (reference utils/quant.py:141-142, `grad_output.t().mm(input)`): the
+ * dense GEMM runs faster on a transposed copy of dY than on the strided view.
+ * ------------------------------------------------------------------------- */
+int lq_transpose_bf16(const void *src, void *dst, int64_t R, int64_t C, void *stream);
+
+/* ---------------------------------------------------------------------------
  * Measurement aid, no counterpart in the reference: a plain streaming copy of
  * nbytes (a multiple of 16, both pointers 16-byte aligned) from src to dst.
  * Its known traffic (nbytes read + nbytes written) calibrates the HBM byte

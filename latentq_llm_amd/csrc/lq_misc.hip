@@ -160,3 +160,49 @@ extern "C" int lq_calib_copy(const void *src, void *dst, int64_t nbytes, void *s
                        (const u32x4_t *)src, (u32x4_t *)dst, n16);
     return lq_check_launch("lq_calib_copy");
 }
+
+// ---- bf16 matrix transpose --------------------------------------------------
+// dst[c][r] = src[r][c] for a row-major [R, C] matrix, 64 x 64 tiles through LDS, 16-byte global
+// accesses on both sides. The weight gradient dW = dY^T X is a GEMM whose left operand is read
+// along its strided dimension; the vendor GEMM runs 20-35 % faster on a transposed copy of dY,
+// and this pass costs a tenth of that GEMM.
+__global__ __launch_bounds__(256) void transpose_bf16_kernel(const unsigned short *__restrict__ src,
+                                                            unsigned short *__restrict__ dst, int R, int C) {
+    __shared__ unsigned short tile[64][66];  // 132-byte rows: the column gathers below spread over the banks
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int t = threadIdx.x, sub = t >> 3, ch = (t & 7) * 8;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int r = sub + 32 * i;
+        if (r0 + r < R && c0 + ch < C) {
+            const u32x4_t v = *reinterpret_cast<const u32x4_t *>(src + (long long)(r0 + r) * C + c0 + ch);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) *reinterpret_cast<unsigned *>(&tile[r][ch + 2 * j]) = v[j];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int c = sub + 32 * i;  // output row
+        if (c0 + c < C && r0 + ch < R) {
+            u32x4_t v;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                v[j] = (unsigned)tile[ch + 2 * j][c] | ((unsigned)tile[ch + 2 * j + 1][c] << 16);
+            *reinterpret_cast<u32x4_t *>(dst + (long long)(c0 + c) * R + r0 + ch) = v;
+        }
+    }
+}
+
+extern "C" int lq_transpose_bf16(const void *src, void *dst, int64_t R, int64_t C, void *stream) {
+    LQ_REQUIRE(src && dst, "lq_transpose_bf16: null pointer argument");
+    LQ_REQUIRE(R > 0 && C > 0 && R % 8 == 0 && C % 8 == 0, "lq_transpose_bf16: R=%lld and C=%lld must be positive multiples of 8",
+               (long long)R, (long long)C);
+    LQ_REQUIRE(R < (1ll << 31) && C < (1ll << 31) && (C + 63) / 64 < 0x7FFFFFFFll && (R + 63) / 64 <= 65535 * 64ll,
+               "lq_transpose_bf16: matrix too large");
+    LQ_REQUIRE(lq_aligned(src, 16) && lq_aligned(dst, 16), "lq_transpose_bf16: buffers must be 16-byte aligned");
+    LQ_REQUIRE((R + 63) / 64 <= 65535, "lq_transpose_bf16: more than 65535 row tiles");
+    hipLaunchKernelGGL(transpose_bf16_kernel, dim3((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64)), dim3(256), 0,
+                       (hipStream_t)stream, (const unsigned short *)src, (unsigned short *)dst, (int)R, (int)C);
+    return lq_check_launch("lq_transpose_bf16");
+}

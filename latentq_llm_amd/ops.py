@@ -236,6 +236,27 @@ def adam8_latent_w4_step(grad, codes, residual_int, scales, zeros, shape, state1
     return codes
 
 
+def transpose_bf16(x):
+    """Contiguous transpose of a 2-D bf16 matrix whose sides are multiples of 8."""
+    _chk(x, torch.bfloat16, "x")
+    if x.dim() != 2 or x.shape[0] % 8 or x.shape[1] % 8:
+        raise ValueError("x must be 2-D with both sides multiples of 8")
+    R, C = x.shape
+    out = torch.empty((C, R), dtype=torch.bfloat16, device=x.device)
+    with torch.cuda.device(x.device):
+        _C.call("lq_transpose_bf16", x.data_ptr(), out.data_ptr(), R, C, _stream(x))
+    return out
+
+
+def weight_grad(dy, x):
+    """dW = dY^T X for 2-D bf16 operands: the vendor GEMM on a transposed copy of dY when the
+    shapes allow it, on the strided view otherwise."""
+    if (dy.is_cuda and dy.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and dy.dim() == 2 and dy.is_contiguous()
+            and dy.shape[0] % 8 == 0 and dy.shape[1] % 8 == 0 and dy.shape[0] >= 256):
+        return transpose_bf16(dy).mm(x)
+    return dy.t().mm(x)
+
+
 def repack_gptq_to_native(qweight, shape):
     N, K = shape
     _chk(qweight, torch.int32, "qweight")

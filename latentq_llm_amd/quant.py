@@ -188,7 +188,7 @@ class QLinearFunctionW4(torch.autograd.Function):
             grad_input = ops.a16w4_dx(dy, weight_d, scales, zeros, shape)
             if grad_input.dtype != input.dtype:
                 grad_input = grad_input.to(input.dtype)
-        dict_temp.append(grad_output.t().mm(input))
+        dict_temp.append(ops.weight_grad(grad_output, input))  # dW = dY^T X (utils/quant.py:141-142)
         if bias is not None and ctx.needs_input_grad[_BIAS_FLAG]:
             grad_bias = grad_output.sum(0)
         return grad_input, None, None, grad_bias
@@ -244,7 +244,7 @@ def _a8w8_backward_common(ctx, grad_output, input_f, weight_f, bias, detach_dw):
     grad_input = grad_bias = None
     if ctx.needs_input_grad[0]:
         grad_input = grad_output.mm(weight_f)
-    dw = grad_output.t().mm(input_f)
+    dw = ops.weight_grad(grad_output, input_f)
     dict_temp.append(dw.data if detach_dw else dw)
     if bias is not None and ctx.needs_input_grad[_BIAS_FLAG]:
         grad_bias = grad_output.sum(0)

@@ -54,6 +54,8 @@ def test_bad_arguments_are_rejected_without_a_gpu(hip_lib):
     assert lib.lq_latent_w4_reconstruct(p, p, p, res, p, 8, 128, 128, 2, 0.3, 2, 0.25, 4, None) == -1
     assert b"b1 < b2" in lib.lq_last_error()
     assert lib.lq_calib_copy(p, p, 10, None) == -1
+    assert lib.lq_transpose_bf16(p, p, 12, 64, None) == -1
+    assert b"multiples of 8" in lib.lq_last_error()
     assert lib.lq_adam8_update(p, p, p, p, p, p, p, p, p, 2048, 2048, 0.9, 0.95, 1e-8, 1e-3, None) == -1
     assert b"exactly one of param and direction" in lib.lq_last_error()
     assert lib.lq_adam8_update(p, p, None, p, p, p, p, p, p, 2048, 512, 0.9, 0.95, 1e-8, 1e-3, None) == -1

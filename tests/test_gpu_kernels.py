@@ -322,3 +322,20 @@ def test_error_reporting(ops):
         ops.a16w4_forward(x, packed, scales, zeros, (N, K))
     with pytest.raises(ValueError):
         ops.a16w4_forward(dev(x)[:, :64].contiguous(), dev(packed), dev(scales), dev(zeros), (N, K))
+
+
+# ------------------------------------------------------------- transpose / dW --
+@pytest.mark.parametrize("R,C", [(8, 8), (64, 64), (72, 136), (2048, 4096), (1000, 11008)])
+def test_transpose_bf16(ops, R, C):
+    x = randn_bf16((R, C), R + C)
+    got = ops.transpose_bf16(dev(x))
+    assert got.shape == (C, R) and got.is_contiguous()
+    assert torch.equal(got.cpu(), x.t().contiguous())
+
+
+def test_weight_grad_matches_the_strided_gemm(ops):
+    dy, x = randn_bf16((512, 384), 1), randn_bf16((512, 256), 2)
+    got = ops.weight_grad(dev(dy), dev(x))
+    want = dy.float().t().mm(x.float())
+    assert got.shape == (384, 256)
+    assert util.rel_l2(got.float().cpu(), want) < 5e-3
