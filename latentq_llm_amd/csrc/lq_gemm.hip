@@ -578,6 +578,32 @@ extern "C" int lq_a16w4_fwd(const void *x, const void *codes, const void *scales
     LQ_REQUIRE(N % 16 == 0, "lq_a16w4_fwd: N=%lld must be a multiple of 16", (long long)N);
     if (M <= 16)
         return lq_gemv_a16w4_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
+    if (M <= 128) {
+        // A few more tokens than one GEMV takes: the GEMM's 128-row tiles would be mostly padding and
+        // its grid (N/128 workgroups, each walking all of K) fills a fraction of the device, so
+        // chunks of 16 tokens through the GEMV can be faster: the first streams the weights from
+        // HBM at near memory speed, the others find them in the last-level cache. Rough costs in
+        // microseconds: the GEMM takes ~0.6 per 64-k step and round of workgroups; a GEMV chunk its
+        // bytes at ~1.8 TB/s the first time (at least 6) and ~2.3 TB/s after (at least 8; measured).
+        const int chunks = (int)((M + 15) / 16);
+        const double bytes = (double)(N * K / 2 + N * (K / LQ_GROUP) * 4);
+        const double first_us = bytes / 1.8e6 > 6.0 ? bytes / 1.8e6 : 6.0;
+        const double next_us = bytes / 2.3e6 > 8.0 ? bytes / 2.3e6 : 8.0;
+        const double est_gemv = first_us + (chunks - 1) * next_us;
+        const long long tiles = ((M + 127) / 128) * ((N + 127) / 128);
+        const long long slots = 2ll * lq_device_cu_count();
+        const double est_gemm = 0.6 * (double)(K / 64) * (double)((tiles + slots - 1) / slots);
+        if (est_gemv < est_gemm) {
+            for (int c = 0; c < chunks; ++c) {
+                const int rows = (int)(M - 16 * c < 16 ? M - 16 * c : 16);
+                rc = lq_gemv_a16w4_launch((const unsigned short *)x + (long long)c * 16 * K, codes, scales, zeros,
+                                          bias_or_null, (unsigned short *)y + (long long)c * 16 * N, rows, (int)N, (int)K,
+                                          (hipStream_t)stream);
+                if (rc) return rc;
+            }
+            return LQ_OK;
+        }
+    }
     // Two forward kernels. The weights-direct one (128 x 256 tiles, two workgroups per CU) wins when
     // its tiles can occupy every CU twice; otherwise the staged 256 x 128 kernel, whose producer
     // waves hide more latency with a single workgroup per CU, is faster.

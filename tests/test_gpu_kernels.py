@@ -176,6 +176,12 @@ def test_a16w4_fwd_gemm(ops, co, M, N, K, bias):
     _fwd_case(ops, co, M, N, K, seed=M + N + K, with_bias=bias)
 
 
+@pytest.mark.parametrize("M,N,K,bias", [(17, 4096, 4096, True), (32, 11008, 4096, False), (37, 1024, 11008, True)])
+def test_a16w4_fwd_a_few_more_tokens_than_one_gemv(ops, co, M, N, K, bias):
+    """17..64 tokens on matrices large enough that chunks of 16 through the GEMV beat the GEMM."""
+    _fwd_case(ops, co, M, N, K, seed=M + N + K, with_bias=bias)
+
+
 @pytest.mark.parametrize("M", [1, 2, 4, 5, 16])
 @pytest.mark.parametrize("N,K,bias", [(16, 128, False), (64, 640, True), (4096, 4096, False), (256, 11008, True)])
 def test_a16w4_fwd_gemv(ops, co, M, N, K, bias):
