@@ -94,6 +94,20 @@ int lq_a16w4_fwd(const void *x, const void *codes, const void *scales, const voi
 int lq_a16w4_dx(const void *dy, const void *codes, const void *scales, const void *zeros,
                 void *dx, int64_t M, int64_t N, int64_t K, int group, void *stream);
 
+/* The same two products with a scratch buffer the library may use (it allocates nothing itself):
+ * when the output has so few 128 x 128 tiles that they would occupy less than half of the device,
+ * the reduction is cut into up to 8 slices, each workgroup writes an fp32 partial tile into the
+ * workspace and a second kernel adds the slices in a fixed order (results are deterministic), adds
+ * the bias and rounds to bf16. workspace: 16-byte aligned device memory of workspace_bytes bytes,
+ * or null; M*out_columns*4 bytes per slice are used, fewer slices if the buffer is smaller. Calls
+ * that share a workspace must be ordered on one stream. No counterpart in the reference (its
+ * dense mm leaves this to the vendor library). */
+int lq_a16w4_fwd_ws(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias_or_null,
+                    void *y, int64_t M, int64_t N, int64_t K, int group, void *workspace, int64_t workspace_bytes,
+                    void *stream);
+int lq_a16w4_dx_ws(const void *dy, const void *codes, const void *scales, const void *zeros, void *dx, int64_t M,
+                   int64_t N, int64_t K, int group, void *workspace, int64_t workspace_bytes, void *stream);
+
 /* Dequantise the whole matrix to bf16[N,K] with the reference arithmetic
  * (DeQfunc_4bit_g, utils/quant.py:66-72). Used for the dW-side consumers and
  * for checks; not on the forward/backward GEMM path. */

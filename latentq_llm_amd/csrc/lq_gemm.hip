@@ -61,6 +61,10 @@ struct GemmParams {
     int R;                       // reduction length (K for fwd/i8, N for dx)
     int Kw;                      // K of the weight matrix (row length of W in elements)
     int tiles_m, tiles_n;
+    // split reduction: workgroup (tile, blockIdx.y) covers steps_per_split reduction steps from
+    // blockIdx.y * steps_per_split and writes its fp32 partial tile to partial[blockIdx.y][M][C]
+    int steps_per_split;
+    float *partial;
 };
 
 typedef __attribute__((address_space(3))) void lds_void;
@@ -138,7 +142,9 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
     const int bw = rest < GN ? rest : GN;
     const int tile_m = within / bw, tile_n = band * GN + within % bw;
     const int m0 = tile_m * BM, c0 = tile_n * BN;
-    const int nk = p.R / RT;
+    // reduction steps of this workgroup: all of them, or one slice of a split reduction
+    const int k0 = p.partial ? (int)blockIdx.y * p.steps_per_split : 0;
+    const int nk = p.partial ? (p.R / RT - k0 < p.steps_per_split ? p.R / RT - k0 : p.steps_per_split) : p.R / RT;
     const int groups_per_row = p.Kw / LQ_GROUP;
 
     if (is_weight_wave) {
@@ -168,7 +174,7 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
                 const int row = c >> 3, ch = c & 7;
                 int gr = c0 + row;
                 gr = gr < p.C ? gr : p.C - 1;
-                b_src[i] = (const unsigned char *)p.b + (long long)gr * p.Kw + ch * 16;
+                b_src[i] = (const unsigned char *)p.b + (long long)gr * p.Kw + ch * 16 + (long long)k0 * ROWB;
                 b_dst[i] = row * ROWB + ((ch ^ swz(row)) << 4);
             }
         } else if constexpr (MODE == MODE_W4_FWD) {
@@ -177,16 +183,16 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             b_w0 = (tid % TPR) * NW;
             int gr = c0 + b_row;
             gr = gr < p.C ? gr : p.C - 1;
-            b_src[0] = (const unsigned char *)p.b + (long long)gr * (p.Kw / 2) + b_w0 * 4;
-            s_src[0] = p.scales + (long long)gr * groups_per_row;
-            z_src[0] = p.zeros + (long long)gr * groups_per_row;
+            b_src[0] = (const unsigned char *)p.b + (long long)gr * (p.Kw / 2) + b_w0 * 4 + (long long)k0 * 32;
+            s_src[0] = p.scales + (long long)gr * groups_per_row + k0 / 2;  // k0 is even: a group is two steps
+            z_src[0] = p.zeros + (long long)gr * groups_per_row + k0 / 2;
         } else {
             b_row = tid >> 2;  // n within the tile (the tile offset along n is added per tile)
             b_w0 = tid & 3;    // 32 of the tile's 128 output columns k
-            b_src[0] = (const unsigned char *)p.b + (long long)b_row * (p.Kw / 2) + c0 / 2 + b_w0 * 16;
+            b_src[0] = (const unsigned char *)p.b + ((long long)k0 * 64 + b_row) * (p.Kw / 2) + c0 / 2 + b_w0 * 16;
             const int g = (c0 + b_w0 * 32) / LQ_GROUP;
-            s_src[0] = p.scales + (long long)b_row * groups_per_row + g;
-            z_src[0] = p.zeros + (long long)b_row * groups_per_row + g;
+            s_src[0] = p.scales + ((long long)k0 * 64 + b_row) * groups_per_row + g;
+            z_src[0] = p.zeros + ((long long)k0 * 64 + b_row) * groups_per_row + g;
         }
 
         struct Stage {
@@ -295,7 +301,7 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
         gr = gr < p.M ? gr : p.M - 1;
         a_off[i] = (unsigned)((gr - m0) * lda + ch * 16);
     }
-    const unsigned char *a_base = (const unsigned char *)p.a + m0 * lda;
+    const unsigned char *a_base = (const unsigned char *)p.a + m0 * lda + (long long)k0 * ROWB;
     // LDS-direct load: lane l of the wave writes 16 bytes at (wave-uniform base) + 16*l. Written as
     // inline assembly (M0 = LDS base, one wait state, then the load with a scalar base and a 32-bit
     // lane offset) so that the compiler's wait-count insertion does not see an LDS write it cannot
@@ -451,6 +457,27 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
     // contiguous bytes of a row. The B buffers are free here (the weight waves wrote their last
     // tile before the final barrier, and no load is in flight into them); a wave's staging area
     // is private, row pitch TN*2 + 16 bytes.
+    if (p.partial) {
+        // split reduction: the fp32 accumulators as they are, 16 bytes per lane; a second kernel adds
+        // the slices in a fixed order, adds the bias and rounds
+        float *part = p.partial + (long long)blockIdx.y * p.M * p.C;
+#pragma unroll
+        for (int j = 0; j < FM; ++j) {
+            const int m = m0 + wm * TM + j * 32 + frag_row;
+            if (m >= p.M) continue;
+#pragma unroll
+            for (int i = 0; i < FN; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int c = c0 + wn * TN + i * 32 + 8 * q + 4 * kh;
+                    if (c >= p.C) continue;
+                    f32x4_t v = {(float)acc[i][j][4 * q], (float)acc[i][j][4 * q + 1], (float)acc[i][j][4 * q + 2],
+                                 (float)acc[i][j][4 * q + 3]};
+                    *reinterpret_cast<f32x4_t *>(part + (long long)m * p.C + c) = v;
+                }
+        }
+        return;
+    }
     unsigned short *out = (unsigned short *)p.c;
     constexpr int EP = TN * 2 + 16;
     constexpr int EP_WAVE = 32 * EP;
@@ -519,8 +546,32 @@ int launch_gemm(GemmParams p, hipStream_t st, const char *who) {
     auto kern = gemm_kernel<MODE, BM, BN, WM, WN>;
     const long long nwg = (long long)p.tiles_m * p.tiles_n;
     if (nwg > 0x7FFFFFFFll) return lq_fail(LQ_ERR_BAD_ARG, "%s: problem too large", who);
-    hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(128 * WM * WN), 0, st, p);
+    const int total_steps = p.R / ((MODE == MODE_I8) ? 128 : 64);
+    const unsigned splits = p.partial ? (unsigned)((total_steps + p.steps_per_split - 1) / p.steps_per_split) : 1u;
+    hipLaunchKernelGGL(kern, dim3((unsigned)nwg, splits), dim3(128 * WM * WN), 0, st, p);
     return lq_check_launch(who);
+}
+
+// out[m][c] = bf16(sum over the slices, in order, of partial[s][m][c] (+ bias[c])); 8 columns per thread
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ partial,
+                                                           const unsigned short *__restrict__ bias,
+                                                           unsigned short *__restrict__ out, long long MC, int C, int splits) {
+    const long long e = ((long long)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (e >= MC) return;
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < splits; ++s) {
+        const f32x4_t a = *reinterpret_cast<const f32x4_t *>(partial + (long long)s * MC + e);
+        const f32x4_t b = *reinterpret_cast<const f32x4_t *>(partial + (long long)s * MC + e + 4);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { v[k] += a[k]; v[4 + k] += b[k]; }
+    }
+    if (bias) {
+        const int c = (int)(e % C);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] += lq_bf16_bits_to_f32(bias[c + k]);
+    }
+    *reinterpret_cast<u32x4_t *>(out + e) = u32x4_t{lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3]),
+                                                    lq_pack_bf16(v[4], v[5]), lq_pack_bf16(v[6], v[7])};
 }
 
 }  // namespace
@@ -538,11 +589,15 @@ static int lq_device_cu_count() {
     return cached[dev];
 }
 
-// 128 x 128 tiles when 256 x 128 tiles would leave compute units without a workgroup
+// 128 x 128 or 256 x 128 tiles. Measured: a workgroup alone on a compute unit takes ~0.54 us per
+// 64-deep step with the small tile and ~0.75 with the large one, and a second small-tile workgroup
+// on the same unit adds its full time, so a grid costs about (rounds of one workgroup per unit) x
+// pace: small tiles while they fit in one round, large ones otherwise.
 static bool small_tiles(const GemmParams &p) {
-    if (p.M <= 128) return true;
-    const long long big = (long long)((p.M + 255) / 256) * ((p.C + 127) / 128);
-    return big < lq_device_cu_count();
+    const long long cus = lq_device_cu_count();
+    const long long cols = (p.C + 127) / 128;
+    const long long small = (long long)((p.M + 127) / 128) * cols, big = (long long)((p.M + 255) / 256) * cols;
+    return 0.54 * (double)((small + cus - 1) / cus) < 0.75 * (double)((big + cus - 1) / cus);
 }
 
 // weights-direct forward GEMM (lq_gemm_fwd.hip)
@@ -570,30 +625,74 @@ static int check_w4_common(const char *who, const void *a, const void *codes, co
     return LQ_OK;
 }
 
-extern "C" int lq_a16w4_fwd(const void *x, const void *codes, const void *scales, const void *zeros,
-                            const void *bias_or_null, void *y, int64_t M, int64_t N, int64_t K, int group,
-                            void *stream) {
-    int rc = check_w4_common("lq_a16w4_fwd", x, codes, scales, zeros, y, M, N, K, group);
+// Rough time of a grid of 128 x 128 tiles in microseconds (measured): a workgroup alone on a compute
+// unit takes ~0.56 per 64-deep step and two on one unit take twice that each, so what counts is the
+// number of rounds of one workgroup per unit; prologue and epilogue cost about three steps, the
+// launch ~4 us.
+static double gemm128_est_us(long long workgroups, int steps) {
+    const long long cus = lq_device_cu_count();
+    return 0.56 * (steps + 3) * (double)((workgroups + cus - 1) / cus) + 4.0;
+}
+
+// Split reduction for grids that fill less than half of the compute units: 128 x 128 tiles, the
+// reduction cut into up to 8 slices of an even number of steps (at least 8) so that every unit
+// gets at most one workgroup, fp32 partial tiles in the caller's workspace, then a reduce kernel.
+// Returns the number of slices (1 = do not split) and the estimated time in microseconds (the
+// partial tiles are written and read back through the last-level cache at ~5 TB/s; ~3 us for the
+// second launch).
+static int plan_split(long long M, long long C, int total_steps, size_t ws_bytes, int *steps_per_split, double *est_us) {
+    const long long tiles = ((M + 127) / 128) * ((C + 127) / 128);
+    const long long cus = lq_device_cu_count();
+    if (!ws_bytes || tiles * 2 > cus) return 1;
+    long long S = cus / tiles;
+    if (S > 8) S = 8;
+    const long long fit = (long long)(ws_bytes / ((size_t)M * C * 4));
+    if (S > fit) S = fit;
+    if (S < 2) return 1;
+    int per = (int)((total_steps + S - 1) / S);
+    per += per & 1;
+    if (per < 8) per = 8;
+    S = (total_steps + per - 1) / per;
+    if (S < 2) return 1;
+    *steps_per_split = per;
+    *est_us = gemm128_est_us(tiles * S, per) + 3.0 + 2.0 * S * M * C * 4 / 5.0e6;
+    return (int)S;
+}
+
+static int launch_split_reduce(const GemmParams &p, int splits, hipStream_t st, const char *who) {
+    const long long MC = (long long)p.M * p.C;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((MC / 8 + 255) / 256)), dim3(256), 0, st, p.partial, p.bias,
+                       (unsigned short *)p.c, MC, p.C, splits);
+    return lq_check_launch(who);
+}
+
+static int a16w4_fwd_impl(const char *who, const void *x, const void *codes, const void *scales, const void *zeros,
+                          const void *bias_or_null, void *y, int64_t M, int64_t N, int64_t K, int group, void *workspace,
+                          size_t ws_bytes, void *stream) {
+    int rc = check_w4_common(who, x, codes, scales, zeros, y, M, N, K, group);
     if (rc) return rc;
-    LQ_REQUIRE(N % 16 == 0, "lq_a16w4_fwd: N=%lld must be a multiple of 16", (long long)N);
+    LQ_REQUIRE(N % 16 == 0, "%s: N=%lld must be a multiple of 16", who, (long long)N);
+    LQ_REQUIRE(!workspace || lq_aligned(workspace, 16), "%s: the workspace must be 16-byte aligned", who);
     if (M <= 16)
         return lq_gemv_a16w4_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
+    int per = 0;
+    double est_split = 0.0;
+    const int splits = plan_split(M, N, (int)(K / 64), workspace ? ws_bytes : 0, &per, &est_split);
+    const long long tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    const double est_gemm = gemm128_est_us(tiles, (int)(K / 64));
     if (M <= 128) {
         // A few more tokens than one GEMV takes: the GEMM's 128-row tiles would be mostly padding and
         // its grid (N/128 workgroups, each walking all of K) fills a fraction of the device, so
         // chunks of 16 tokens through the GEMV can be faster: the first streams the weights from
         // HBM at near memory speed, the others find them in the last-level cache. Rough costs in
-        // microseconds: the GEMM takes ~0.6 per 64-k step and round of workgroups; a GEMV chunk its
-        // bytes at ~1.8 TB/s the first time (at least 6) and ~2.3 TB/s after (at least 8; measured).
+        // microseconds: the GEMM as gemm128_est_us has it; a GEMV chunk its bytes at ~1.8 TB/s the
+        // first time (at least 6) and ~2.3 TB/s after (at least 5; measured).
         const int chunks = (int)((M + 15) / 16);
         const double bytes = (double)(N * K / 2 + N * (K / LQ_GROUP) * 4);
         const double first_us = bytes / 1.8e6 > 6.0 ? bytes / 1.8e6 : 6.0;
-        const double next_us = bytes / 2.3e6 > 8.0 ? bytes / 2.3e6 : 8.0;
+        const double next_us = bytes / 2.3e6 > 5.0 ? bytes / 2.3e6 : 5.0;
         const double est_gemv = first_us + (chunks - 1) * next_us;
-        const long long tiles = ((M + 127) / 128) * ((N + 127) / 128);
-        const long long slots = 2ll * lq_device_cu_count();
-        const double est_gemm = 0.6 * (double)(K / 64) * (double)((tiles + slots - 1) / slots);
-        if (est_gemv < est_gemm) {
+        if (est_gemv < est_gemm && (splits < 2 || est_gemv < est_split)) {
             for (int c = 0; c < chunks; ++c) {
                 const int rows = (int)(M - 16 * c < 16 ? M - 16 * c : 16);
                 rc = lq_gemv_a16w4_launch((const unsigned short *)x + (long long)c * 16 * K, codes, scales, zeros,
@@ -604,31 +703,75 @@ extern "C" int lq_a16w4_fwd(const void *x, const void *codes, const void *scales
             return LQ_OK;
         }
     }
-    // Two forward kernels. The weights-direct one (128 x 256 tiles, two workgroups per CU) wins when
-    // its tiles can occupy every CU twice; otherwise the staged 256 x 128 kernel, whose producer
-    // waves hide more latency with a single workgroup per CU, is faster.
-    // the weights-direct kernel loads scales and zeros four groups at a time: rows must be 4-byte aligned
-    if (lq_gemm_fwd_direct_workgroups((int)M, (int)N) >= 1ll * lq_device_cu_count() && (K / LQ_GROUP) % 2 == 0)
-        return lq_gemm_fwd_direct_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
     GemmParams p = {};
     p.a = x; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.bias = (const unsigned short *)bias_or_null; p.c = y;
     p.M = (int)M; p.C = (int)N; p.R = (int)K; p.Kw = (int)K;
-    if (small_tiles(p)) return launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, "lq_a16w4_fwd");
-    return launch_gemm<MODE_W4_FWD, 256, 128, 2, 2>(p, (hipStream_t)stream, "lq_a16w4_fwd");
+    if (splits >= 2 && est_split < est_gemm) {
+        p.partial = (float *)workspace;
+        p.steps_per_split = per;
+        rc = launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
+        return rc ? rc : launch_split_reduce(p, splits, (hipStream_t)stream, who);
+    }
+    // Two forward kernels. The weights-direct one (128 x 256 tiles, two workgroups per CU) wins when
+    // its tiles give every CU a workgroup; otherwise the staged kernel. The weights-direct kernel
+    // loads scales and zeros four groups at a time: rows must be 4-byte aligned.
+    if (lq_gemm_fwd_direct_workgroups((int)M, (int)N) >= 1ll * lq_device_cu_count() && (K / LQ_GROUP) % 2 == 0)
+        return lq_gemm_fwd_direct_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
+    if (small_tiles(p)) return launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
+    return launch_gemm<MODE_W4_FWD, 256, 128, 2, 2>(p, (hipStream_t)stream, who);
 }
 
-extern "C" int lq_a16w4_dx(const void *dy, const void *codes, const void *scales, const void *zeros, void *dx,
-                           int64_t M, int64_t N, int64_t K, int group, void *stream) {
-    int rc = check_w4_common("lq_a16w4_dx", dy, codes, scales, zeros, dx, M, N, K, group);
+extern "C" int lq_a16w4_fwd(const void *x, const void *codes, const void *scales, const void *zeros,
+                            const void *bias_or_null, void *y, int64_t M, int64_t N, int64_t K, int group,
+                            void *stream) {
+    return a16w4_fwd_impl("lq_a16w4_fwd", x, codes, scales, zeros, bias_or_null, y, M, N, K, group, nullptr, 0, stream);
+}
+
+extern "C" int lq_a16w4_fwd_ws(const void *x, const void *codes, const void *scales, const void *zeros,
+                               const void *bias_or_null, void *y, int64_t M, int64_t N, int64_t K, int group,
+                               void *workspace, int64_t workspace_bytes, void *stream) {
+    return a16w4_fwd_impl("lq_a16w4_fwd_ws", x, codes, scales, zeros, bias_or_null, y, M, N, K, group, workspace,
+                          workspace && workspace_bytes > 0 ? (size_t)workspace_bytes : 0, stream);
+}
+
+static int a16w4_dx_impl(const char *who, const void *dy, const void *codes, const void *scales, const void *zeros,
+                         void *dx, int64_t M, int64_t N, int64_t K, int group, void *workspace, size_t ws_bytes,
+                         void *stream) {
+    int rc = check_w4_common(who, dy, codes, scales, zeros, dx, M, N, K, group);
     if (rc) return rc;
-    LQ_REQUIRE(N % 64 == 0, "lq_a16w4_dx: N=%lld must be a multiple of 64", (long long)N);
+    LQ_REQUIRE(N % 64 == 0, "%s: N=%lld must be a multiple of 64", who, (long long)N);
+    LQ_REQUIRE(!workspace || lq_aligned(workspace, 16), "%s: the workspace must be 16-byte aligned", who);
     GemmParams p = {};
     p.a = dy; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.c = dx;
     p.M = (int)M; p.C = (int)K; p.R = (int)N; p.Kw = (int)K;
-    if (small_tiles(p)) return launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, "lq_a16w4_dx");
-    return launch_gemm<MODE_W4_DX, 256, 128, 2, 2>(p, (hipStream_t)stream, "lq_a16w4_dx");
+    int per = 0;
+    double est_split = 0.0;
+    const int splits = plan_split(M, K, (int)(N / 64), workspace ? ws_bytes : 0, &per, &est_split);
+    if (splits >= 2) {
+        const long long tiles = ((M + 127) / 128) * ((K + 127) / 128);
+        if (est_split < gemm128_est_us(tiles, (int)(N / 64))) {
+            p.partial = (float *)workspace;
+            p.steps_per_split = per;
+            rc = launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
+            return rc ? rc : launch_split_reduce(p, splits, (hipStream_t)stream, who);
+        }
+    }
+    if (small_tiles(p)) return launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
+    return launch_gemm<MODE_W4_DX, 256, 128, 2, 2>(p, (hipStream_t)stream, who);
+}
+
+extern "C" int lq_a16w4_dx(const void *dy, const void *codes, const void *scales, const void *zeros, void *dx,
+                           int64_t M, int64_t N, int64_t K, int group, void *stream) {
+    return a16w4_dx_impl("lq_a16w4_dx", dy, codes, scales, zeros, dx, M, N, K, group, nullptr, 0, stream);
+}
+
+extern "C" int lq_a16w4_dx_ws(const void *dy, const void *codes, const void *scales, const void *zeros, void *dx,
+                              int64_t M, int64_t N, int64_t K, int group, void *workspace, int64_t workspace_bytes,
+                              void *stream) {
+    return a16w4_dx_impl("lq_a16w4_dx_ws", dy, codes, scales, zeros, dx, M, N, K, group, workspace,
+                         workspace && workspace_bytes > 0 ? (size_t)workspace_bytes : 0, stream);
 }
 
 extern "C" int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const float *sw, const void *bias_or_null,

@@ -69,6 +69,26 @@ def philox_uniform(n: int, seed: int, offset: int = 0, device="cuda"):
     return out
 
 
+# Scratch for the split-reduction GEMM of skinny problems (fp32 partial tiles): one buffer per device
+# and stream, allocated on first need and kept; the library itself never allocates.
+_WORKSPACE = {}
+WORKSPACE_MAX_BYTES = 64 << 20
+
+
+def _workspace(t, rows, cols):
+    """(pointer, bytes) of a scratch buffer for a rows x cols fp32 result cut into up to 8 slices, or
+    (None, 0) when the problem is not one the split reduction is meant for (more than 1024 rows)."""
+    if rows > 1024:
+        return None, 0
+    need = min(8 * rows * cols * 4, WORKSPACE_MAX_BYTES)
+    key = (t.device.index, _stream(t))
+    buf = _WORKSPACE.get(key)
+    if buf is None or buf.numel() < need:
+        buf = torch.empty(need, dtype=torch.uint8, device=t.device)
+        _WORKSPACE[key] = buf
+    return buf.data_ptr(), buf.numel()
+
+
 def a16w4_forward(x, codes, scales, zeros, shape, bias=None, out=None):
     """Y[M,N] = X[M,K] . deq(W)[N,K]^T (+ bias) in bf16 with fp32 accumulation."""
     N, K = shape
@@ -92,8 +112,9 @@ def a16w4_forward(x, codes, scales, zeros, shape, bias=None, out=None):
     if M == 0:
         return y
     with torch.cuda.device(x.device):
-        _C.call("lq_a16w4_fwd", x.data_ptr(), codes.data_ptr(), scales.data_ptr(), zeros.data_ptr(),
-                None if bias is None else bias.data_ptr(), y.data_ptr(), M, N, K, GROUP, _stream(x))
+        ws, ws_bytes = _workspace(x, M, N) if M > 16 else (None, 0)
+        _C.call("lq_a16w4_fwd_ws", x.data_ptr(), codes.data_ptr(), scales.data_ptr(), zeros.data_ptr(),
+                None if bias is None else bias.data_ptr(), y.data_ptr(), M, N, K, GROUP, ws, ws_bytes, _stream(x))
     return y
 
 
@@ -116,8 +137,9 @@ def a16w4_dx(dy, codes, scales, zeros, shape, out=None):
     if M == 0:
         return dx
     with torch.cuda.device(dy.device):
-        _C.call("lq_a16w4_dx", dy.data_ptr(), codes.data_ptr(), scales.data_ptr(), zeros.data_ptr(), dx.data_ptr(),
-                M, N, K, GROUP, _stream(dy))
+        ws, ws_bytes = _workspace(dy, M, K)
+        _C.call("lq_a16w4_dx_ws", dy.data_ptr(), codes.data_ptr(), scales.data_ptr(), zeros.data_ptr(), dx.data_ptr(),
+                M, N, K, GROUP, ws, ws_bytes, _stream(dy))
     return dx
 
 

@@ -48,6 +48,12 @@ def test_bad_arguments_are_rejected_without_a_gpu(hip_lib):
     misaligned = C.c_void_p(p.value + 2)
     assert lib.lq_a16w4_fwd(misaligned, p, p, p, None, p, 32, 16, 128, 128, None) == -1
     assert b"aligned" in lib.lq_last_error()
+    assert lib.lq_a16w4_fwd_ws(p, p, p, p, None, p, 32, 16, 128, 128, misaligned, 4096, None) == -1
+    assert b"workspace" in lib.lq_last_error()
+    assert lib.lq_a16w4_dx_ws(p, p, p, p, p, 32, 64, 128, 128, misaligned, 4096, None) == -1
+    assert b"workspace" in lib.lq_last_error()
+    assert lib.lq_a16w4_dx_ws(p, p, p, p, p, 4, 48, 128, 128, None, 0, None) == -1
+    assert b"multiple of 64" in lib.lq_last_error()
     res = C.cast((C.c_char * 4096)(), C.c_void_p)
     assert lib.lq_latent_w4_requant(p, p, p, p, res, 8, 100, 128, 2, 0.125, 2, 0.25, 4, None) == -1
     assert b"multiple of 128" in lib.lq_last_error()

@@ -345,3 +345,49 @@ def test_weight_grad_matches_the_strided_gemm(ops):
     want = dy.float().t().mm(x.float())
     assert got.shape == (384, 256)
     assert util.rel_l2(got.float().cpu(), want) < 5e-3
+
+
+# ------------------------------------------------------- split reduction (skinny grids) --
+@pytest.mark.parametrize("M,N,K,bias", [(512, 1024, 4096, True), (200, 2048, 1280, False), (130, 4096, 11008, True)])
+def test_a16w4_fwd_split_reduction(ops, co, M, N, K, bias):
+    """Grids of a few dozen tiles with a long reduction: the forward product runs as slices of K with
+    fp32 partial tiles in the scratch buffer (slice lengths 16+16+16+16, 8+8+4 and 44+44+44+40 steps)."""
+    _fwd_case(ops, co, M, N, K, seed=M + N + K, with_bias=bias)
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 4096, 1024), (200, 1280, 2048), (64, 11008, 4096)])
+def test_a16w4_dx_split_reduction(ops, co, M, N, K):
+    codes, packed, scales, zeros = make_w4(N, K, M + N)
+    dy = randn_bf16((M, N), 7)
+    _, want64 = co.a16w4_dx(bits(dy), packed.numpy(), bits(scales), bits(zeros), M, N, K, want_f64=True)
+    got = ops.a16w4_dx(dev(dy), dev(packed), dev(scales), dev(zeros), (N, K)).float().cpu()
+    assert rel_l2(got, torch.from_numpy(want64)) <= REL_L2_TOL
+
+
+def test_split_reduction_identity_is_exact_and_deterministic(ops, co):
+    """X = identity through the split path: every output is one dequantised weight plus exact zeros
+    from the other slices, so the result equals the reference dequantisation bit for bit; and two
+    runs give the same bits (the slices are added in a fixed order)."""
+    N, K = 256, 1024
+    codes, packed, scales, zeros = make_w4(N, K, 23)
+    x = dev(torch.eye(K, dtype=torch.bfloat16))
+    got = ops.a16w4_forward(x, dev(packed), dev(scales), dev(zeros), (N, K))
+    want = co.dequant(packed.numpy(), bits(scales), bits(zeros), N, K)
+    assert np.array_equal(bits(got).T, want)
+    xr = dev(randn_bf16((K, K), 3))
+    a = ops.a16w4_forward(xr, dev(packed), dev(scales), dev(zeros), (N, K))
+    b = ops.a16w4_forward(xr, dev(packed), dev(scales), dev(zeros), (N, K))
+    assert torch.equal(a, b)
+
+
+def test_workspace_entry_points_without_a_workspace_match_the_plain_ones(ops):
+    """lq_a16w4_fwd (no scratch) and lq_a16w4_fwd_ws agree within the bf16 output rounding."""
+    from latentq_llm_amd import _C
+    M, N, K = 256, 1024, 2048
+    codes, packed, scales, zeros = make_w4(N, K, 41)
+    x, p, s, z = dev(randn_bf16((M, K), 42)), dev(packed), dev(scales), dev(zeros)
+    y0 = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+    st = torch.cuda.current_stream().cuda_stream
+    _C.call("lq_a16w4_fwd", x.data_ptr(), p.data_ptr(), s.data_ptr(), z.data_ptr(), None, y0.data_ptr(), M, N, K, 128, st)
+    y1 = ops.a16w4_forward(x, p, s, z, (N, K))
+    assert rel_l2(y1.float().cpu(), y0.float().cpu()) < 4e-3
