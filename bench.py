@@ -41,11 +41,18 @@ def synth_w4(N, K, seed, device):
     return codes.to(device), scales.to(device), zeros.to(device)
 
 
-def event_time(fn, iters, warm=30):
-    """Average seconds per call of fn(), HIP events on the current (= launch) stream."""
-    for _ in range(warm):
-        fn()
-    torch.cuda.synchronize()
+def event_time(fn, iters, warm=30, warm_seconds=0.08):
+    """Average seconds per call of fn(), HIP events on the current (= launch) stream. The warm-up
+    runs at least `warm` calls and at least `warm_seconds` of work: after an idle period the
+    device takes tens of milliseconds to settle at its sustained clock (a GEMM timed over the
+    first 5 ms reads ~10 % low)."""
+    t0 = time.perf_counter()
+    done = 0
+    while done < warm or time.perf_counter() - t0 < warm_seconds:
+        for _ in range(10):
+            fn()
+        done += 10
+        torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(iters):
@@ -389,8 +396,8 @@ def _cpu_model():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-mlp", action="store_true", help="skip the side measurements (requant, GEMV, A8W8)")
     ap.add_argument("--profile-target", choices=["gemm", "requant", "gemv", "a8w8", "latent", "adam8"],

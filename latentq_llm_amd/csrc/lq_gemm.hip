@@ -602,10 +602,13 @@ static bool small_tiles(const GemmParams &p) {
 
 // weights-direct forward GEMM (lq_gemm_fwd.hip)
 long long lq_gemm_fwd_direct_workgroups(int M, int N);
-int lq_gemm_i8_direct_launch(const void *x8, const void *w8, const float *sx, const float *sw, const void *bias, void *y,
-                             int *acc_or_null, int M, int N, int K, hipStream_t st);
 int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
                               void *y, int M, int N, int K, hipStream_t st);
+
+// int8 GEMM with 256 x 256 tiles (lq_gemm_i8.hip)
+long long lq_gemm_i8_256_workgroups(int M, int N);
+int lq_gemm_i8_256_launch(const void *x8, const void *w8, const float *sx, const float *sw, const void *bias, void *y,
+                          int *acc_or_null, int M, int N, int K, hipStream_t st);
 
 // GEMV path (lq_gemv.hip)
 int lq_gemv_a16w4_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
@@ -784,8 +787,10 @@ extern "C" int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const 
     LQ_REQUIRE(lq_aligned(x, 16) && lq_aligned(w, 16) && lq_aligned(y, 16) && lq_aligned(sx, 4) && lq_aligned(sw, 4) &&
                    (!acc_or_null || lq_aligned(acc_or_null, 16)),
                "lq_a8w8_fwd: x, w, y, acc must be 16-byte aligned");
-    if (lq_gemm_fwd_direct_workgroups((int)M, (int)N) >= 2ll * lq_device_cu_count())
-        return lq_gemm_i8_direct_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, (hipStream_t)stream);
+    // 256 x 256 tiles, both operands through LDS, when they occupy more than half of the compute
+    // units; below that the staged kernel's smaller tiles fill the device better
+    if (lq_gemm_i8_256_workgroups((int)M, (int)N) * 2 > (long long)lq_device_cu_count())
+        return lq_gemm_i8_256_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, (hipStream_t)stream);
     GemmParams p = {};
     p.a = x; p.b = w; p.sx = sx; p.sw = sw; p.bias = (const unsigned short *)bias_or_null; p.c = y;
     p.acc_out = acc_or_null;

@@ -1,7 +1,5 @@
-// Weights-direct forward GEMMs for gfx950:
+// Weights-direct forward GEMM for gfx950:
 //   A16W4, M > 16:  Y[M,N] = X[M,K] . deq(W)[N,K]^T (+ bias), bf16 MFMA
-//   A8W8 (template flag I8): the same structure on int8 operands, int32 accumulators and the fused
-//   scale epilogue; a lane then loads 64 bytes of its weight row per step and no dequantisation is needed.
 //
 // The weights never pass through LDS. An MFMA B-side lane needs 8 consecutive k of one weight
 // row, and 8 consecutive k of a row are exactly one 32-bit word of packed codes: every lane
@@ -51,13 +49,11 @@
 namespace {
 
 struct FwdParams {
-    const unsigned char *x;   // bf16 [M, K] (int8 variant: int8 [M, K])
-    const unsigned char *w;   // packed codes, K/2 bytes per row (int8 variant: int8 [N, K])
+    const unsigned char *x;   // bf16 [M, K]
+    const unsigned char *w;   // packed codes, K/2 bytes per row
     const unsigned short *scales;
     const unsigned short *zeros;
     const unsigned short *bias;  // bf16 [N] or null
-    const float *sx, *sw;        // int8 variant: per-row and per-column scales
-    int *acc_out;                // int8 variant: optional int32 [M, N]
     unsigned short *y;           // bf16 [M, N]
     int M, N, K;
     int tiles_m, tiles_n;
@@ -69,18 +65,16 @@ template <int I>
 using ic = std::integral_constant<int, I>;
 
 constexpr int BM = 128, BN = 256;
-constexpr int ROWB = 128;            // bytes of A per tile row and step: 64 bf16 or 128 int8
+constexpr int ROWB = 128;            // bytes of A per tile row and step: 64 bf16
 constexpr int STAGE = BM * ROWB;     // 16 KB per A stage
 
-template <bool I8>
 __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
-    constexpr int ESZ = I8 ? 1 : 2;          // bytes per A element
-    constexpr int WROW = I8 ? 128 : 32;      // bytes of one weight row consumed per step
-    // 16-byte weight loads per lane and column tile in one batch: int8, the 4 pieces of one step;
-    // int4, the pieces of two consecutive steps (steps 2j and 2j+1 are 64 contiguous bytes of a
-    // row across the two lane halves: fetched together they pull their cache line through L1 twice
-    // instead of four times)
-    constexpr int NB = I8 ? 4 : 2;
+    constexpr int ESZ = 2;    // bytes per A element
+    constexpr int WROW = 32;  // bytes of one weight row consumed per step
+    // 16-byte weight loads per lane and column tile in one batch: the pieces of two consecutive
+    // steps (steps 2j and 2j+1 are 64 contiguous bytes of a row across the two lane halves: fetched
+    // together they pull their cache line through L1 twice instead of four times)
+    constexpr int NB = 2;
     __shared__ __attribute__((aligned(16))) unsigned char lds_a0[STAGE];
     __shared__ __attribute__((aligned(16))) unsigned char lds_a1[STAGE];
     __shared__ __attribute__((aligned(16))) unsigned char lds_a2[STAGE];
@@ -149,7 +143,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         u32x4_t d = {(unsigned)a, (unsigned)(a >> 32) & 0xFFFFu, bytes, 0x00020000u};
         return d;
     };
-    const unsigned wpitch = I8 ? (unsigned)p.K : (unsigned)(p.K / 2);  // bytes per weight row
+    const unsigned wpitch = (unsigned)(p.K / 2);  // bytes per weight row
     const u32x4_t w_rsrc = make_rsrc(p.w + (long long)c0 * wpitch, (unsigned)rows_here * wpitch);
     const u32x4_t s_rsrc = make_rsrc(p.scales + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u);
     const u32x4_t z_rsrc = make_rsrc(p.zeros + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u);
@@ -161,8 +155,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         q_off[i] = n * (unsigned)groups_per_row * 2u;
     }
 
-    using acc_t = typename std::conditional<I8, i32x16_t, f32x16_t>::type;
-    acc_t acc[2][4];
+    f32x16_t acc[2][4];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -173,23 +166,15 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     // All global loads of the loop are inline assembly: the compiler then inserts no vmcnt waits of
     // its own (it could only wait for everything, LDS-direct loads included); the single
     // s_waitcnt of a step is tied to the loaded registers instead.
-    u32x4_t cw[2][NB], cn[2][NB];  // weights of the current and of the next batch (int4 codes or int8)
+    u32x4_t cw[2][NB], cn[2][NB];  // codes of the current and of the next batch
     // Raw bf16 scales / zeros of four consecutive groups of the lane's two rows (one 8-byte load per
     // row every 8 steps: a 2-byte load per group would pull a whole cache line through L1 each time).
     // The 8-byte loads need 4-byte aligned rows: the launcher requires an even number of groups per row.
     u32x2_t qs[2], qz[2];
     float s[2], nzs[2];
     auto load_codes_one = [&](int kt, u32x4_t (*c)[NB], int i) {
-        {
-            asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(c[i][0]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
-            if constexpr (!I8) {
-                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:32" : "=v"(c[i][1]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
-            } else {
-                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:16" : "=v"(c[i][1]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
-                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:32" : "=v"(c[i][2]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
-                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:48" : "=v"(c[i][3]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
-            }
-        }
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(c[i][0]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:32" : "=v"(c[i][1]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
     };
     auto load_codes = [&](int kt, u32x4_t (*c)[NB]) {
 #pragma unroll
@@ -220,26 +205,18 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) af[j] = *reinterpret_cast<const u32x4_t *>(la + j * 4096 + a_frag[t]);
     };
-    // par = which step of the batch (int4 only)
+    // par = which step of the batch
     auto deq_one = [&](const u32x4_t (*c)[NB], int par, int t, u32x4_t *bf, int i) {
-        if constexpr (I8) {
-            bf[i] = c[i][t];  // 16 int8 of the lane's row: already the MFMA operand
-        } else {
-            float f[8];
-            lq_dequant_word_f32(c[i][par][t], s[i], nzs[i], f);
-            bf[i] = u32x4_t{lq_pack_bf16(f[0], f[1]), lq_pack_bf16(f[2], f[3]), lq_pack_bf16(f[4], f[5]),
-                            lq_pack_bf16(f[6], f[7])};
-        }
+        float f[8];
+        lq_dequant_word_f32(c[i][par][t], s[i], nzs[i], f);
+        bf[i] = u32x4_t{lq_pack_bf16(f[0], f[1]), lq_pack_bf16(f[2], f[3]), lq_pack_bf16(f[4], f[5]),
+                        lq_pack_bf16(f[6], f[7])};
     };
     auto mfma_half = [&](const u32x4_t *af, const u32x4_t *bf, int i) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            if constexpr (I8)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf[i]),
-                                                                 __builtin_bit_cast(i32x4_t, af[j]), acc[i][j], 0, 0, 0);
-            else
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[i]),
-                                                                   __builtin_bit_cast(bf16x8_t, af[j]), acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[i]),
+                                                               __builtin_bit_cast(bf16x8_t, af[j]), acc[i][j], 0, 0, 0);
     };
 
     // The one synchronisation point of a step (and the end of the prologue): everything this wave
@@ -248,11 +225,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     auto wait_and_meet = [&](auto newest, auto with_qparams) {
         constexpr int NEWEST = decltype(newest)::value;
         (void)cn; (void)qs; (void)qz;  // named outside the constexpr branches so that the lambda captures them
-        if constexpr (I8) {
-            asm volatile("s_waitcnt vmcnt(%8) lgkmcnt(0)\n\ts_barrier"
-                         : "+v"(cn[0][0]), "+v"(cn[0][1]), "+v"(cn[0][2]), "+v"(cn[0][3]), "+v"(cn[1][0]), "+v"(cn[1][1]),
-                           "+v"(cn[1][2]), "+v"(cn[1][3]) : "n"(NEWEST) : "memory");
-        } else if constexpr (decltype(with_qparams)::value != 0) {
+        if constexpr (decltype(with_qparams)::value != 0) {
             asm volatile("s_waitcnt vmcnt(%8) lgkmcnt(0)\n\ts_barrier"
                          : "+v"(cn[0][0]), "+v"(cn[0][1]), "+v"(cn[1][0]), "+v"(cn[1][1]), "+v"(qs[0]), "+v"(qs[1]), "+v"(qz[0]),
                            "+v"(qz[1]) : "n"(NEWEST) : "memory");
@@ -283,8 +256,8 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         const unsigned char *la = abuf(ic<AI>());
         const unsigned char *la_after = abuf(ic<(AI + 1) % 3>());
         unsigned char *la_load = abuf(ic<(AI + 2) % 3>());
-        // int8: the next step's weights every step; int4: the next pair of steps on even steps
-        const int kt_codes = I8 ? (kt + 1 < nk ? kt + 1 : kt) : (kt + 2 < nk ? kt + 2 : kt);
+        // the codes of the next pair of steps are loaded on even steps
+        const int kt_codes = kt + 2 < nk ? kt + 2 : kt;
         const int kt_a = kt + 2 < nk ? kt + 2 : nk - 1;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -292,7 +265,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
             for (int i = 0; i < 2; ++i) {
                 if (t == 3 && i == 0) {
                     wait_and_meet(ic<2>(), ic<ODD ? 0 : 1>());
-                    if (!I8 && ODD) use_qparams((kt + 1) >> 1);
+                    if (ODD) use_qparams((kt + 1) >> 1);
                 }
                 const unsigned char *src = t < 3 ? la : la_after;
                 const int tn = (t + 1) & 3;
@@ -300,16 +273,16 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
                 // their LDS latency
                 if (i == 0) read_a(src, tn, af[tn & 1]);
                 if (t < 3) deq_one(cw, ODD ? 1 : 0, tn, bf[tn & 1], i);
-                else if (I8 || ODD) deq_one(cn, 0, 0, bf[0], i);
+                else if (ODD) deq_one(cn, 0, 0, bf[0], i);
                 else deq_one(cw, 1, 0, bf[0], i);
-                if (t == 0 && (I8 || !ODD)) load_codes_one(kt_codes, cn, i);
-                if (t == 1 && !I8 && !ODD) load_qparams_one((kt + 2) >> 1 < groups_per_row ? (kt + 2) >> 1 : groups_per_row - 1, i);
+                if (t == 0 && !ODD) load_codes_one(kt_codes, cn, i);
+                if (t == 1 && !ODD) load_qparams_one((kt + 2) >> 1 < groups_per_row ? (kt + 2) >> 1 : groups_per_row - 1, i);
                 if (t >= 2) issue_a_one(kt_a, la_load, 2 * (t - 2) + i);
                 mfma_half(af[t & 1], bf[t & 1], i);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        if (I8 || ODD) {
+        if (ODD) {
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -317,7 +290,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         }
     };
 
-    if (!I8) load_qparams(0);
+    load_qparams(0);
     load_codes(0, cn);
     issue_a(0, lds_a0);
     issue_a(nk > 1 ? 1 : 0, lds_a1);
@@ -326,7 +299,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int b = 0; b < NB; ++b) cw[i][b] = cn[i][b];
-    if (!I8) use_qparams(0);
+    use_qparams(0);
     read_a(lds_a0, 0, af[0]);
     deq_one(cw, 0, 0, bf[0], 0);
     deq_one(cw, 0, 0, bf[0], 1);
@@ -341,7 +314,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
         step(kt + 5, ic<2>(), ic<1>());
     }
     // kt is a multiple of 6 here, so the stage and parity phases restart at 0; 0..5 steps remain
-    // (an even number for int4 weights, whose K is a multiple of 128 = two steps)
+    // (an even number: K is a multiple of 128 = two steps)
     const int rem = nk - kt;
     if (rem > 0) step(kt, ic<0>(), ic<0>());
     if (rem > 1) step(kt + 1, ic<1>(), ic<1>());
@@ -363,7 +336,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     unsigned char *ep = ((wave & 2) ? lds_a1 : lds_a0) + (wave & 1) * (32 * EP);
     const int ep_row = lane >> 3, ep_chunk = lane & 7;
     const int c_lane = c0 + wave * 64 + ep_chunk * 8;  // first of the 8 columns this lane stores
-    float bias_v[2][4][4], sw_v[2][4][4];
+    float bias_v[2][4][4];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -373,14 +346,10 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
             for (int e = 0; e < 4; ++e) {
                 const bool in = c + e < p.N;
                 bias_v[i][q][e] = (p.bias && in) ? lq_bf16_bits_to_f32(p.bias[c + e]) : 0.0f;
-                if constexpr (I8) sw_v[i][q][e] = in ? p.sw[c + e] : 0.0f;
             }
         }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const int m = m0 + j * 32 + r;
-        float sxm = 1.0f;
-        if constexpr (I8) sxm = m < p.M ? p.sx[m] : 0.0f;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
 #pragma unroll
@@ -388,19 +357,11 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    if constexpr (I8) v[e] = ((float)acc[i][j][4 * q + e] * sxm) * sw_v[i][q][e];
-                    else v[e] = acc[i][j][4 * q + e];
+                    v[e] = acc[i][j][4 * q + e];
                     if (p.bias) v[e] += bias_v[i][q][e];
                 }
                 u32x2_t o = {lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3])};
                 *reinterpret_cast<u32x2_t *>(ep + r * EP + (i * 32 + 8 * q + 4 * h) * 2) = o;
-                if constexpr (I8) {
-                    const int c = c0 + wave * 64 + i * 32 + 8 * q + 4 * h;
-                    if (p.acc_out && m < p.M && c < p.N) {
-                        i32x4_t a4 = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                        *reinterpret_cast<i32x4_t *>(p.acc_out + (long long)m * p.N + c) = a4;
-                    }
-                }
             }
         }
 #pragma unroll
@@ -419,15 +380,14 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
 // can fill the device two per CU.
 long long lq_gemm_fwd_direct_workgroups(int M, int N) { return (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN); }
 
-static int launch_direct(FwdParams p, bool i8, hipStream_t st, const char *who) {
+static int launch_direct(FwdParams p, hipStream_t st, const char *who) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     const long long nwg = (long long)p.tiles_m * p.tiles_n;
     if (nwg > 0x7FFFFFFFll) return lq_fail(LQ_ERR_BAD_ARG, "%s: problem too large", who);
     // the 32-bit lane offsets of the activation and weight loads span 128 / 256 rows
     if ((long long)BN * p.K * 2 >= (1ll << 32)) return lq_fail(LQ_ERR_BAD_ARG, "%s: K too large", who);
-    if (i8) hipLaunchKernelGGL(gemm_fwd_direct_kernel<true>, dim3((unsigned)nwg), dim3(256), 0, st, p);
-    else hipLaunchKernelGGL(gemm_fwd_direct_kernel<false>, dim3((unsigned)nwg), dim3(256), 0, st, p);
+    hipLaunchKernelGGL(gemm_fwd_direct_kernel, dim3((unsigned)nwg), dim3(256), 0, st, p);
     return lq_check_launch(who);
 }
 
@@ -439,15 +399,5 @@ int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scal
     p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.bias = (const unsigned short *)bias; p.y = (unsigned short *)y;
     p.M = M; p.N = N; p.K = K;
-    return launch_direct(p, false, st, "lq_a16w4_fwd");
-}
-
-// Called by lq_a8w8_fwd (lq_gemm.hip) after argument validation: K % 128 == 0, N % 16 == 0.
-int lq_gemm_i8_direct_launch(const void *x8, const void *w8, const float *sx, const float *sw, const void *bias, void *y,
-                             int *acc_or_null, int M, int N, int K, hipStream_t st) {
-    FwdParams p = {};
-    p.x = (const unsigned char *)x8; p.w = (const unsigned char *)w8; p.sx = sx; p.sw = sw;
-    p.bias = (const unsigned short *)bias; p.y = (unsigned short *)y; p.acc_out = acc_or_null;
-    p.M = M; p.N = N; p.K = K;
-    return launch_direct(p, true, st, "lq_a8w8_fwd");
+    return launch_direct(p, st, "lq_a16w4_fwd");
 }

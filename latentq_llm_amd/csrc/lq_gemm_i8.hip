@@ -1,0 +1,261 @@
+// A8W8 GEMM with 256 x 256 tiles for gfx950:
+//   Y[M,N] = bf16(((int32) X8[M,K] . W8[N,K]^T) * sx[m] * sw[n] (+ bias)), optional int32 accumulators.
+//
+// int8 operands need no dequantisation, so both operands go from global memory into LDS with
+// LDS-direct loads (no registers, no vector-ALU work) and what bounds a tile scheme is the traffic
+// between L2 and the compute units: per unit of MFMA work a 128 x 256 tile moves 1.5 times the
+// bytes of a 256 x 256 tile, and at int8 rates (twice the reduction depth per MFMA cycle of bf16)
+// that traffic, not the matrix core, set the pace of the 128 x 256 kernel.
+//
+// Workgroup: 512 threads = 8 waves in a 2 (m) x 4 (n) grid; a wave owns 128 x 64 outputs (4 x 2
+// MFMA 32x32x32 tiles, 128 accumulator registers), two waves per SIMD. One workgroup per CU: two
+// LDS stages of 64 KB (256 rows of A and 256 rows of B, 128 bytes = 128 k each).
+//
+// Reduction step = 128 k in four slices of 32. Lane l: r = l % 32, h = l / 32. In slice t the
+// lane's operand of row r is chunk 4h + t (16 bytes) of the row's 128 bytes, for A and B alike
+// (any assignment of k to slices and halves is valid as long as both operands use the same one).
+// Chunk c of tile row x sits at position c ^ ((x >> 1) & 7): fragment reads are conflict-free and
+// the swizzle is free, since an LDS-direct load lets a lane choose the global chunk that lands in
+// its fixed LDS slot.
+//
+// Pipeline: one s_barrier per step, before the last slice. Past it every wave's fragment reads of
+// the current stage have returned, so the last slice and the next step's first slice issue the
+// loads of the step after next into it (4 per thread each), while the last slice already reads
+// the next stage's first fragments; the wait in front of the barrier covers those loads one step
+// later. Loads are inline assembly with explicit waits, as in the other GEMM kernels.
+//
+// D = Wfrag x Xfrag^T: a lane owns 4 consecutive n of one m; the epilogue applies the scales and
+// regroups the bf16 results through LDS into 16-byte pieces of full output rows.
+#include "lq_common.h"
+
+#include <type_traits>
+
+namespace {
+
+struct I8Params {
+    const unsigned char *x;  // int8 [M, K]
+    const unsigned char *w;  // int8 [N, K]
+    const float *sx;         // [M]
+    const float *sw;         // [N]
+    const unsigned short *bias;  // bf16 [N] or null
+    int *acc_out;                // optional int32 [M, N]
+    unsigned short *y;           // bf16 [M, N]
+    int M, N, K;
+    int tiles_m, tiles_n;
+};
+
+typedef __attribute__((address_space(3))) void lds_void;
+
+template <int I>
+using ic = std::integral_constant<int, I>;
+
+constexpr int BM = 256, BN = 256;
+constexpr int ROWB = 128;                   // bytes (= k) per tile row and step
+constexpr int A_STAGE = BM * ROWB;          // 32 KB
+constexpr int STAGE = (BM + BN) * ROWB;     // 64 KB: A rows, then B rows
+constexpr int NT = 512;
+
+__global__ __launch_bounds__(NT) void gemm_i8_256_kernel(I8Params p) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds0[STAGE];
+    __shared__ __attribute__((aligned(16))) unsigned char lds1[STAGE];
+    auto stage = [&](auto i) -> unsigned char * {
+        constexpr int I = decltype(i)::value;
+        return I == 0 ? lds0 : lds1;
+    };
+
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int r = lane & 31, h = lane >> 5;
+    const int wm = wave & 1, wn = wave >> 1;
+
+    // Workgroup ids are dealt round-robin over the 8 XCDs (id % 8): give each XCD a contiguous
+    // range of the tile sequence, ordered in bands of GN tile columns walked row by row, so the
+    // workgroups resident on one XCD share a few A row-blocks and B column-blocks in its L2.
+    const int nwg = p.tiles_m * p.tiles_n;
+    int id = blockIdx.x;
+    {
+        const int per = nwg / 8;
+        if (id < per * 8) id = (id % 8) * per + id / 8;
+    }
+    constexpr int GN = 8;
+    const int band = id / (p.tiles_m * GN);
+    const int within = id - band * (p.tiles_m * GN);
+    const int rest = p.tiles_n - band * GN;
+    const int bw = rest < GN ? rest : GN;
+    const int tile_m = within / bw, tile_n = band * GN + within % bw;
+    const int m0 = tile_m * BM, c0 = tile_n * BN;
+    const int nk = p.K / ROWB;
+
+    // ---- staging: 2048 16-byte slots per operand and stage; slot s = i*512 + thread -> row s/8,
+    // position s%8. Rows past the end of a matrix re-read its last row (their results are dropped).
+    unsigned a_off[4], b_off[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = i * 64 + (int)(threadIdx.x >> 3);
+        const int pos = threadIdx.x & 7;
+        const int chunk = pos ^ ((row >> 1) & 7);
+        int ga = m0 + row, gb = c0 + row;
+        ga = ga < p.M ? ga : p.M - 1;
+        gb = gb < p.N ? gb : p.N - 1;
+        a_off[i] = (unsigned)((long long)(ga - m0) * p.K + chunk * 16);
+        b_off[i] = (unsigned)((long long)(gb - c0) * p.K + chunk * 16);
+    }
+    const unsigned char *a_base = p.x + (long long)m0 * p.K;
+    const unsigned char *b_base = p.w + (long long)c0 * p.K;
+    // load i (0..7) of a step: 0..3 fill the A rows of the stage, 4..7 its B rows
+    auto issue_one = [&](int kt, unsigned char *st, int i) {
+        const bool is_b = i >= 4;
+        const unsigned char *src = (is_b ? b_base : a_base) + (long long)kt * ROWB;
+        const unsigned lds_addr = (unsigned)reinterpret_cast<size_t>(
+            (lds_void *)(st + (is_b ? A_STAGE : 0) + ((i & 3) * NT + wave * 64) * 16));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :: "s"(lds_addr), "v"(is_b ? b_off[i & 3] : a_off[i & 3]), "s"(src) : "memory");
+    };
+
+    // ---- fragments: tile row x + r, chunk (4h + t) at position chunk ^ ((r >> 1) & 7)
+    int frag[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) frag[t] = r * ROWB + (((4 * h + t) ^ ((r >> 1) & 7)) << 4);
+    const int a_rows = wm * 128 * ROWB, b_rows = A_STAGE + wn * 64 * ROWB;
+    auto read_frags = [&](const unsigned char *st, int t, u32x4_t *af, u32x4_t *bf) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) af[j] = *reinterpret_cast<const u32x4_t *>(st + a_rows + j * 32 * ROWB + frag[t]);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) bf[i] = *reinterpret_cast<const u32x4_t *>(st + b_rows + i * 32 * ROWB + frag[t]);
+    };
+
+    i32x16_t acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0;
+
+    u32x4_t af[2][4], bf[2][2];
+    // Step kt on stage S: the operands of its first slice are already in af[0] / bf[0].
+    auto step = [&](int kt, auto si) {
+        constexpr int S = decltype(si)::value;
+        unsigned char *cur = stage(ic<S>()), *nxt = stage(ic<S ^ 1>());
+        const int kt1 = kt + 1 < nk ? kt + 1 : nk - 1, kt2 = kt + 2 < nk ? kt + 2 : nk - 1;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            if (t == 3) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            if (t < 3) read_frags(cur, t + 1, af[(t + 1) & 1], bf[(t + 1) & 1]);
+            else read_frags(nxt, 0, af[0], bf[0]);
+            if (t == 0) {
+                // second half of the next step's loads (its stage was released by the previous barrier)
+#pragma unroll
+                for (int i = 4; i < 8; ++i) issue_one(kt1, nxt, i);
+            }
+            if (t == 3) {
+                // first half of the loads of the step after next, into the stage just released
+#pragma unroll
+                for (int i = 0; i < 4; ++i) issue_one(kt2, cur, i);
+            }
+            // the reads and loads above go out before this slice's MFMAs, which cover their latency
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf[t & 1][i]),
+                                                                     __builtin_bit_cast(i32x4_t, af[t & 1][j]), acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // prologue: step 0 entirely, the first half of step 1; wait for step 0 (all but the 4 newest)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) issue_one(0, lds0, i);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) issue_one(nk > 1 ? 1 : 0, lds1, i);
+    asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");
+    read_frags(lds0, 0, af[0], bf[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    int kt = 0;
+    for (; kt + 2 <= nk; kt += 2) {
+        step(kt, ic<0>());
+        step(kt + 1, ic<1>());
+    }
+    if (kt < nk) step(kt, ic<0>());
+    // the clamped prefetches of the last steps are still writing LDS: drain them
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    // ---- epilogue: acc[i][j][q]: column c0 + 64*wn + 32i + 8*(q/4) + 4h + q%4, row m0 + 128*wm + 32j + r.
+    // Every wave passes its block through a private LDS area, 32 rows (one j) at a time, and stores
+    // 16 bytes per lane with 8 lanes on the 128 contiguous bytes of a row: full cache lines.
+    __syncthreads();
+    constexpr int EP = 144;  // row pitch of the staging area
+    unsigned char *ep = lds0 + wave * (32 * EP);
+    const int ep_row = lane >> 3, ep_chunk = lane & 7;
+    const int cw0 = c0 + wn * 64;
+    const int c_lane = cw0 + ep_chunk * 8;  // first of the 8 columns this lane stores
+    float bias_v[2][4][4], sw_v[2][4][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int c = cw0 + i * 32 + 8 * q + 4 * h;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const bool in = c + e < p.N;
+                bias_v[i][q][e] = (p.bias && in) ? lq_bf16_bits_to_f32(p.bias[c + e]) : 0.0f;
+                sw_v[i][q][e] = in ? p.sw[c + e] : 0.0f;
+            }
+        }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int mrow0 = m0 + wm * 128 + j * 32;
+        const int m = mrow0 + r;
+        const float sxm = m < p.M ? p.sx[m] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = ((float)acc[i][j][4 * q + e] * sxm) * sw_v[i][q][e];
+                    if (p.bias) v[e] += bias_v[i][q][e];
+                }
+                u32x2_t o = {lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3])};
+                *reinterpret_cast<u32x2_t *>(ep + r * EP + (i * 32 + 8 * q + 4 * h) * 2) = o;
+                const int c = cw0 + i * 32 + 8 * q + 4 * h;
+                if (p.acc_out && m < p.M && c < p.N) {
+                    i32x4_t a4 = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                    *reinterpret_cast<i32x4_t *>(p.acc_out + (long long)m * p.N + c) = a4;
+                }
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int row = it * 8 + ep_row;
+            const u32x4_t o = *reinterpret_cast<const u32x4_t *>(ep + row * EP + ep_chunk * 16);
+            const int mm = mrow0 + row;
+            if (mm < p.M && c_lane < p.N) *reinterpret_cast<u32x4_t *>(p.y + (long long)mm * p.N + c_lane) = o;
+        }
+    }
+}
+
+}  // namespace
+
+// Number of 256 x 256 tiles of an [M, N] output.
+long long lq_gemm_i8_256_workgroups(int M, int N) { return (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN); }
+
+// Called by lq_a8w8_fwd (lq_gemm.hip) after argument validation: K % 128 == 0, N % 16 == 0.
+int lq_gemm_i8_256_launch(const void *x8, const void *w8, const float *sx, const float *sw, const void *bias, void *y,
+                          int *acc_or_null, int M, int N, int K, hipStream_t st) {
+    I8Params p = {};
+    p.x = (const unsigned char *)x8; p.w = (const unsigned char *)w8; p.sx = sx; p.sw = sw;
+    p.bias = (const unsigned short *)bias; p.y = (unsigned short *)y; p.acc_out = acc_or_null;
+    p.M = M; p.N = N; p.K = K;
+    p.tiles_m = (M + BM - 1) / BM;
+    p.tiles_n = (N + BN - 1) / BN;
+    const long long nwg = (long long)p.tiles_m * p.tiles_n;
+    if (nwg > 0x7FFFFFFFll) return lq_fail(LQ_ERR_BAD_ARG, "lq_a8w8_fwd: problem too large");
+    // the 32-bit lane offsets of the loads span 256 rows
+    if ((long long)BN * K >= (1ll << 32)) return lq_fail(LQ_ERR_BAD_ARG, "lq_a8w8_fwd: K too large");
+    hipLaunchKernelGGL(gemm_i8_256_kernel, dim3((unsigned)nwg), dim3(NT), 0, st, p);
+    return lq_check_launch("lq_a8w8_fwd");
+}

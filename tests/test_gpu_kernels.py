@@ -269,7 +269,9 @@ def test_a16w4_adjoint_identity(ops):
 @pytest.mark.parametrize("M,N,K,bias", [(17, 16, 128, False), (64, 128, 256, True), (130, 272, 384, False),
                                         (300, 512, 1024, True), (2048, 2048, 2048, False),
                                         # ragged and large enough for the weights-direct kernel; odd number of K steps
-                                        (4100, 4112, 384, True)])
+                                        (4100, 4112, 384, True),
+                                        # one and two K steps through the 256 x 256 tile kernel
+                                        (3600, 3648, 128, False), (3330, 3840, 256, True)])
 def test_a8w8(ops, co, M, N, K, bias):
     g = torch.Generator().manual_seed(M + N + K)
     x8 = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
