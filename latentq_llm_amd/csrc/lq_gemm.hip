@@ -716,12 +716,22 @@ static int a16w4_fwd_impl(const char *who, const void *x, const void *codes, con
         rc = launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
         return rc ? rc : launch_split_reduce(p, splits, (hipStream_t)stream, who);
     }
-    // Two forward kernels. The weights-direct one (128 x 256 tiles, two workgroups per CU) wins when
-    // its tiles give every CU a workgroup; otherwise the staged kernel. The weights-direct kernel
+    // Three forward kernels, chosen by a rough time per 64-deep step (microseconds, measured): the
+    // weights-direct kernel (128 x 256 tiles) takes ~0.86 with one workgroup on a compute unit and
+    // ~1.45 for two sharing it; the staged kernel ~0.56 per round of 128 x 128 tiles and ~0.88 per
+    // round of 256 x 128 tiles (one workgroup per unit and round). The weights-direct kernel
     // loads scales and zeros four groups at a time: rows must be 4-byte aligned.
-    if (lq_gemm_fwd_direct_workgroups((int)M, (int)N) >= 1ll * lq_device_cu_count() && (K / LQ_GROUP) % 2 == 0)
+    const long long cus = lq_device_cu_count();
+    const long long wg_direct = lq_gemm_fwd_direct_workgroups((int)M, (int)N);
+    const long long rem = wg_direct % (2 * cus);
+    const double est_direct = (K / LQ_GROUP) % 2 != 0 ? 1e30
+                              : 1.45 * (double)(wg_direct / (2 * cus)) + (rem == 0 ? 0.0 : rem <= cus ? 0.86 : 1.45);
+    const long long cols = (N + 127) / 128;
+    const double est_small = 0.56 * (double)((((M + 127) / 128) * cols + cus - 1) / cus);
+    const double est_big = 0.88 * (double)((((M + 255) / 256) * cols + cus - 1) / cus);
+    if (est_direct <= est_small && est_direct <= est_big)
         return lq_gemm_fwd_direct_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
-    if (small_tiles(p)) return launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
+    if (est_small <= est_big) return launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
     return launch_gemm<MODE_W4_FWD, 256, 128, 2, 2>(p, (hipStream_t)stream, who);
 }
 
