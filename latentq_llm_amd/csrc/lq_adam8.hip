@@ -69,16 +69,46 @@ __device__ __forceinline__ void block_minmax(float &lo, float &hi, float (*red)[
     }
 }
 
-// x[8] -> uint8 codes with the block's (scale, max); returns them packed, 8 bytes
+// x[8] -> uint8 codes with the block's (scale, max); returns them packed, 8 bytes.
+// The quotient (hi - x) / scale must be the correctly rounded one (a quotient one ulp off can fall
+// on the other side of a rounding tie). The divisor is shared by the whole block, so the division
+// is done with its correctly rounded reciprocal r = RN(1 / scale) and two residual corrections:
+// q0 = t*r; q1 = q0 + (t - q0*scale)*r is within one ulp of t/scale, and one more correction of a
+// quotient within one ulp returns RN(t / scale) exactly (Markstein's theorem; the residuals are
+// exact as long as they do not underflow, and a numerator below 2^-100 gives code 0 either way
+// because scale >= 1e-10). Half the instructions of an IEEE division. A scale above 2^60 (or NaN)
+// takes the plain division.
 __device__ __forceinline__ u32x2_t quantize8(const float x[8], float scale, float hi) {
     unsigned w[2] = {0u, 0u};
+    const bool fast = scale <= 0x1p60f;
+    const float r = 1.0f / scale;
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-        float q = rintf((hi - x[k]) / scale);
+        const float t = hi - x[k];
+        float q;
+        if (fast) {
+            const float q0 = t * r;
+            const float q1 = fmaf(fmaf(-q0, scale, t), r, q0);
+            q = fmaf(fmaf(-q1, scale, t), r, q1);
+        } else {
+            q = t / scale;
+        }
+        q = rintf(q);
         q = fminf(fmaxf(q, 0.0f), 255.0f);
         w[k >> 2] |= ((unsigned)q & 0xFFu) << (8 * (k & 3));
     }
     return u32x2_t{w[0], w[1]};
+}
+
+// bf16(sqrt(v)) for a bf16 value v. The square root of a number with 8 significant bits never
+// comes closer than 2^-19 (relative) to the midpoint of two bf16 values, so any fp32 square root
+// within two ulps rounds to the same bf16 value as the correctly rounded one (checked for every
+// bf16 input by the CPU tests); the hardware's v_sqrt_f32 (one ulp) replaces the ~12-instruction
+// correctly rounded sequence. Inputs below 2^-100 (the instruction does not take denormals) go
+// through the exact one.
+__device__ __forceinline__ float sqrt_bf16_to_bf16(float v) {
+    if (v >= 0x1p-100f) return bf16r(__builtin_amdgcn_sqrtf(v));
+    return bf16r(__builtin_sqrtf(v));
 }
 
 template <int BS, bool LATENT>
@@ -117,7 +147,7 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
         mk = bf16r(fmaf(a.one_minus_beta1, g, mk));
         vk = bf16r(vk * a.beta2);
         vk = bf16r(fmaf(a.one_minus_beta2 * g, g, vk));
-        float dk = bf16r(__builtin_sqrtf(vk));
+        float dk = sqrt_bf16_to_bf16(vk);
         dk = bf16r(dk + a.eps);
         m[k] = mk;
         d[k] = dk;

@@ -265,3 +265,52 @@ def test_gptq_layout_brute_force():
     for n, k in [(0, 0), (3, 7), (15, 127), (9, 64), (1, 9)]:
         assert (int(gptq[k // 8, n]) >> (4 * (k % 8))) & 15 == int(codes[n, k])
     assert np.array_equal(co.gptq_to_native(gptq, N, K), packed.numpy().view(np.uint8))
+
+
+# ------------------------------------------- shortcuts of the fused Adam kernel --
+def _bf16_rne_bits(x32: np.ndarray) -> np.ndarray:
+    u = x32.view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint32)
+
+
+def test_sqrt_of_bf16_rounds_the_same_within_two_ulps():
+    """Every finite bf16 v >= 2^-100: all fp32 values within two ulps of the correctly rounded
+    sqrt(v) round to the same bf16 value, so a one-ulp hardware square root may stand in for the
+    correctly rounded one before the bf16 rounding (what the fused Adam kernel does)."""
+    b = np.arange(0x0000, 0x7F80, dtype=np.uint32)  # all non-negative finite bf16 bit patterns
+    v = (b << 16).view(np.float32)
+    v = v[v >= np.float32(2.0 ** -100)]
+    assert v.size > 28_000
+    exact = np.sqrt(v)  # IEEE: correctly rounded in fp32
+    want = _bf16_rne_bits(exact)
+    for d in (-2, -1, 1, 2):
+        near = (exact.view(np.int32) + d).view(np.float32)
+        assert np.array_equal(_bf16_rne_bits(near), want), d
+    # and the margin is wide: the closest approach to a rounding tie, in fp32 ulps
+    frac = exact.view(np.uint32) & 0xFFFF
+    assert int(np.abs(frac.astype(np.int64) - 0x8000).min()) > 8
+
+
+def test_two_step_reciprocal_division_equals_ieee_division():
+    """q0 = t*r, q1 = q0 + (t - q0*s)*r, q2 = q1 + (t - q1*s)*r with r = RN(1/s) returns RN(t/s):
+    the quotient of the 8-bit moment quantiser (numerators in [0, 255*s], s >= 1e-10), checked on
+    random and adversarial operands in float64-backed exact arithmetic."""
+    rng = np.random.default_rng(5)
+    n = 2_000_000
+    s = np.exp(rng.uniform(np.log(1e-10), np.log(1e3), n)).astype(np.float32)
+    # numerators: random in [0, 255 s], plus values next to rounding ties of the quotient
+    q_target = rng.uniform(0, 255.5, n)
+    q_target[: n // 2] = np.floor(q_target[: n // 2]) + 0.5
+    t = (q_target * s.astype(np.float64)).astype(np.float32)
+    t[: n // 4] = np.nextafter(t[: n // 4], np.float32(np.inf))
+    t[n // 4: n // 2: 2] = np.nextafter(t[n // 4: n // 2: 2], np.float32(0))
+    want = t / s  # IEEE fp32 division
+    r = np.float32(1.0) / s
+
+    def fma(a, b, c):  # exact product and sum in float64 (24 x 24 bits fit), one rounding to fp32
+        return (a.astype(np.float64) * b.astype(np.float64) + c.astype(np.float64)).astype(np.float32)
+
+    q0 = t * r
+    q1 = fma(fma(-q0, s, t), r, q0)
+    q2 = fma(fma(-q1, s, t), r, q1)
+    assert np.array_equal(q2.view(np.uint32), want.view(np.uint32))
