@@ -1,0 +1,110 @@
+"""GPU tests under HIP graph capture: the C-ABI entry points neither allocate nor synchronise, so a
+decode or prefill step built from them can be captured once and replayed. Every replay is checked
+against the eager result for the same inputs, with eager work and synchronisations between the
+replays (a graph node that only works on its first replay would show here)."""
+import pytest
+import torch
+
+from tests.util import make_w4, randn_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops(hip_lib):
+    assert torch.cuda.is_available()
+    from latentq_llm_amd import ops
+    return ops
+
+
+def dev(t):
+    return t.cuda()
+
+
+class _Mlp:
+    """down(silu(gate(x)) * up(x)) on preallocated buffers (nothing is allocated inside step())."""
+
+    def __init__(self, ops, M, hid, ffn):
+        self.ops, self.shape = ops, (M, hid, ffn)
+        self.gate = [dev(t) for t in make_w4(ffn, hid, 1)[1:]]
+        self.up = [dev(t) for t in make_w4(ffn, hid, 2)[1:]]
+        self.down = [dev(t) for t in make_w4(hid, ffn, 3)[1:]]
+        self.x = torch.zeros(M, hid, dtype=torch.bfloat16, device="cuda")
+        self.g = torch.empty(M, ffn, dtype=torch.bfloat16, device="cuda")
+        self.u = torch.empty_like(self.g)
+        self.h = torch.empty_like(self.g)
+        self.y = torch.empty(M, hid, dtype=torch.bfloat16, device="cuda")
+
+    def step(self):
+        M, hid, ffn = self.shape
+        o = self.ops
+        o.a16w4_forward(self.x, *self.gate, (ffn, hid), out=self.g)
+        o.a16w4_forward(self.x, *self.up, (ffn, hid), out=self.u)
+        torch.mul(torch.nn.functional.silu(self.g), self.u, out=self.h)
+        o.a16w4_forward(self.h, *self.down, (hid, ffn), out=self.y)
+
+
+# M = 4: the GEMV; M = 48: the GEMV in chunks or the split reduction; M = 200: split reduction with the
+# scratch buffer (allocated by the eager warm-up, before the capture); M = 640: plain GEMM kernels
+@pytest.mark.parametrize("M,hid,ffn", [(4, 512, 1408), (48, 1024, 2816), (200, 1024, 2816), (640, 512, 1408)])
+def test_mlp_forward_replays_match_eager(ops, M, hid, ffn):
+    blk = _Mlp(ops, M, hid, ffn)
+    inputs = [dev(randn_bf16((M, hid), 10 + i)) for i in range(4)]
+    want = []
+    for x in inputs:  # eager results (also the warm-up that sizes the scratch buffer)
+        blk.x.copy_(x)
+        blk.step()
+        want.append(blk.y.clone())
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        blk.step()  # warm-up on the capture stream (its own scratch buffer)
+    torch.cuda.current_stream().wait_stream(s)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=s):
+        blk.step()
+    for rep in range(2):
+        for x, w in zip(inputs, want):
+            blk.x.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(blk.y, w), f"replay differs from eager (M={M}, pass {rep})"
+            # eager work between replays, through the same entry points and the same scratch
+            blk.x.copy_(inputs[0])
+            blk.step()
+            torch.cuda.synchronize()
+            assert torch.equal(blk.y, want[0])
+
+
+def test_requant_and_a8w8_replay(ops):
+    """The requantizer (seed and offset are launch arguments, fixed at capture) and the int8 GEMM."""
+    N, K = 256, 1024
+    _, packed, scales, zeros = make_w4(N, K, 5)
+    p, sc, z = dev(packed), dev(scales), dev(zeros)
+    grad = torch.zeros(N, K, dtype=torch.bfloat16, device="cuda")
+    out = torch.empty_like(p)
+    x8 = torch.zeros(300, K, dtype=torch.int8, device="cuda")
+    w8 = torch.randint(-127, 128, (N, K), dtype=torch.int8, device="cuda")
+    sx, sw = torch.rand(300, device="cuda") + 0.1, torch.rand(N, device="cuda") + 0.1
+    grads = [dev(randn_bf16((N, K), 20 + i, 1e-3)) for i in range(3)]
+    xs = [torch.randint(-127, 128, (300, K), dtype=torch.int8, device="cuda") for _ in range(3)]
+    want = []
+    for g, x in zip(grads, xs):
+        want.append((ops.requant_sr(p, sc, z, g, 1e-2, (N, K), seed=9, offset=3).clone(), ops.a8w8_forward(x, w8, sx, sw).clone()))
+    y8 = [None]
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=s):
+        ops.requant_sr(p, sc, z, grad, 1e-2, (N, K), seed=9, offset=3, out=out)
+        y8[0] = ops.a8w8_forward(x8, w8, sx, sw)
+    for rep in range(2):
+        for (g, x), (wc, wy) in zip(zip(grads, xs), want):
+            grad.copy_(g)
+            x8.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, wc) and torch.equal(y8[0], wy), f"pass {rep}"
+            ops.requant_sr(p, sc, z, grads[0], 1e-2, (N, K), seed=1, offset=0)  # eager work in between
+            torch.cuda.synchronize()
