@@ -393,3 +393,24 @@ def test_workspace_entry_points_without_a_workspace_match_the_plain_ones(ops):
     _C.call("lq_a16w4_fwd", x.data_ptr(), p.data_ptr(), s.data_ptr(), z.data_ptr(), None, y0.data_ptr(), M, N, K, 128, st)
     y1 = ops.a16w4_forward(x, p, s, z, (N, K))
     assert rel_l2(y1.float().cpu(), y0.float().cpu()) < 4e-3
+
+
+@pytest.mark.parametrize("slices", [0, 1, 2, 3, 8])
+def test_workspace_smaller_than_wanted_is_used_as_far_as_it_goes(ops, slices):
+    """A scratch buffer that holds fewer slices than the planner would like (or none) only changes the
+    split, never the validity: results stay within the output rounding of the plain entry point."""
+    from latentq_llm_amd import _C
+    M, N, K = 128, 2048, 1024  # dX: 16 tiles of 128 x 128, 32 reduction steps: up to 4 slices of 8 steps
+    codes, packed, scales, zeros = make_w4(N, K, 77)
+    dy, p, s, z = dev(randn_bf16((M, N), 78)), dev(packed), dev(scales), dev(zeros)
+    st = torch.cuda.current_stream().cuda_stream
+    ref = torch.empty(M, K, dtype=torch.bfloat16, device="cuda")
+    _C.call("lq_a16w4_dx", dy.data_ptr(), p.data_ptr(), s.data_ptr(), z.data_ptr(), ref.data_ptr(), M, N, K, 128, st)
+    nbytes = slices * M * K * 4 + 64
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    out = torch.empty_like(ref)
+    _C.call("lq_a16w4_dx_ws", dy.data_ptr(), p.data_ptr(), s.data_ptr(), z.data_ptr(), out.data_ptr(), M, N, K, 128,
+            ws.data_ptr(), nbytes, st)
+    assert rel_l2(out.float().cpu(), ref.float().cpu()) < 4e-3
+    if slices < 2:
+        assert torch.equal(out, ref)  # no room for a split: the same kernel as the plain entry point
