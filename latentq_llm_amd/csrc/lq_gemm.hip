@@ -628,38 +628,43 @@ static int check_w4_common(const char *who, const void *a, const void *codes, co
     return LQ_OK;
 }
 
-// Rough time of a grid of 128 x 128 tiles in microseconds (measured): a workgroup alone on a compute
-// unit takes ~0.56 per 64-deep step and two on one unit take twice that each, so what counts is the
-// number of rounds of one workgroup per unit; prologue and epilogue cost about three steps, the
-// launch ~4 us.
-static double gemm128_est_us(long long workgroups, int steps) {
-    const long long cus = lq_device_cu_count();
-    return 0.56 * (steps + 3) * (double)((workgroups + cus - 1) / cus) + 4.0;
-}
+// Split reduction for grids that fill less than half of the compute units: the reduction is cut
+// into up to 8 slices of an even number of steps (at least 8) so that every unit gets at most one
+// workgroup, fp32 partial tiles go to the caller's workspace, then a reduce kernel adds them. Both
+// staged tile heights are tried (128 x 128 at ~0.56 us per step, 256 x 128 at pace_big); the plan
+// with the smaller estimated time is returned (splits = 1: do not split). The estimate counts the
+// partial tiles written and read back through the last-level cache at ~5 TB/s and ~3 us for the
+// second launch.
+struct SplitPlan {
+    int splits = 1, steps_per_split = 0;
+    bool big = false;
+    double est_us = 1e30;
+};
 
-// Split reduction for grids that fill less than half of the compute units: 128 x 128 tiles, the
-// reduction cut into up to 8 slices of an even number of steps (at least 8) so that every unit
-// gets at most one workgroup, fp32 partial tiles in the caller's workspace, then a reduce kernel.
-// Returns the number of slices (1 = do not split) and the estimated time in microseconds (the
-// partial tiles are written and read back through the last-level cache at ~5 TB/s; ~3 us for the
-// second launch).
-static int plan_split(long long M, long long C, int total_steps, size_t ws_bytes, int *steps_per_split, double *est_us) {
-    const long long tiles = ((M + 127) / 128) * ((C + 127) / 128);
+static SplitPlan plan_split(long long M, long long C, int total_steps, size_t ws_bytes, double pace_big) {
+    SplitPlan best;
+    if (!ws_bytes) return best;
     const long long cus = lq_device_cu_count();
-    if (!ws_bytes || tiles * 2 > cus) return 1;
-    long long S = cus / tiles;
-    if (S > 8) S = 8;
     const long long fit = (long long)(ws_bytes / ((size_t)M * C * 4));
-    if (S > fit) S = fit;
-    if (S < 2) return 1;
-    int per = (int)((total_steps + S - 1) / S);
-    per += per & 1;
-    if (per < 8) per = 8;
-    S = (total_steps + per - 1) / per;
-    if (S < 2) return 1;
-    *steps_per_split = per;
-    *est_us = gemm128_est_us(tiles * S, per) + 3.0 + 2.0 * S * M * C * 4 / 5.0e6;
-    return (int)S;
+    for (int big = 0; big < 2; ++big) {
+        const long long tiles = ((M + (big ? 255 : 127)) / (big ? 256 : 128)) * ((C + 127) / 128);
+        if (tiles * 2 > cus) continue;
+        long long S = cus / tiles;
+        if (S > 8) S = 8;
+        if (S > fit) S = fit;
+        if (S < 2) continue;
+        int per = (int)((total_steps + S - 1) / S);
+        per += per & 1;
+        if (per < 8) per = 8;
+        S = (total_steps + per - 1) / per;
+        if (S < 2) continue;
+        const double est = (big ? pace_big : 0.56) * (per + 3) * (double)((tiles * S + cus - 1) / cus) + 4.0 + 3.0 +
+                           2.0 * S * M * C * 4 / 5.0e6;
+        if (est < best.est_us) {
+            best.splits = (int)S; best.steps_per_split = per; best.big = big != 0; best.est_us = est;
+        }
+    }
+    return best;
 }
 
 static int launch_split_reduce(const GemmParams &p, int splits, hipStream_t st, const char *who) {
@@ -678,24 +683,36 @@ static int a16w4_fwd_impl(const char *who, const void *x, const void *codes, con
     LQ_REQUIRE(!workspace || lq_aligned(workspace, 16), "%s: the workspace must be 16-byte aligned", who);
     if (M <= 16)
         return lq_gemv_a16w4_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
-    int per = 0;
-    double est_split = 0.0;
-    const int splits = plan_split(M, N, (int)(K / 64), workspace ? ws_bytes : 0, &per, &est_split);
-    const long long tiles = ((M + 127) / 128) * ((N + 127) / 128);
-    const double est_gemm = gemm128_est_us(tiles, (int)(K / 64));
+    // Rough time per 64-deep step of the three forward kernels without a split (microseconds,
+    // measured): the weights-direct kernel (128 x 256 tiles) takes ~0.86 with one workgroup on a
+    // compute unit and ~1.45 for two sharing it; the staged kernel ~0.56 per round of 128 x 128
+    // tiles and ~0.88 per round of 256 x 128 tiles (one workgroup per unit and round). The
+    // weights-direct kernel loads scales and zeros four groups at a time: rows must be 4-byte aligned.
+    const long long cus = lq_device_cu_count();
+    const long long wg_direct = lq_gemm_fwd_direct_workgroups((int)M, (int)N);
+    const long long rem = wg_direct % (2 * cus);
+    const double est_direct = (K / LQ_GROUP) % 2 != 0 ? 1e30
+                              : 1.45 * (double)(wg_direct / (2 * cus)) + (rem == 0 ? 0.0 : rem <= cus ? 0.86 : 1.45);
+    const long long cols = (N + 127) / 128;
+    const double est_small = 0.56 * (double)((((M + 127) / 128) * cols + cus - 1) / cus);
+    const double est_big = 0.88 * (double)((((M + 255) / 256) * cols + cus - 1) / cus);
+    const double step_us = est_direct < est_small ? (est_direct < est_big ? est_direct : est_big)
+                                                  : (est_small < est_big ? est_small : est_big);
+    const double est_gemm = step_us * (double)(K / 64 + 3) + 4.0;
+    const SplitPlan plan = plan_split(M, N, (int)(K / 64), workspace ? ws_bytes : 0, 0.88);
     if (M <= 128) {
         // A few more tokens than one GEMV takes: the GEMM's 128-row tiles would be mostly padding and
         // its grid (N/128 workgroups, each walking all of K) fills a fraction of the device, so
         // chunks of 16 tokens through the GEMV can be faster: the first streams the weights from
         // HBM at near memory speed, the others find them in the last-level cache. Rough costs in
-        // microseconds: the GEMM as gemm128_est_us has it; a GEMV chunk its bytes at ~1.8 TB/s the
-        // first time (at least 6) and ~2.3 TB/s after (at least 5; measured).
+        // microseconds: a GEMV chunk takes its bytes at ~1.8 TB/s the first time (at least 6) and
+        // ~2.3 TB/s after (at least 5; measured).
         const int chunks = (int)((M + 15) / 16);
         const double bytes = (double)(N * K / 2 + N * (K / LQ_GROUP) * 4);
         const double first_us = bytes / 1.8e6 > 6.0 ? bytes / 1.8e6 : 6.0;
         const double next_us = bytes / 2.3e6 > 5.0 ? bytes / 2.3e6 : 5.0;
         const double est_gemv = first_us + (chunks - 1) * next_us;
-        if (est_gemv < est_gemm && (splits < 2 || est_gemv < est_split)) {
+        if (est_gemv < est_gemm && est_gemv < plan.est_us) {
             for (int c = 0; c < chunks; ++c) {
                 const int rows = (int)(M - 16 * c < 16 ? M - 16 * c : 16);
                 rc = lq_gemv_a16w4_launch((const unsigned short *)x + (long long)c * 16 * K, codes, scales, zeros,
@@ -710,25 +727,13 @@ static int a16w4_fwd_impl(const char *who, const void *x, const void *codes, con
     p.a = x; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.bias = (const unsigned short *)bias_or_null; p.c = y;
     p.M = (int)M; p.C = (int)N; p.R = (int)K; p.Kw = (int)K;
-    if (splits >= 2 && est_split < est_gemm) {
+    if (plan.splits >= 2 && plan.est_us < est_gemm) {
         p.partial = (float *)workspace;
-        p.steps_per_split = per;
-        rc = launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
-        return rc ? rc : launch_split_reduce(p, splits, (hipStream_t)stream, who);
+        p.steps_per_split = plan.steps_per_split;
+        rc = plan.big ? launch_gemm<MODE_W4_FWD, 256, 128, 2, 2>(p, (hipStream_t)stream, who)
+                      : launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
+        return rc ? rc : launch_split_reduce(p, plan.splits, (hipStream_t)stream, who);
     }
-    // Three forward kernels, chosen by a rough time per 64-deep step (microseconds, measured): the
-    // weights-direct kernel (128 x 256 tiles) takes ~0.86 with one workgroup on a compute unit and
-    // ~1.45 for two sharing it; the staged kernel ~0.56 per round of 128 x 128 tiles and ~0.88 per
-    // round of 256 x 128 tiles (one workgroup per unit and round). The weights-direct kernel
-    // loads scales and zeros four groups at a time: rows must be 4-byte aligned.
-    const long long cus = lq_device_cu_count();
-    const long long wg_direct = lq_gemm_fwd_direct_workgroups((int)M, (int)N);
-    const long long rem = wg_direct % (2 * cus);
-    const double est_direct = (K / LQ_GROUP) % 2 != 0 ? 1e30
-                              : 1.45 * (double)(wg_direct / (2 * cus)) + (rem == 0 ? 0.0 : rem <= cus ? 0.86 : 1.45);
-    const long long cols = (N + 127) / 128;
-    const double est_small = 0.56 * (double)((((M + 127) / 128) * cols + cus - 1) / cus);
-    const double est_big = 0.88 * (double)((((M + 255) / 256) * cols + cus - 1) / cus);
     if (est_direct <= est_small && est_direct <= est_big)
         return lq_gemm_fwd_direct_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
     if (est_small <= est_big) return launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
@@ -759,19 +764,22 @@ static int a16w4_dx_impl(const char *who, const void *dy, const void *codes, con
     p.a = dy; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.c = dx;
     p.M = (int)M; p.C = (int)K; p.R = (int)N; p.Kw = (int)K;
-    int per = 0;
-    double est_split = 0.0;
-    const int splits = plan_split(M, K, (int)(N / 64), workspace ? ws_bytes : 0, &per, &est_split);
-    if (splits >= 2) {
-        const long long tiles = ((M + 127) / 128) * ((K + 127) / 128);
-        if (est_split < gemm128_est_us(tiles, (int)(N / 64))) {
-            p.partial = (float *)workspace;
-            p.steps_per_split = per;
-            rc = launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
-            return rc ? rc : launch_split_reduce(p, splits, (hipStream_t)stream, who);
-        }
+    // without a split: rounds of one workgroup per compute unit at ~0.54 us per 64-deep step for
+    // 128 x 128 tiles, ~0.75 for 256 x 128 (the comparison small_tiles() makes for the int8 path)
+    const long long cus = lq_device_cu_count();
+    const long long cols = (K + 127) / 128;
+    const double est_small = 0.54 * (double)((((M + 127) / 128) * cols + cus - 1) / cus);
+    const double est_big = 0.75 * (double)((((M + 255) / 256) * cols + cus - 1) / cus);
+    const double est_gemm = (est_small < est_big ? est_small : est_big) * (double)(N / 64 + 3) + 4.0;
+    const SplitPlan plan = plan_split(M, K, (int)(N / 64), workspace ? ws_bytes : 0, 0.75);
+    if (plan.splits >= 2 && plan.est_us < est_gemm) {
+        p.partial = (float *)workspace;
+        p.steps_per_split = plan.steps_per_split;
+        rc = plan.big ? launch_gemm<MODE_W4_DX, 256, 128, 2, 2>(p, (hipStream_t)stream, who)
+                      : launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
+        return rc ? rc : launch_split_reduce(p, plan.splits, (hipStream_t)stream, who);
     }
-    if (small_tiles(p)) return launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
+    if (est_small < est_big) return launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
     return launch_gemm<MODE_W4_DX, 256, 128, 2, 2>(p, (hipStream_t)stream, who);
 }
 
