@@ -77,8 +77,8 @@ WORKSPACE_MAX_BYTES = 64 << 20
 
 def _workspace(t, rows, cols):
     """(pointer, bytes) of a scratch buffer for a rows x cols fp32 result cut into up to 8 slices, or
-    (None, 0) when the problem is not one the split reduction is meant for (more than 1024 rows)."""
-    if rows > 1024:
+    (None, 0) when the problem is not one the split reduction is meant for (more than 2048 rows)."""
+    if rows > 2048:
         return None, 0
     need = min(8 * rows * cols * 4, WORKSPACE_MAX_BYTES)
     key = (t.device.index, _stream(t))
