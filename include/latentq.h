@@ -108,6 +108,20 @@ int lq_a16w4_fwd_ws(const void *x, const void *codes, const void *scales, const 
 int lq_a16w4_dx_ws(const void *dy, const void *codes, const void *scales, const void *zeros, void *dx, int64_t M,
                    int64_t N, int64_t K, int group, void *workspace, int64_t workspace_bytes, void *stream);
 
+/* Which kernel lq_a16w4_fwd(_ws) (backward = 0) or lq_a16w4_dx(_ws) (backward = 1) would run for a
+ * shape and a workspace size, and how it would cut the reduction; launches nothing. *kernel is
+ * one of LQ_PLAN_*; *splits > 1 means a split reduction of *steps_per_split 64-deep steps per slice
+ * followed by the reduce kernel. compute_units <= 0 asks the current device. The choice follows a
+ * rough cost model of measured per-step times (see lq_gemm.hip); it is exposed so that callers and
+ * tests can see it. No counterpart in the reference. */
+#define LQ_PLAN_GEMV 0         /* M <= 16: one GEMV launch */
+#define LQ_PLAN_GEMV_CHUNKS 1  /* 17..128 tokens: GEMV launches of 16 tokens each */
+#define LQ_PLAN_DIRECT 2       /* weights-direct forward kernel, 128 x 256 tiles */
+#define LQ_PLAN_STAGED_128 3   /* staged kernel, 128 x 128 tiles */
+#define LQ_PLAN_STAGED_256 4   /* staged kernel, 256 x 128 tiles */
+int lq_a16w4_plan(int backward, int64_t M, int64_t N, int64_t K, int64_t workspace_bytes, int compute_units,
+                  int *kernel, int *splits, int *steps_per_split);
+
 /* Dequantise the whole matrix to bf16[N,K] with the reference arithmetic
  * (DeQfunc_4bit_g, utils/quant.py:66-72). Used for the dW-side consumers and
  * for checks; not on the forward/backward GEMM path. */

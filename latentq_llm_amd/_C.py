@@ -24,6 +24,7 @@ SIGNATURES = {
     "lq_a16w4_fwd_ws": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp],
     "lq_a16w4_dx": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
     "lq_a16w4_dx_ws": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp],
+    "lq_a16w4_plan": [_i32, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp],
     "lq_a16w4_dequant": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp],
     "lq_a8w8_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "lq_act_quant_i8": [_vp, _vp, _vp, _i64, _vp],

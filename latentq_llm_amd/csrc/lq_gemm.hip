@@ -641,10 +641,9 @@ struct SplitPlan {
     double est_us = 1e30;
 };
 
-static SplitPlan plan_split(long long M, long long C, int total_steps, size_t ws_bytes, double pace_big) {
+static SplitPlan plan_split(long long M, long long C, int total_steps, size_t ws_bytes, double pace_big, long long cus) {
     SplitPlan best;
     if (!ws_bytes) return best;
-    const long long cus = lq_device_cu_count();
     const long long fit = (long long)(ws_bytes / ((size_t)M * C * 4));
     for (int big = 0; big < 2; ++big) {
         const long long tiles = ((M + (big ? 255 : 127)) / (big ? 256 : 128)) * ((C + 127) / 128);
@@ -667,6 +666,77 @@ static SplitPlan plan_split(long long M, long long C, int total_steps, size_t ws
     return best;
 }
 
+// Which kernel runs a product, and how its reduction is cut (the values of LQ_PLAN_* in latentq.h).
+struct W4Plan {
+    int kernel = LQ_PLAN_STAGED_128;
+    int splits = 1, steps_per_split = 0;
+};
+
+// Forward pass, M > 16. Rough time per 64-deep step of the three kernels without a split
+// (microseconds, measured): the weights-direct kernel (128 x 256 tiles) takes ~0.86 with one
+// workgroup on a compute unit and ~1.45 for two sharing it; the staged kernel ~0.56 per round of
+// 128 x 128 tiles and ~0.88 per round of 256 x 128 tiles (one workgroup per unit and round). The
+// weights-direct kernel loads scales and zeros four groups at a time: rows must be 4-byte aligned,
+// i.e. the number of groups per row even.
+static W4Plan plan_fwd(long long M, long long N, long long K, size_t ws_bytes, long long cus) {
+    W4Plan out;
+    const long long wg_direct = lq_gemm_fwd_direct_workgroups((int)M, (int)N);
+    const long long rem = wg_direct % (2 * cus);
+    const double est_direct = (K / LQ_GROUP) % 2 != 0 ? 1e30
+                              : 1.45 * (double)(wg_direct / (2 * cus)) + (rem == 0 ? 0.0 : rem <= cus ? 0.86 : 1.45);
+    const long long cols = (N + 127) / 128;
+    const double est_small = 0.56 * (double)((((M + 127) / 128) * cols + cus - 1) / cus);
+    const double est_big = 0.88 * (double)((((M + 255) / 256) * cols + cus - 1) / cus);
+    double step_us = est_direct;
+    out.kernel = LQ_PLAN_DIRECT;
+    if (est_small < step_us) { step_us = est_small; out.kernel = LQ_PLAN_STAGED_128; }
+    if (est_big < step_us) { step_us = est_big; out.kernel = LQ_PLAN_STAGED_256; }
+    double est_gemm = step_us * (double)(K / 64 + 3) + 4.0;
+    const SplitPlan sp = plan_split(M, N, (int)(K / 64), ws_bytes, 0.88, cus);
+    if (sp.splits >= 2 && sp.est_us < est_gemm) {
+        out.kernel = sp.big ? LQ_PLAN_STAGED_256 : LQ_PLAN_STAGED_128;
+        out.splits = sp.splits;
+        out.steps_per_split = sp.steps_per_split;
+        est_gemm = sp.est_us;
+    }
+    if (M <= 128) {
+        // A few more tokens than one GEMV takes: the GEMM's 128-row tiles would be mostly padding and
+        // its grid (N/128 workgroups, each walking all of K) fills a fraction of the device, so
+        // chunks of 16 tokens through the GEMV can be faster: the first streams the weights from
+        // HBM at near memory speed, the others find them in the last-level cache. Rough costs in
+        // microseconds: a GEMV chunk takes its bytes at ~1.8 TB/s the first time (at least 6) and
+        // ~2.3 TB/s after (at least 5; measured).
+        const long long chunks = (M + 15) / 16;
+        const double bytes = (double)(N * K / 2 + N * (K / LQ_GROUP) * 4);
+        const double first_us = bytes / 1.8e6 > 6.0 ? bytes / 1.8e6 : 6.0;
+        const double next_us = bytes / 2.3e6 > 5.0 ? bytes / 2.3e6 : 5.0;
+        if (first_us + (chunks - 1) * next_us < est_gemm) {
+            out.kernel = LQ_PLAN_GEMV_CHUNKS;
+            out.splits = 1;
+            out.steps_per_split = 0;
+        }
+    }
+    return out;
+}
+
+// dX: rounds of one workgroup per compute unit at ~0.54 us per 64-deep step for 128 x 128 tiles,
+// ~0.75 for 256 x 128 (the comparison small_tiles() makes for the int8 path), or a split reduction.
+static W4Plan plan_dx(long long M, long long N, long long K, size_t ws_bytes, long long cus) {
+    W4Plan out;
+    const long long cols = (K + 127) / 128;
+    const double est_small = 0.54 * (double)((((M + 127) / 128) * cols + cus - 1) / cus);
+    const double est_big = 0.75 * (double)((((M + 255) / 256) * cols + cus - 1) / cus);
+    out.kernel = est_small < est_big ? LQ_PLAN_STAGED_128 : LQ_PLAN_STAGED_256;
+    const double est_gemm = (est_small < est_big ? est_small : est_big) * (double)(N / 64 + 3) + 4.0;
+    const SplitPlan sp = plan_split(M, K, (int)(N / 64), ws_bytes, 0.75, cus);
+    if (sp.splits >= 2 && sp.est_us < est_gemm) {
+        out.kernel = sp.big ? LQ_PLAN_STAGED_256 : LQ_PLAN_STAGED_128;
+        out.splits = sp.splits;
+        out.steps_per_split = sp.steps_per_split;
+    }
+    return out;
+}
+
 static int launch_split_reduce(const GemmParams &p, int splits, hipStream_t st, const char *who) {
     const long long MC = (long long)p.M * p.C;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((MC / 8 + 255) / 256)), dim3(256), 0, st, p.partial, p.bias,
@@ -683,61 +753,31 @@ static int a16w4_fwd_impl(const char *who, const void *x, const void *codes, con
     LQ_REQUIRE(!workspace || lq_aligned(workspace, 16), "%s: the workspace must be 16-byte aligned", who);
     if (M <= 16)
         return lq_gemv_a16w4_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
-    // Rough time per 64-deep step of the three forward kernels without a split (microseconds,
-    // measured): the weights-direct kernel (128 x 256 tiles) takes ~0.86 with one workgroup on a
-    // compute unit and ~1.45 for two sharing it; the staged kernel ~0.56 per round of 128 x 128
-    // tiles and ~0.88 per round of 256 x 128 tiles (one workgroup per unit and round). The
-    // weights-direct kernel loads scales and zeros four groups at a time: rows must be 4-byte aligned.
-    const long long cus = lq_device_cu_count();
-    const long long wg_direct = lq_gemm_fwd_direct_workgroups((int)M, (int)N);
-    const long long rem = wg_direct % (2 * cus);
-    const double est_direct = (K / LQ_GROUP) % 2 != 0 ? 1e30
-                              : 1.45 * (double)(wg_direct / (2 * cus)) + (rem == 0 ? 0.0 : rem <= cus ? 0.86 : 1.45);
-    const long long cols = (N + 127) / 128;
-    const double est_small = 0.56 * (double)((((M + 127) / 128) * cols + cus - 1) / cus);
-    const double est_big = 0.88 * (double)((((M + 255) / 256) * cols + cus - 1) / cus);
-    const double step_us = est_direct < est_small ? (est_direct < est_big ? est_direct : est_big)
-                                                  : (est_small < est_big ? est_small : est_big);
-    const double est_gemm = step_us * (double)(K / 64 + 3) + 4.0;
-    const SplitPlan plan = plan_split(M, N, (int)(K / 64), workspace ? ws_bytes : 0, 0.88);
-    if (M <= 128) {
-        // A few more tokens than one GEMV takes: the GEMM's 128-row tiles would be mostly padding and
-        // its grid (N/128 workgroups, each walking all of K) fills a fraction of the device, so
-        // chunks of 16 tokens through the GEMV can be faster: the first streams the weights from
-        // HBM at near memory speed, the others find them in the last-level cache. Rough costs in
-        // microseconds: a GEMV chunk takes its bytes at ~1.8 TB/s the first time (at least 6) and
-        // ~2.3 TB/s after (at least 5; measured).
+    const W4Plan plan = plan_fwd(M, N, K, workspace ? ws_bytes : 0, lq_device_cu_count());
+    if (plan.kernel == LQ_PLAN_GEMV_CHUNKS) {
         const int chunks = (int)((M + 15) / 16);
-        const double bytes = (double)(N * K / 2 + N * (K / LQ_GROUP) * 4);
-        const double first_us = bytes / 1.8e6 > 6.0 ? bytes / 1.8e6 : 6.0;
-        const double next_us = bytes / 2.3e6 > 5.0 ? bytes / 2.3e6 : 5.0;
-        const double est_gemv = first_us + (chunks - 1) * next_us;
-        if (est_gemv < est_gemm && est_gemv < plan.est_us) {
-            for (int c = 0; c < chunks; ++c) {
-                const int rows = (int)(M - 16 * c < 16 ? M - 16 * c : 16);
-                rc = lq_gemv_a16w4_launch((const unsigned short *)x + (long long)c * 16 * K, codes, scales, zeros,
-                                          bias_or_null, (unsigned short *)y + (long long)c * 16 * N, rows, (int)N, (int)K,
-                                          (hipStream_t)stream);
-                if (rc) return rc;
-            }
-            return LQ_OK;
+        for (int c = 0; c < chunks; ++c) {
+            const int rows = (int)(M - 16 * c < 16 ? M - 16 * c : 16);
+            rc = lq_gemv_a16w4_launch((const unsigned short *)x + (long long)c * 16 * K, codes, scales, zeros, bias_or_null,
+                                      (unsigned short *)y + (long long)c * 16 * N, rows, (int)N, (int)K, (hipStream_t)stream);
+            if (rc) return rc;
         }
+        return LQ_OK;
     }
+    if (plan.kernel == LQ_PLAN_DIRECT)
+        return lq_gemm_fwd_direct_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
     GemmParams p = {};
     p.a = x; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.bias = (const unsigned short *)bias_or_null; p.c = y;
     p.M = (int)M; p.C = (int)N; p.R = (int)K; p.Kw = (int)K;
-    if (plan.splits >= 2 && plan.est_us < est_gemm) {
+    if (plan.splits >= 2) {
         p.partial = (float *)workspace;
         p.steps_per_split = plan.steps_per_split;
-        rc = plan.big ? launch_gemm<MODE_W4_FWD, 256, 128, 2, 2>(p, (hipStream_t)stream, who)
-                      : launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
-        return rc ? rc : launch_split_reduce(p, plan.splits, (hipStream_t)stream, who);
     }
-    if (est_direct <= est_small && est_direct <= est_big)
-        return lq_gemm_fwd_direct_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
-    if (est_small <= est_big) return launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
-    return launch_gemm<MODE_W4_FWD, 256, 128, 2, 2>(p, (hipStream_t)stream, who);
+    rc = plan.kernel == LQ_PLAN_STAGED_256 ? launch_gemm<MODE_W4_FWD, 256, 128, 2, 2>(p, (hipStream_t)stream, who)
+                                           : launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
+    if (rc || plan.splits < 2) return rc;
+    return launch_split_reduce(p, plan.splits, (hipStream_t)stream, who);
 }
 
 extern "C" int lq_a16w4_fwd(const void *x, const void *codes, const void *scales, const void *zeros,
@@ -764,23 +804,32 @@ static int a16w4_dx_impl(const char *who, const void *dy, const void *codes, con
     p.a = dy; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.c = dx;
     p.M = (int)M; p.C = (int)K; p.R = (int)N; p.Kw = (int)K;
-    // without a split: rounds of one workgroup per compute unit at ~0.54 us per 64-deep step for
-    // 128 x 128 tiles, ~0.75 for 256 x 128 (the comparison small_tiles() makes for the int8 path)
-    const long long cus = lq_device_cu_count();
-    const long long cols = (K + 127) / 128;
-    const double est_small = 0.54 * (double)((((M + 127) / 128) * cols + cus - 1) / cus);
-    const double est_big = 0.75 * (double)((((M + 255) / 256) * cols + cus - 1) / cus);
-    const double est_gemm = (est_small < est_big ? est_small : est_big) * (double)(N / 64 + 3) + 4.0;
-    const SplitPlan plan = plan_split(M, K, (int)(N / 64), workspace ? ws_bytes : 0, 0.75);
-    if (plan.splits >= 2 && plan.est_us < est_gemm) {
+    const W4Plan plan = plan_dx(M, N, K, workspace ? ws_bytes : 0, lq_device_cu_count());
+    if (plan.splits >= 2) {
         p.partial = (float *)workspace;
         p.steps_per_split = plan.steps_per_split;
-        rc = plan.big ? launch_gemm<MODE_W4_DX, 256, 128, 2, 2>(p, (hipStream_t)stream, who)
-                      : launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
-        return rc ? rc : launch_split_reduce(p, plan.splits, (hipStream_t)stream, who);
     }
-    if (est_small < est_big) return launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
-    return launch_gemm<MODE_W4_DX, 256, 128, 2, 2>(p, (hipStream_t)stream, who);
+    rc = plan.kernel == LQ_PLAN_STAGED_256 ? launch_gemm<MODE_W4_DX, 256, 128, 2, 2>(p, (hipStream_t)stream, who)
+                                           : launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
+    if (rc || plan.splits < 2) return rc;
+    return launch_split_reduce(p, plan.splits, (hipStream_t)stream, who);
+}
+
+// The plan the two entry points above would follow, without launching anything.
+extern "C" int lq_a16w4_plan(int backward, int64_t M, int64_t N, int64_t K, int64_t workspace_bytes, int compute_units,
+                             int *kernel, int *splits, int *steps_per_split) {
+    LQ_REQUIRE(kernel && splits && steps_per_split, "lq_a16w4_plan: null pointer argument");
+    LQ_REQUIRE(M > 0 && N > 0 && K > 0 && K % LQ_GROUP == 0 && M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31),
+               "lq_a16w4_plan: need positive M, N, K with K a multiple of %d", LQ_GROUP);
+    LQ_REQUIRE(backward ? N % 64 == 0 : N % 16 == 0, "lq_a16w4_plan: N=%lld must be a multiple of %d", (long long)N,
+               backward ? 64 : 16);
+    const long long cus = compute_units > 0 ? compute_units : lq_device_cu_count();
+    const size_t ws = workspace_bytes > 0 ? (size_t)workspace_bytes : 0;
+    W4Plan plan;
+    if (!backward && M <= 16) plan.kernel = LQ_PLAN_GEMV;
+    else plan = backward ? plan_dx(M, N, K, ws, cus) : plan_fwd(M, N, K, ws, cus);
+    *kernel = plan.kernel; *splits = plan.splits; *steps_per_split = plan.steps_per_split;
+    return LQ_OK;
 }
 
 extern "C" int lq_a16w4_dx(const void *dy, const void *codes, const void *scales, const void *zeros, void *dx,

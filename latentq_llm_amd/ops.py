@@ -143,6 +143,21 @@ def a16w4_dx(dy, codes, scales, zeros, shape, out=None):
     return dx
 
 
+PLAN_KERNELS = {0: "gemv", 1: "gemv_chunks", 2: "direct_128x256", 3: "staged_128x128", 4: "staged_256x128"}
+
+
+def a16w4_plan(M: int, shape, backward: bool = False, workspace_bytes: int = WORKSPACE_MAX_BYTES, compute_units: int = 0):
+    """(kernel name, splits, steps per slice) the forward / dX entry points would use for M tokens on an
+    [N, K] matrix; compute_units = 0 asks the current device. Launches nothing (works without a GPU when
+    compute_units is given)."""
+    import ctypes
+    N, K = shape
+    k, sp, per = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    _C.call("lq_a16w4_plan", int(bool(backward)), M, N, K, workspace_bytes, compute_units, ctypes.addressof(k),
+            ctypes.addressof(sp), ctypes.addressof(per))
+    return PLAN_KERNELS[k.value], sp.value, per.value
+
+
 def a16w4_dequant(codes, scales, zeros, shape):
     N, K = shape
     _codes_ok(codes, N, K)

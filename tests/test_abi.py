@@ -94,3 +94,48 @@ def test_product_does_not_import_the_oracle():
                 src = open(os.path.join(dirpath, f)).read()
                 assert not re.search(r"^\s*(from|import)\s+oracle\b", src, flags=re.M), f
                 assert "lq_oracle" not in src, f
+
+
+def test_dispatch_plan_host_logic(hip_lib):
+    """The kernel choice of the A16W4 entry points is host arithmetic over (M, N, K, workspace, CUs):
+    checked here for a 256-CU device without launching anything."""
+    from latentq_llm_amd import ops
+    ws = 64 << 20
+
+    def plan(M, N, K, backward=False, workspace=ws):
+        return ops.a16w4_plan(M, (N, K), backward=backward, workspace_bytes=workspace, compute_units=256)
+
+    # decode sizes
+    assert plan(1, 11008, 4096) == ("gemv", 1, 0) and plan(16, 4096, 11008) == ("gemv", 1, 0)
+    assert plan(17, 11008, 4096)[0] == "gemv_chunks"
+    # 2048 tokens on the 7B MLP matrices: weights-direct forward, large staged tiles backward, no split
+    assert plan(2048, 11008, 4096) == ("direct_128x256", 1, 0)
+    assert plan(2048, 4096, 11008) == ("direct_128x256", 1, 0)
+    assert plan(2048, 11008, 4096, backward=True) == ("staged_256x128", 1, 0)
+    assert plan(2048, 4096, 11008, backward=True) == ("staged_256x128", 1, 0)
+    # an odd number of groups per row rules the weights-direct kernel out
+    assert plan(2048, 11008, 4096 + 128)[0] != "direct_128x256"
+    # one round of small tiles beats everything else when it fits
+    assert plan(256, 11008, 4096) == ("staged_128x128", 1, 0)
+    # skinny grids: split reduction, slices of an even number of steps >= 8 that cover the reduction
+    for M, N, K, back in [(128, 11008, 4096, True), (512, 11008, 4096, True), (1024, 11008, 4096, True),
+                          (128, 4096, 11008, False), (512, 4096, 11008, False), (200, 2048, 1280, False)]:
+        kern, splits, per = plan(M, N, K, back)
+        steps = (N if back else K) // 64
+        assert kern.startswith("staged") and 2 <= splits <= 8, (M, N, K, back, kern, splits)
+        assert per % 2 == 0 and per >= 8 and (splits - 1) * per < steps <= splits * per
+        rows = 256 if kern == "staged_256x128" else 128
+        cols = K if back else N
+        assert -(-M // rows) * -(-cols // 128) * splits <= 256, "at most one workgroup per compute unit"
+        # the partial tiles fit the workspace; without one there is no split
+        assert splits * M * cols * 4 <= ws
+        assert plan(M, N, K, back, workspace=0)[1] == 1
+    # a workspace that holds two slices caps the split at two
+    M, N, K = 128, 11008, 4096
+    assert plan(M, N, K, True, workspace=2 * M * K * 4)[1] == 2
+    # bad arguments
+    from latentq_llm_amd._C import LatentQError
+    with pytest.raises(LatentQError, match="multiple of 64"):
+        plan(128, 11008 + 16, 4096, backward=True)
+    with pytest.raises(LatentQError, match="multiple of 128"):
+        plan(128, 11008, 4096 + 64)
