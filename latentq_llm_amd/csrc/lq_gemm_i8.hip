@@ -1,15 +1,17 @@
-// A8W8 GEMM with 256 x 256 tiles for gfx950:
+// A8W8 GEMM for gfx950, both operands through LDS-direct loads:
 //   Y[M,N] = bf16(((int32) X8[M,K] . W8[N,K]^T) * sx[m] * sw[n] (+ bias)), optional int32 accumulators.
 //
 // int8 operands need no dequantisation, so both operands go from global memory into LDS with
 // LDS-direct loads (no registers, no vector-ALU work) and what bounds a tile scheme is the traffic
 // between L2 and the compute units: per unit of MFMA work a 128 x 256 tile moves 1.5 times the
 // bytes of a 256 x 256 tile, and at int8 rates (twice the reduction depth per MFMA cycle of bf16)
-// that traffic, not the matrix core, set the pace of the 128 x 256 kernel.
+// that traffic, not the matrix core, set the pace of a 128 x 256 kernel.
 //
-// Workgroup: 512 threads = 8 waves in a 2 (m) x 4 (n) grid; a wave owns 128 x 64 outputs (4 x 2
-// MFMA 32x32x32 tiles, 128 accumulator registers), two waves per SIMD. One workgroup per CU: two
-// LDS stages of 64 KB (256 rows of A and 256 rows of B, 128 bytes = 128 k each).
+// Main instance: 256 x 256 tile, 512 threads = 8 waves in a 2 (m) x 4 (n) grid; a wave owns
+// 128 x 64 outputs (4 x 2 MFMA 32x32x32 tiles, 128 accumulator registers), two waves per SIMD. One
+// workgroup per CU: two LDS stages of 64 KB (256 rows of A and 256 rows of B, 128 bytes = 128 k
+// each). Second instance for small outputs: 128 x 128 tile, 4 waves (2 x 2, 64 x 64 each), two
+// stages of 32 KB, two workgroups per CU.
 //
 // Reduction step = 128 k in four slices of 32. Lane l: r = l % 32, h = l / 32. In slice t the
 // lane's operand of row r is chunk 4h + t (16 bytes) of the row's 128 bytes, for A and B alike
@@ -49,13 +51,20 @@ typedef __attribute__((address_space(3))) void lds_void;
 template <int I>
 using ic = std::integral_constant<int, I>;
 
-constexpr int BM = 256, BN = 256;
-constexpr int ROWB = 128;                   // bytes (= k) per tile row and step
-constexpr int A_STAGE = BM * ROWB;          // 32 KB
-constexpr int STAGE = (BM + BN) * ROWB;     // 64 KB: A rows, then B rows
-constexpr int NT = 512;
+constexpr int ROWB = 128;  // bytes (= k) per tile row and step
 
-__global__ __launch_bounds__(NT) void gemm_i8_256_kernel(I8Params p) {
+// BM x BN tile, WM x WN waves. Two instances: 256 x 256 with 2 x 4 waves (one workgroup per CU) and
+// 128 x 128 with 2 x 2 waves (64 KB of LDS: two per CU) for outputs too small to fill the device
+// with the large tile. Both fill a stage with 4 + 4 loads per thread.
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) {
+    constexpr int NT = 64 * WM * WN;
+    constexpr int A_STAGE = BM * ROWB;       // A rows, then B rows
+    constexpr int STAGE = (BM + BN) * ROWB;
+    constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
+    constexpr int FM = TM / 32, FN = TN / 32;
+    static_assert(BM * 8 == 4 * NT && BN * 8 == 4 * NT, "a stage is 4 + 4 loads per thread");
+    static_assert(FN == 2, "the epilogue regroups 64 columns per wave");
     __shared__ __attribute__((aligned(16))) unsigned char lds0[STAGE];
     __shared__ __attribute__((aligned(16))) unsigned char lds1[STAGE];
     auto stage = [&](auto i) -> unsigned char * {
@@ -66,7 +75,7 @@ __global__ __launch_bounds__(NT) void gemm_i8_256_kernel(I8Params p) {
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
     const int r = lane & 31, h = lane >> 5;
-    const int wm = wave & 1, wn = wave >> 1;
+    const int wm = wave % WM, wn = wave / WM;
 
     // Workgroup ids are dealt round-robin over the 8 XCDs (id % 8): give each XCD a contiguous
     // range of the tile sequence, ordered in bands of GN tile columns walked row by row, so the
@@ -91,7 +100,7 @@ __global__ __launch_bounds__(NT) void gemm_i8_256_kernel(I8Params p) {
     unsigned a_off[4], b_off[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int row = i * 64 + (int)(threadIdx.x >> 3);
+        const int row = i * (NT / 8) + (int)(threadIdx.x >> 3);
         const int pos = threadIdx.x & 7;
         const int chunk = pos ^ ((row >> 1) & 7);
         int ga = m0 + row, gb = c0 + row;
@@ -116,23 +125,23 @@ __global__ __launch_bounds__(NT) void gemm_i8_256_kernel(I8Params p) {
     int frag[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) frag[t] = r * ROWB + (((4 * h + t) ^ ((r >> 1) & 7)) << 4);
-    const int a_rows = wm * 128 * ROWB, b_rows = A_STAGE + wn * 64 * ROWB;
+    const int a_rows = wm * TM * ROWB, b_rows = A_STAGE + wn * TN * ROWB;
     auto read_frags = [&](const unsigned char *st, int t, u32x4_t *af, u32x4_t *bf) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) af[j] = *reinterpret_cast<const u32x4_t *>(st + a_rows + j * 32 * ROWB + frag[t]);
+        for (int j = 0; j < FM; ++j) af[j] = *reinterpret_cast<const u32x4_t *>(st + a_rows + j * 32 * ROWB + frag[t]);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) bf[i] = *reinterpret_cast<const u32x4_t *>(st + b_rows + i * 32 * ROWB + frag[t]);
+        for (int i = 0; i < FN; ++i) bf[i] = *reinterpret_cast<const u32x4_t *>(st + b_rows + i * 32 * ROWB + frag[t]);
     };
 
-    i32x16_t acc[2][4];
+    i32x16_t acc[FN][FM];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < FN; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < FM; ++j)
 #pragma unroll
             for (int q = 0; q < 16; ++q) acc[i][j][q] = 0;
 
-    u32x4_t af[2][4], bf[2][2];
+    u32x4_t af[2][FM], bf[2][FN];
     // Step kt on stage S: the operands of its first slice are already in af[0] / bf[0].
     auto step = [&](int kt, auto si) {
         constexpr int S = decltype(si)::value;
@@ -156,9 +165,9 @@ __global__ __launch_bounds__(NT) void gemm_i8_256_kernel(I8Params p) {
             // the reads and loads above go out before this slice's MFMAs, which cover their latency
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < FN; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                for (int j = 0; j < FM; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf[t & 1][i]),
                                                                      __builtin_bit_cast(i32x4_t, af[t & 1][j]), acc[i][j], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
@@ -182,7 +191,7 @@ __global__ __launch_bounds__(NT) void gemm_i8_256_kernel(I8Params p) {
     // the clamped prefetches of the last steps are still writing LDS: drain them
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    // ---- epilogue: acc[i][j][q]: column c0 + 64*wn + 32i + 8*(q/4) + 4h + q%4, row m0 + 128*wm + 32j + r.
+    // ---- epilogue: acc[i][j][q]: column c0 + 64*wn + 32i + 8*(q/4) + 4h + q%4, row m0 + TM*wm + 32j + r.
     // Every wave passes its block through a private LDS area, 32 rows (one j) at a time, and stores
     // 16 bytes per lane with 8 lanes on the 128 contiguous bytes of a row: full cache lines.
     __syncthreads();
@@ -191,9 +200,9 @@ __global__ __launch_bounds__(NT) void gemm_i8_256_kernel(I8Params p) {
     const int ep_row = lane >> 3, ep_chunk = lane & 7;
     const int cw0 = c0 + wn * 64;
     const int c_lane = cw0 + ep_chunk * 8;  // first of the 8 columns this lane stores
-    float bias_v[2][4][4], sw_v[2][4][4];
+    float bias_v[FN][4][4], sw_v[FN][4][4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < FN; ++i)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int c = cw0 + i * 32 + 8 * q + 4 * h;
@@ -205,12 +214,12 @@ __global__ __launch_bounds__(NT) void gemm_i8_256_kernel(I8Params p) {
             }
         }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int mrow0 = m0 + wm * 128 + j * 32;
+    for (int j = 0; j < FM; ++j) {
+        const int mrow0 = m0 + wm * TM + j * 32;
         const int m = mrow0 + r;
         const float sxm = m < p.M ? p.sx[m] : 0.0f;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < FN; ++i) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 float v[4];
@@ -241,21 +250,23 @@ __global__ __launch_bounds__(NT) void gemm_i8_256_kernel(I8Params p) {
 }  // namespace
 
 // Number of 256 x 256 tiles of an [M, N] output.
-long long lq_gemm_i8_256_workgroups(int M, int N) { return (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN); }
+long long lq_gemm_i8_256_workgroups(int M, int N) { return (long long)((M + 255) / 256) * ((N + 255) / 256); }
 
 // Called by lq_a8w8_fwd (lq_gemm.hip) after argument validation: K % 128 == 0, N % 16 == 0.
-int lq_gemm_i8_256_launch(const void *x8, const void *w8, const float *sx, const float *sw, const void *bias, void *y,
-                          int *acc_or_null, int M, int N, int K, hipStream_t st) {
+// tile = 256 or 128 (square tiles).
+int lq_gemm_i8_tile_launch(const void *x8, const void *w8, const float *sx, const float *sw, const void *bias, void *y,
+                           int *acc_or_null, int M, int N, int K, int tile, hipStream_t st) {
     I8Params p = {};
     p.x = (const unsigned char *)x8; p.w = (const unsigned char *)w8; p.sx = sx; p.sw = sw;
     p.bias = (const unsigned short *)bias; p.y = (unsigned short *)y; p.acc_out = acc_or_null;
     p.M = M; p.N = N; p.K = K;
-    p.tiles_m = (M + BM - 1) / BM;
-    p.tiles_n = (N + BN - 1) / BN;
+    p.tiles_m = (M + tile - 1) / tile;
+    p.tiles_n = (N + tile - 1) / tile;
     const long long nwg = (long long)p.tiles_m * p.tiles_n;
     if (nwg > 0x7FFFFFFFll) return lq_fail(LQ_ERR_BAD_ARG, "lq_a8w8_fwd: problem too large");
-    // the 32-bit lane offsets of the loads span 256 rows
-    if ((long long)BN * K >= (1ll << 32)) return lq_fail(LQ_ERR_BAD_ARG, "lq_a8w8_fwd: K too large");
-    hipLaunchKernelGGL(gemm_i8_256_kernel, dim3((unsigned)nwg), dim3(NT), 0, st, p);
+    // the 32-bit lane offsets of the loads span up to 256 rows
+    if (256ll * K >= (1ll << 32)) return lq_fail(LQ_ERR_BAD_ARG, "lq_a8w8_fwd: K too large");
+    if (tile == 256) hipLaunchKernelGGL((gemm_i8_tile_kernel<256, 256, 2, 4>), dim3((unsigned)nwg), dim3(512), 0, st, p);
+    else hipLaunchKernelGGL((gemm_i8_tile_kernel<128, 128, 2, 2>), dim3((unsigned)nwg), dim3(256), 0, st, p);
     return lq_check_launch("lq_a8w8_fwd");
 }
