@@ -115,6 +115,11 @@ template <int BS, bool LATENT>
 __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
     constexpr int W = BS / 8;  // threads per block of the moments
     __shared__ float red[4][2];
+    __shared__ float vtab[16];  // latent mode: dequantised values of the 16 residual nibbles
+    if constexpr (LATENT) {
+        lq_latent_fill_value_table(vtab, a.dequant_curve);
+        __syncthreads();
+    }
     const long long T = (long long)blockIdx.x * 256 + threadIdx.x;
     const bool live = T < a.n_threads;  // n is a multiple of BS: a block is all-live or all-dead
     const long long Tc = live ? T : 0;
@@ -153,8 +158,7 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
         d[k] = dk;
         const float ratio = mk / dk;
         if constexpr (LATENT) {
-            const int nib = (int)((rword >> (28 - 4 * k)) & 0xFu) - 8;
-            const float p = bf16r(lq_latent_value(lq_code(cword, k), nib, ws, wz, a.dequant_curve));
+            const float p = bf16r(lq_latent_value(lq_code(cword, k), vtab[(rword >> (28 - 4 * k)) & 0xFu], ws, wz));
             out[k] = bf16r(fmaf(a.neg_step, ratio, p));
         } else if (a.param) {
             const float p = (k & 1) ? lq_bf16_hi(p4[k >> 1]) : lq_bf16_lo(p4[k >> 1]);

@@ -25,6 +25,9 @@ __global__ __launch_bounds__(256) void latent_reconstruct_kernel(const u32x4_t *
                                                                  const u32x4_t *__restrict__ residual,
                                                                  u32x4_t *__restrict__ latent, long long n_chunks,
                                                                  CodecParams p) {
+    __shared__ float vtab[16];
+    lq_latent_fill_value_table(vtab, p);
+    __syncthreads();
     const long long L = (long long)blockIdx.x * 256 + threadIdx.x;
     if (L >= n_chunks) return;
     const u32x4_t cw = codes[L], rw = residual[L];
@@ -35,8 +38,7 @@ __global__ __launch_bounds__(256) void latent_reconstruct_kernel(const u32x4_t *
         float v[8];
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            const int nib = (int)((rw[i] >> (28 - 4 * k)) & 0xFu) - 8;
-            v[k] = lq_latent_value(lq_code(cw[i], k), nib, s, z, p);
+            v[k] = lq_latent_value(lq_code(cw[i], k), vtab[(rw[i] >> (28 - 4 * k)) & 0xFu], s, z);
         }
         latent[L * 4 + i] = u32x4_t{lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3]), lq_pack_bf16(v[4], v[5]),
                                     lq_pack_bf16(v[6], v[7])};

@@ -7,10 +7,18 @@
 
 __device__ __forceinline__ float lq_bf16r(float v) { return lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(v)); }
 
-// latent = bf16(bf16(bf16(value(nibble)) * s) + bf16(bf16(q - z) * s)); the caller applies the last rounding
-__device__ __forceinline__ float lq_latent_value(unsigned code, int nib, float s, float z, const CodecParams &pd) {
+// The dequantised value of a residual nibble depends on nothing but the nibble, so a workgroup keeps
+// the 16 values bf16(value(n - 8)) in LDS and an element costs one LDS read instead of the curve's
+// dozen selects and operations. Threads 0..15 fill the table; the caller synchronises before use.
+__device__ __forceinline__ void lq_latent_fill_value_table(float *tab, const CodecParams &pd) {
+    if (threadIdx.x < 16) tab[threadIdx.x] = lq_bf16r(value_3fold((int)threadIdx.x - 8, pd));
+}
+
+// latent = bf16(bf16(bf16(value(nibble)) * s) + bf16(bf16(q - z) * s)) with value_bf16 =
+// bf16(value(nibble)) from the table; the caller applies the last rounding
+__device__ __forceinline__ float lq_latent_value(unsigned code, float value_bf16, float s, float z) {
     const float wq = lq_bf16r(lq_bf16r((float)code - z) * s);
-    const float r = lq_bf16r(lq_bf16r(value_3fold(nib, pd)) * s);
+    const float r = lq_bf16r(value_bf16 * s);
     return r + wq;
 }
 
