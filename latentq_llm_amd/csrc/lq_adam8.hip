@@ -156,7 +156,20 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
         dk = bf16r(dk + a.eps);
         m[k] = mk;
         d[k] = dk;
-        const float ratio = mk / dk;
+        float ratio;
+        if (!LATENT && !a.param) {
+            // Only bf16(m / d) is stored here, and the quotient of two bf16 numbers never comes closer
+            // than 2^-17 (relative) to the midpoint of two bf16 values (256 m_a = (2j+1) m_b has no
+            // solution with 8-bit significands), so any fp32 quotient within a few ulps rounds to the
+            // same bf16 value as the correctly rounded one (every significand pair is checked by the
+            // CPU tests): reciprocal and product instead of the division sequence. Results outside
+            // [2^-100, 2^100] (bf16 subnormals, overflow, NaN; zero numerators excepted) take the division.
+            ratio = mk * __builtin_amdgcn_rcpf(dk);
+            const float ar = fabsf(ratio);
+            if (!(ar <= 0x1p100f && (ar >= 0x1p-100f || mk == 0.0f))) ratio = mk / dk;
+        } else {
+            ratio = mk / dk;
+        }
         if constexpr (LATENT) {
             const float p = bf16r(lq_latent_value(lq_code(cword, k), vtab[(rword >> (28 - 4 * k)) & 0xFu], ws, wz));
             out[k] = bf16r(fmaf(a.neg_step, ratio, p));

@@ -314,3 +314,18 @@ def test_two_step_reciprocal_division_equals_ieee_division():
     q1 = fma(fma(-q0, s, t), r, q0)
     q2 = fma(fma(-q1, s, t), r, q1)
     assert np.array_equal(q2.view(np.uint32), want.view(np.uint32))
+
+
+def test_quotient_of_bf16_rounds_the_same_within_three_ulps():
+    """a / b for bf16 a, b: all fp32 values within three ulps of the correctly rounded quotient round
+    to the same bf16 value (checked for every pair of significands; the exponents only shift the
+    result), so the fused Adam kernel may form bf16(m / d) from a reciprocal and a product."""
+    ma = np.arange(128, 256, dtype=np.float32)
+    a, b = np.meshgrid(ma, ma, indexing="ij")
+    q = (a / b).astype(np.float32).ravel()  # IEEE: correctly rounded, 2^-1 < q < 2
+    want = _bf16_rne_bits(q)
+    for d in (-3, -2, -1, 1, 2, 3):
+        near = (q.view(np.int32) + d).view(np.float32)
+        assert np.array_equal(_bf16_rne_bits(near), want), d
+    frac = q.view(np.uint32) & 0xFFFF
+    assert int(np.abs(frac.astype(np.int64) - 0x8000).min()) > 16  # distance to a tie, in fp32 ulps
