@@ -16,7 +16,7 @@
 // consumes 32 bytes of every row (chunks 2s and 2s+1), i.e. 4 steps per tile. Bank conflicts of
 // the 16-byte fragment reads (consecutive rows, same chunk) are avoided by XOR swizzles:
 //   * chunk c of A row r sits at position c ^ ((r >> 1) & 7);
-//   * chunk c of B row r sits at position c ^ ((r ^ (r >> 3)) & 7) (MODE_W4_DX: see swz_dx_piece).
+//   * chunk c of B row r sits at position c ^ ((r ^ (r >> 3)) & 7) (MODE_W4_DX: see dx_slot).
 //
 // The MFMA is issued with the weight fragment as the first operand and the activation
 // fragment as the second, so that D[i][j] has i = output column (n), j = row (m): a
@@ -76,13 +76,22 @@ template <int I>
 using ic = std::integral_constant<int, I>;
 
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
-// dX tile ([n][k], 256-byte rows of eight 32-byte pieces, each two 16-byte halves): with j = n & 3,
-// piece c of row n sits at c ^ (2j | (j & 1)) and its halves are swapped when j >= 2. The 16
-// lanes of a staging write (4 consecutive rows x 4 quarter rows) then fall on 16 different
-// 16-byte slots of the bank space, and a transposing read (rows n..n+3 at two adjacent pieces,
-// per 32 lanes) covers every bank once.
-__device__ __forceinline__ int swz_dx_piece(int row) { return ((row & 3) << 1) | (row & 1); }
-__device__ __forceinline__ int swz_dx_half(int row) { return (row >> 1) & 1; }
+// dX tile ([n][k], 256-byte rows of eight 32-byte pieces c32 = k / 16, each two 16-byte halves).
+// Byte offset within row n of half `half` of piece c32, with j = n & 3:
+//   piece = ((c32 >> 1) ^ j) | (((c32 & 1) ^ (j >> 1)) << 2),  half ^= j & 1.
+// Writes: a staging instruction puts lane (row, quarter q) on piece c32 = 2q + e with e and the half
+// fixed. LDS takes a 16-byte write instruction 8 lanes (2 rows x 4 quarters, 128 bytes) at a time
+// over 32 banks: their slots modulo 8 are 2 (q ^ j) + (half ^ (j & 1)), all different; the 16
+// lanes of 4 rows also fall on 16 different slots of 256 bytes. Reads: a transposing read covers,
+// per 32 lanes, rows n..n+3 at the two pieces (c, c + 1), c even: pieces (q ^ j) and (q ^ j) + 4
+// for j = 0..3, every bank once. (An earlier layout spread the quarters over pieces 2q ^ f(j): two
+// of the four quarters of a row then shared their slot modulo 8, and the counters showed one
+// bank-conflict cycle per write cycle.)
+__device__ __forceinline__ int dx_slot(int row, int c32, int half) {
+    const int j = row & 3;
+    const int piece = ((c32 >> 1) ^ j) | (((c32 & 1) ^ (j >> 1)) << 2);
+    return (piece << 5) | ((half ^ (j & 1)) << 4);
+}
 
 template <int MODE, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
@@ -260,8 +269,7 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
                     u32x4_t v = {lq_pack_bf16(f[0], f[1]), lq_pack_bf16(f[2], f[3]), lq_pack_bf16(f[4], f[5]),
                                  lq_pack_bf16(f[6], f[7])};
                     const int c32 = b_w0 * 2 + (w >> 1);  // 32-byte piece of the 256-byte row
-                    *reinterpret_cast<u32x4_t *>(lb + b_row * 256 + ((c32 ^ swz_dx_piece(b_row)) << 5) +
-                                                 (((w & 1) ^ swz_dx_half(b_row)) << 4)) = v;
+                    *reinterpret_cast<u32x4_t *>(lb + b_row * 256 + dx_slot(b_row, c32, w & 1)) = v;
                 }
             }
         };
@@ -358,8 +366,7 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
 #pragma unroll
         for (int i = 0; i < FN; ++i) {
             const int c32 = (wn * TN + i * 32) / 16 + colblk;
-            dx_off[i] = row_lane * 256 + ((c32 ^ swz_dx_piece(row_lane)) << 5) +
-                        ((((i16 & 3) >> 1) ^ swz_dx_half(row_lane)) << 4) + (i16 & 1) * 8;
+            dx_off[i] = row_lane * 256 + dx_slot(row_lane, c32, (i16 & 3) >> 1) + (i16 & 1) * 8;
         }
     }
     auto read_frags = [&](const unsigned char *la, const unsigned char *lb, int ks, u32x4_t *af, u32x4_t *bf) {
