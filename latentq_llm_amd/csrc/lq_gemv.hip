@@ -88,6 +88,11 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
     // then takes its groups from LDS
     constexpr int kQPieces = 2;  // 16-byte pieces per thread: up to 64*WAVES*2*16 bytes of scales + zeros
     const int q_bytes = 16 * NT * G * 2;
+    // LDS row pitch of the staged block: rows whose length is a multiple of 16 bytes get 16 bytes of
+    // padding (a 64-byte pitch would put the 16 rows a group is read from on 4 bank groups); other
+    // lengths keep the block as it is (its 16-byte pieces straddle rows)
+    const int q_row = G * 2, q_pitch = (q_row % 16 == 0) ? q_row + 16 : q_row;
+    const int q_lds = 16 * NT * q_pitch;  // bytes per array in LDS
     u32x4_t qstage[kQPieces];
     if constexpr (QS) {
         const unsigned char *sb = (const unsigned char *)(scales + (long long)blockIdx.x * (16 * NT) * G);
@@ -130,15 +135,19 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
 #pragma unroll
                 for (int i = 0; i < kQPieces; ++i) {
                     const int o = ((int)threadIdx.x + i * 64 * WAVES) * 16;
-                    if (o < 2 * q_bytes) *reinterpret_cast<u32x4_t *>(sq + o) = qstage[i];
+                    if (o < 2 * q_bytes) {
+                        const int oa = o < q_bytes ? o : o - q_bytes;
+                        const int dst = q_pitch == q_row ? oa : (oa / q_row) * q_pitch + oa % q_row;
+                        *reinterpret_cast<u32x4_t *>(sq + (o < q_bytes ? 0 : q_lds) + dst) = qstage[i];
+                    }
                 }
                 __syncthreads();
                 first = false;
             }
 #pragma unroll
             for (int j = 0; j < NT; ++j) {
-                const unsigned short *ls = reinterpret_cast<const unsigned short *>(sq) + (j * 16 + n) * G;
-                const unsigned short *lz = reinterpret_cast<const unsigned short *>(sq + q_bytes) + (j * 16 + n) * G;
+                const unsigned short *ls = reinterpret_cast<const unsigned short *>(sq + (j * 16 + n) * q_pitch);
+                const unsigned short *lz = reinterpret_cast<const unsigned short *>(sq + q_lds + (j * 16 + n) * q_pitch);
 #pragma unroll
                 for (int u = 0; u < kUnroll; ++u) {
                     const bool live = g0 + u < G;
@@ -261,7 +270,7 @@ void launch_one(const GemvArgs &a) {
     const bool qs = MP == 16 && (NT == 2 || batches > W) && lq_aligned(a.scales, 16) && lq_aligned(a.zeros, 16) &&
                     2 * q_bytes <= (size_t)64 * W * 2 * 16;
     if (qs)
-        hipLaunchKernelGGL((gemv_kernel<W, MP, NT, true>), dim3(a.N / (16 * NT)), dim3(64 * W), 2 * q_bytes, a.st,
+        hipLaunchKernelGGL((gemv_kernel<W, MP, NT, true>), dim3(a.N / (16 * NT)), dim3(64 * W), 2 * q_bytes + 2 * 16 * NT * 16, a.st,
                            (const unsigned short *)a.x, (const unsigned char *)a.codes, (const unsigned short *)a.scales,
                            (const unsigned short *)a.zeros, (const unsigned short *)a.bias, (unsigned short *)a.y, a.M, a.N, a.K);
     else
