@@ -106,6 +106,20 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
         }
     }
     bool first = true;
+    // every wave runs this exactly once: in its first batch, after that batch's loads are issued, or
+    // after the loop when it has no batch at all (the barrier inside needs all waves)
+    auto publish_q = [&]() {
+#pragma unroll
+        for (int i = 0; i < kQPieces; ++i) {
+            const int o = ((int)threadIdx.x + i * 64 * WAVES) * 16;
+            if (o < 2 * q_bytes) {
+                const int oa = o < q_bytes ? o : o - q_bytes;
+                const int dst = q_pitch == q_row ? oa : (oa / q_row) * q_pitch + oa % q_row;
+                *reinterpret_cast<u32x4_t *>(sq + (o < q_bytes ? 0 : q_lds) + dst) = qstage[i];
+            }
+        }
+        __syncthreads();
+    };
     for (int g0 = wave * kUnroll; g0 < G; g0 += WAVES * kUnroll) {
         const bool full = g0 + kUnroll <= G;  // a short tail batch re-reads the last group with zero scale
         // ---- activations: one LDS-direct load per token row (1 KB = this batch's 512 k), coalesced.
@@ -132,16 +146,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
             }
         if constexpr (QS) {
             if (first) {
-#pragma unroll
-                for (int i = 0; i < kQPieces; ++i) {
-                    const int o = ((int)threadIdx.x + i * 64 * WAVES) * 16;
-                    if (o < 2 * q_bytes) {
-                        const int oa = o < q_bytes ? o : o - q_bytes;
-                        const int dst = q_pitch == q_row ? oa : (oa / q_row) * q_pitch + oa % q_row;
-                        *reinterpret_cast<u32x4_t *>(sq + (o < q_bytes ? 0 : q_lds) + dst) = qstage[i];
-                    }
-                }
-                __syncthreads();
+                publish_q();
                 first = false;
             }
 #pragma unroll
@@ -228,6 +233,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
 
+    if constexpr (QS) {
+        if (first) publish_q();
+    }
 #pragma unroll
     for (int j = 0; j < NT; ++j)
 #pragma unroll

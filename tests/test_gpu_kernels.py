@@ -188,6 +188,14 @@ def test_a16w4_fwd_gemv(ops, co, M, N, K, bias):
     _fwd_case(ops, co, M, N, K, seed=M + N + K, with_bias=bias)
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 8192, 1536), (9, 8224, 1152), (16, 8192, 2560), (12, 512, 5120), (16, 8192, 640)])
+def test_a16w4_fwd_gemv_many_tokens_staged_scales(ops, co, M, N, K):
+    """5..16 tokens with the scales and zeros of a workgroup's rows staged through LDS: 32-row workgroups
+    on tall matrices (also with a wave that has no batch of its own: 3 and 5 batches on 4 waves), several
+    batches per wave on 8 waves, padded (K = 2560, 5120: 80- and 160-byte rows) and unpadded rows."""
+    _fwd_case(ops, co, M, N, K, seed=M + N + K, with_bias=(M % 2 == 0))
+
+
 def test_a16w4_fwd_identity_is_exact_dequant(ops, co):
     """X = identity: every output is a single dequantised weight, so the GEMM result must equal
     the reference dequantisation bit for bit (checks unpack + bf16 rounding through the kernel)."""
