@@ -1,0 +1,71 @@
+"""Seeded random-shape sweeps over the dispatch of the GEMM entry points (GEMV, chunked GEMV, split
+reduction with both tile heights, staged and weights-direct kernels, the int8 kernels): every shape
+is checked against an fp32 product of the dequantised matrix on the GPU (lq_a16w4_dequant is itself
+checked bit for bit against the CPU oracle elsewhere) and, for int8, against an exact integer product.
+A hang in any configuration shows as a time-out of the case that names the shape."""
+import random
+
+import pytest
+import torch
+
+from tests.util import make_w4
+
+pytestmark = pytest.mark.gpu
+
+TOL = 5e-3  # bf16 output rounding gives ~1.7e-3
+
+
+@pytest.fixture(scope="module")
+def ops(hip_lib):
+    assert torch.cuda.is_available()
+    from latentq_llm_amd import ops
+    return ops
+
+
+def _shapes(seed, n, token_counts, n_choices, k_max):
+    rng = random.Random(seed)
+    out = []
+    for _ in range(n):
+        M = rng.choice(token_counts)
+        N = rng.choice(n_choices) if rng.random() < 0.5 else 64 * rng.randint(1, 160)
+        K = 128 * rng.randint(1, k_max)
+        if N * K > 48e6:
+            K = 128 * max(1, int(48e6 // N) // 128)
+        out.append((M, N, K))
+    return out
+
+
+GEMM_SHAPES = _shapes(1, 40, [17, 33, 100, 128, 129, 250, 384, 511, 640, 777, 1024, 1500, 2050], [4096, 8192, 11008], 40)
+GEMV_SHAPES = _shapes(2, 40, list(range(1, 17)), [64, 512, 4096, 8192, 8224, 11008], 96)
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES + GEMV_SHAPES)
+def test_forward_and_dx_random_shapes(ops, M, N, K):
+    _, packed, scales, zeros = make_w4(N, K, M + N + K)
+    w = (packed.cuda(), scales.cuda(), zeros.cuda())
+    W = ops.a16w4_dequant(*w, (N, K)).float()
+    g = torch.Generator(device="cuda").manual_seed(M * 7 + 1)
+    x = torch.randn(M, K, device="cuda", generator=g).to(torch.bfloat16)
+    bias = torch.randn(N, device="cuda", generator=g).to(torch.bfloat16) if (M + N) % 3 == 0 else None
+    y = ops.a16w4_forward(x, *w, (N, K), bias=bias).float()
+    ref = x.float() @ W.t() + (bias.float() if bias is not None else 0)
+    assert ((y - ref).norm() / ref.norm()).item() < TOL
+    if N % 64:
+        return  # dX needs N % 64 == 0 (the forward pass N % 16)
+    dy = torch.randn(M, N, device="cuda", generator=g).to(torch.bfloat16)
+    dx = ops.a16w4_dx(dy, *w, (N, K)).float()
+    ref = dy.float() @ W
+    assert ((dx - ref).norm() / ref.norm()).item() < TOL
+
+
+@pytest.mark.parametrize("M,N,K", _shapes(3, 24, [17, 100, 256, 300, 1024, 2048, 3000], [2048, 4096, 8192], 24))
+def test_a8w8_random_shapes(ops, M, N, K):
+    g = torch.Generator(device="cuda").manual_seed(M + N + K)
+    x8 = torch.randint(-127, 128, (M, K), device="cuda", generator=g, dtype=torch.int8)
+    w8 = torch.randint(-127, 128, (N, K), device="cuda", generator=g, dtype=torch.int8)
+    sx = torch.rand(M, device="cuda", generator=g) + 0.1
+    sw = torch.rand(N, device="cuda", generator=g) + 0.1
+    y, acc = ops.a8w8_forward(x8, w8, sx, sw, want_acc=True)
+    want = x8.double() @ w8.double().t()  # exact: |acc| < 2^31 << 2^53
+    assert torch.equal(acc.double(), want)
+    assert torch.equal(y, ((want.float() * sx[:, None]) * sw[None, :]).to(torch.bfloat16))
