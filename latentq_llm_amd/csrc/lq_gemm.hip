@@ -867,8 +867,9 @@ extern "C" int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const 
         return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 256, (hipStream_t)stream);
     // the same kernel with 128 x 128 tiles (two workgroups per CU) when there are more of them than
     // compute units, or when the reduction is short (<= 16 steps: less to set up than the staged
-    // kernel's producer waves); measured 16.0 -> 14.6 us on 2048^3, 40.6 -> 39.1 on 2048 x 4096 x 4096.
-    // A lone workgroup per CU on a long reduction is faster in the staged kernel (8 waves).
+    // kernel's producer waves); measured 16.0 -> 13.1 us on 2048^3, 40.6 -> 37.0 on 2048 x 4096 x 4096.
+    // A lone workgroup per CU on a long reduction is faster in the staged kernel (41 against 44 us on
+    // 2048 x 2048 x 8192).
     if (((M + 127) / 128) * ((N + 127) / 128) > (long long)lq_device_cu_count() || K <= 2048)
         return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, (hipStream_t)stream);
     GemmParams p = {};

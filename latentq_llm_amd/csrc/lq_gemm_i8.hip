@@ -10,7 +10,7 @@
 // Main instance: 256 x 256 tile, 512 threads = 8 waves in a 2 (m) x 4 (n) grid; a wave owns
 // 128 x 64 outputs (4 x 2 MFMA 32x32x32 tiles, 128 accumulator registers), two waves per SIMD. One
 // workgroup per CU: two LDS stages of 64 KB (256 rows of A and 256 rows of B, 128 bytes = 128 k
-// each). Second instance for small outputs: 128 x 128 tile, 4 waves (2 x 2, 64 x 64 each), two
+// each). Second instance for small outputs: 128 x 128 tile, 8 waves (2 x 4, 64 x 32 each), two
 // stages of 32 KB, two workgroups per CU.
 //
 // Reduction step = 128 k in four slices of 32. Lane l: r = l % 32, h = l / 32. In slice t the
@@ -54,8 +54,9 @@ using ic = std::integral_constant<int, I>;
 constexpr int ROWB = 128;  // bytes (= k) per tile row and step
 
 // BM x BN tile, WM x WN waves. Two instances: 256 x 256 with 2 x 4 waves (one workgroup per CU) and
-// 128 x 128 with 2 x 2 waves (64 KB of LDS: two per CU) for outputs too small to fill the device
-// with the large tile. Both fill a stage with 4 + 4 loads per thread.
+// 128 x 128 with 2 x 4 waves of 64 x 32 (64 KB of LDS: two per CU) for outputs too small to fill the
+// device with the large tile; with 2 x 2 waves of 64 x 64 it was 5-12 % slower (one wave per SIMD
+// when a workgroup has a CU to itself).
 template <int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) {
     constexpr int NT = 64 * WM * WN;
@@ -63,8 +64,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) 
     constexpr int STAGE = (BM + BN) * ROWB;
     constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
     constexpr int FM = TM / 32, FN = TN / 32;
-    static_assert(BM * 8 == 4 * NT && BN * 8 == 4 * NT, "a stage is 4 + 4 loads per thread");
-    static_assert(FN == 2, "the epilogue regroups 64 columns per wave");
+    constexpr int LA = BM * 8 / NT, LB = BN * 8 / NT;  // 16-byte loads per thread and stage: A, then B
+    static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0 && LA >= 1 && LB >= 1, "a stage divides over the threads");
     __shared__ __attribute__((aligned(16))) unsigned char lds0[STAGE];
     __shared__ __attribute__((aligned(16))) unsigned char lds1[STAGE];
     auto stage = [&](auto i) -> unsigned char * {
@@ -97,28 +98,29 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) 
 
     // ---- staging: 2048 16-byte slots per operand and stage; slot s = i*512 + thread -> row s/8,
     // position s%8. Rows past the end of a matrix re-read its last row (their results are dropped).
-    unsigned a_off[4], b_off[4];
+    unsigned a_off[LA], b_off[LB];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < (LA > LB ? LA : LB); ++i) {
         const int row = i * (NT / 8) + (int)(threadIdx.x >> 3);
         const int pos = threadIdx.x & 7;
         const int chunk = pos ^ ((row >> 1) & 7);
         int ga = m0 + row, gb = c0 + row;
         ga = ga < p.M ? ga : p.M - 1;
         gb = gb < p.N ? gb : p.N - 1;
-        a_off[i] = (unsigned)((long long)(ga - m0) * p.K + chunk * 16);
-        b_off[i] = (unsigned)((long long)(gb - c0) * p.K + chunk * 16);
+        if (i < LA) a_off[i] = (unsigned)((long long)(ga - m0) * p.K + chunk * 16);
+        if (i < LB) b_off[i] = (unsigned)((long long)(gb - c0) * p.K + chunk * 16);
     }
     const unsigned char *a_base = p.x + (long long)m0 * p.K;
     const unsigned char *b_base = p.w + (long long)c0 * p.K;
-    // load i (0..7) of a step: 0..3 fill the A rows of the stage, 4..7 its B rows
+    // load i of a step: 0..LA-1 fill the A rows of the stage, LA..LA+LB-1 its B rows
     auto issue_one = [&](int kt, unsigned char *st, int i) {
-        const bool is_b = i >= 4;
+        const bool is_b = i >= LA;
+        const int ii = is_b ? i - LA : i;
         const unsigned char *src = (is_b ? b_base : a_base) + (long long)kt * ROWB;
         const unsigned lds_addr = (unsigned)reinterpret_cast<size_t>(
-            (lds_void *)(st + (is_b ? A_STAGE : 0) + ((i & 3) * NT + wave * 64) * 16));
+            (lds_void *)(st + (is_b ? A_STAGE : 0) + (ii * NT + wave * 64) * 16));
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                     :: "s"(lds_addr), "v"(is_b ? b_off[i & 3] : a_off[i & 3]), "s"(src) : "memory");
+                     :: "s"(lds_addr), "v"(is_b ? b_off[ii < LB ? ii : 0] : a_off[ii < LA ? ii : 0]), "s"(src) : "memory");
     };
 
     // ---- fragments: tile row x + r, chunk (4h + t) at position chunk ^ ((r >> 1) & 7)
@@ -155,12 +157,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) 
             if (t == 0) {
                 // second half of the next step's loads (its stage was released by the previous barrier)
 #pragma unroll
-                for (int i = 4; i < 8; ++i) issue_one(kt1, nxt, i);
+                for (int i = LA; i < LA + LB; ++i) issue_one(kt1, nxt, i);
             }
             if (t == 3) {
                 // first half of the loads of the step after next, into the stage just released
 #pragma unroll
-                for (int i = 0; i < 4; ++i) issue_one(kt2, cur, i);
+                for (int i = 0; i < LA; ++i) issue_one(kt2, cur, i);
             }
             // the reads and loads above go out before this slice's MFMAs, which cover their latency
             __builtin_amdgcn_sched_barrier(0);
@@ -176,10 +178,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) 
 
     // prologue: step 0 entirely, the first half of step 1; wait for step 0 (all but the 4 newest)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) issue_one(0, lds0, i);
+    for (int i = 0; i < LA + LB; ++i) issue_one(0, lds0, i);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) issue_one(nk > 1 ? 1 : 0, lds1, i);
-    asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");
+    for (int i = 0; i < LA; ++i) issue_one(nk > 1 ? 1 : 0, lds1, i);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(LA) : "memory");
     read_frags(lds0, 0, af[0], bf[0]);
     __builtin_amdgcn_sched_barrier(0);
     int kt = 0;
@@ -191,14 +193,17 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) 
     // the clamped prefetches of the last steps are still writing LDS: drain them
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    // ---- epilogue: acc[i][j][q]: column c0 + 64*wn + 32i + 8*(q/4) + 4h + q%4, row m0 + TM*wm + 32j + r.
+    // ---- epilogue: acc[i][j][q]: column c0 + TN*wn + 32i + 8*(q/4) + 4h + q%4, row m0 + TM*wm + 32j + r.
     // Every wave passes its block through a private LDS area, 32 rows (one j) at a time, and stores
-    // 16 bytes per lane with 8 lanes on the 128 contiguous bytes of a row: full cache lines.
+    // 16 bytes per lane with TN/8 lanes on the contiguous bytes of a row.
     __syncthreads();
-    constexpr int EP = 144;  // row pitch of the staging area
+    constexpr int EP = TN * 2 + 16;   // row pitch of the staging area
+    constexpr int LPR = TN / 8;        // lanes per staged row (16 bytes each)
+    constexpr int RPI = 64 / LPR;      // rows per store instruction
+    static_assert(NT / 64 * 32 * EP <= STAGE, "epilogue staging fits a stage");
     unsigned char *ep = lds0 + wave * (32 * EP);
-    const int ep_row = lane >> 3, ep_chunk = lane & 7;
-    const int cw0 = c0 + wn * 64;
+    const int ep_row = lane / LPR, ep_chunk = lane % LPR;
+    const int cw0 = c0 + wn * TN;
     const int c_lane = cw0 + ep_chunk * 8;  // first of the 8 columns this lane stores
     float bias_v[FN][4][4], sw_v[FN][4][4];
 #pragma unroll
@@ -238,8 +243,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) 
             }
         }
 #pragma unroll
-        for (int it = 0; it < 4; ++it) {
-            const int row = it * 8 + ep_row;
+        for (int it = 0; it < 32 / RPI; ++it) {
+            const int row = it * RPI + ep_row;
             const u32x4_t o = *reinterpret_cast<const u32x4_t *>(ep + row * EP + ep_chunk * 16);
             const int mm = mrow0 + row;
             if (mm < p.M && c_lane < p.N) *reinterpret_cast<u32x4_t *>(p.y + (long long)mm * p.N + c_lane) = o;
@@ -253,7 +258,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) 
 long long lq_gemm_i8_256_workgroups(int M, int N) { return (long long)((M + 255) / 256) * ((N + 255) / 256); }
 
 // Called by lq_a8w8_fwd (lq_gemm.hip) after argument validation: K % 128 == 0, N % 16 == 0.
-// tile = 256 or 128 (square tiles).
+// tile = 256 or 128 (square tiles, 8 waves each).
 int lq_gemm_i8_tile_launch(const void *x8, const void *w8, const float *sx, const float *sw, const void *bias, void *y,
                            int *acc_or_null, int M, int N, int K, int tile, hipStream_t st) {
     I8Params p = {};
@@ -267,6 +272,6 @@ int lq_gemm_i8_tile_launch(const void *x8, const void *w8, const float *sx, cons
     // the 32-bit lane offsets of the loads span up to 256 rows
     if (256ll * K >= (1ll << 32)) return lq_fail(LQ_ERR_BAD_ARG, "lq_a8w8_fwd: K too large");
     if (tile == 256) hipLaunchKernelGGL((gemm_i8_tile_kernel<256, 256, 2, 4>), dim3((unsigned)nwg), dim3(512), 0, st, p);
-    else hipLaunchKernelGGL((gemm_i8_tile_kernel<128, 128, 2, 2>), dim3((unsigned)nwg), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((gemm_i8_tile_kernel<128, 128, 2, 4>), dim3((unsigned)nwg), dim3(512), 0, st, p);
     return lq_check_launch("lq_a8w8_fwd");
 }
