@@ -615,7 +615,7 @@ int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scal
 // int8 GEMM with 256 x 256 tiles (lq_gemm_i8.hip)
 long long lq_gemm_i8_256_workgroups(int M, int N);
 int lq_gemm_i8_tile_launch(const void *x8, const void *w8, const float *sx, const float *sw, const void *bias, void *y,
-                           int *acc_or_null, int M, int N, int K, int tile, hipStream_t st);
+                           int *acc_or_null, int M, int N, int K, int tile, int stages, hipStream_t st);
 
 // GEMV path (lq_gemv.hip)
 int lq_gemv_a16w4_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
@@ -864,14 +864,19 @@ extern "C" int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const 
     // 256 x 256 tiles, both operands through LDS, when they occupy more than half of the compute
     // units; below that the staged kernel's smaller tiles fill the device better
     if (lq_gemm_i8_256_workgroups((int)M, (int)N) * 2 > (long long)lq_device_cu_count())
-        return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 256, (hipStream_t)stream);
+        return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 256, 2, (hipStream_t)stream);
     // the same kernel with 128 x 128 tiles (two workgroups per CU) when there are more of them than
     // compute units, or when the reduction is short (<= 16 steps: less to set up than the staged
     // kernel's producer waves); measured 16.0 -> 13.1 us on 2048^3, 40.6 -> 37.0 on 2048 x 4096 x 4096.
     // A lone workgroup per CU on a long reduction is faster in the staged kernel (41 against 44 us on
     // 2048 x 2048 x 8192).
     if (((M + 127) / 128) * ((N + 127) / 128) > (long long)lq_device_cu_count() || K <= 2048)
-        return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, (hipStream_t)stream);
+        return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 2, (hipStream_t)stream);
+    // a workgroup with a CU to itself and a long reduction: four 32 KB stages (loads three steps
+    // ahead) instead of two; measured 41 -> 37 us on 2048 x 2048 x 8192, 146 -> 127 on K = 32768, but
+    // slower than the staged kernel below 48 steps (27.5 against 24.2 us at K = 4096)
+    if (K >= 6144)
+        return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 4, (hipStream_t)stream);
     GemmParams p = {};
     p.a = x; p.b = w; p.sx = sx; p.sw = sw; p.bias = (const unsigned short *)bias_or_null; p.c = y;
     p.acc_out = acc_or_null;

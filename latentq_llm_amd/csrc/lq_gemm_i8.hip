@@ -10,8 +10,8 @@
 // Main instance: 256 x 256 tile, 512 threads = 8 waves in a 2 (m) x 4 (n) grid; a wave owns
 // 128 x 64 outputs (4 x 2 MFMA 32x32x32 tiles, 128 accumulator registers), two waves per SIMD. One
 // workgroup per CU: two LDS stages of 64 KB (256 rows of A and 256 rows of B, 128 bytes = 128 k
-// each). Second instance for small outputs: 128 x 128 tile, 8 waves (2 x 4, 64 x 32 each), two
-// stages of 32 KB, two workgroups per CU.
+// each). For small outputs: 128 x 128 tile, 8 waves (2 x 4, 64 x 32 each), with two stages of
+// 32 KB (two workgroups per CU) or four (one workgroup per CU, loads three steps ahead).
 //
 // Reduction step = 128 k in four slices of 32. Lane l: r = l % 32, h = l / 32. In slice t the
 // lane's operand of row r is chunk 4h + t (16 bytes) of the row's 128 bytes, for A and B alike
@@ -57,8 +57,9 @@ constexpr int ROWB = 128;  // bytes (= k) per tile row and step
 // 128 x 128 with 2 x 4 waves of 64 x 32 (64 KB of LDS: two per CU) for outputs too small to fill the
 // device with the large tile; with 2 x 2 waves of 64 x 64 it was 5-12 % slower (one wave per SIMD
 // when a workgroup has a CU to itself).
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int NS>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) {
+    static_assert(NS == 2 || NS == 4, "two or four stages");
     constexpr int NT = 64 * WM * WN;
     constexpr int A_STAGE = BM * ROWB;       // A rows, then B rows
     constexpr int STAGE = (BM + BN) * ROWB;
@@ -66,12 +67,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) 
     constexpr int FM = TM / 32, FN = TN / 32;
     constexpr int LA = BM * 8 / NT, LB = BN * 8 / NT;  // 16-byte loads per thread and stage: A, then B
     static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0 && LA >= 1 && LB >= 1, "a stage divides over the threads");
-    __shared__ __attribute__((aligned(16))) unsigned char lds0[STAGE];
-    __shared__ __attribute__((aligned(16))) unsigned char lds1[STAGE];
-    auto stage = [&](auto i) -> unsigned char * {
-        constexpr int I = decltype(i)::value;
-        return I == 0 ? lds0 : lds1;
-    };
+    __shared__ __attribute__((aligned(16))) unsigned char lds_all[NS * STAGE];
+    unsigned char *const lds0 = lds_all;
+    auto stage = [&](auto i) -> unsigned char * { return lds_all + decltype(i)::value * STAGE; };
 
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
@@ -144,25 +142,28 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) 
             for (int q = 0; q < 16; ++q) acc[i][j][q] = 0;
 
     u32x4_t af[2][FM], bf[2][FN];
-    // Step kt on stage S: the operands of its first slice are already in af[0] / bf[0].
+    // Step kt on stage S = kt % NS: the operands of its first slice are already in af[0] / bf[0].
+    // Loads run NS - 1 steps ahead: the barrier of a step releases its stage, into which the last
+    // slice issues the A half of step kt + NS and the next step's first slice the B half; the wait
+    // in front of a barrier leaves the loads of the NS - 2 steps after the next one in flight.
     auto step = [&](int kt, auto si) {
         constexpr int S = decltype(si)::value;
-        unsigned char *cur = stage(ic<S>()), *nxt = stage(ic<S ^ 1>());
-        const int kt1 = kt + 1 < nk ? kt + 1 : nk - 1, kt2 = kt + 2 < nk ? kt + 2 : nk - 1;
+        unsigned char *cur = stage(ic<S>()), *nxt = stage(ic<(S + 1) % NS>()), *prv = stage(ic<(S + NS - 1) % NS>());
+        const int kt_b = kt + NS - 1 < nk ? kt + NS - 1 : nk - 1, kt_a = kt + NS < nk ? kt + NS : nk - 1;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            if (t == 3) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            if (t == 3) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NS - 2) * (LA + LB)) : "memory");
             if (t < 3) read_frags(cur, t + 1, af[(t + 1) & 1], bf[(t + 1) & 1]);
             else read_frags(nxt, 0, af[0], bf[0]);
             if (t == 0) {
-                // second half of the next step's loads (its stage was released by the previous barrier)
+                // B half of the loads of step kt + NS - 1 (its stage was released by the previous barrier)
 #pragma unroll
-                for (int i = LA; i < LA + LB; ++i) issue_one(kt1, nxt, i);
+                for (int i = LA; i < LA + LB; ++i) issue_one(kt_b, prv, i);
             }
             if (t == 3) {
-                // first half of the loads of the step after next, into the stage just released
+                // A half of the loads of step kt + NS, into the stage just released
 #pragma unroll
-                for (int i = 0; i < LA; ++i) issue_one(kt2, cur, i);
+                for (int i = 0; i < LA; ++i) issue_one(kt_a, cur, i);
             }
             // the reads and loads above go out before this slice's MFMAs, which cover their latency
             __builtin_amdgcn_sched_barrier(0);
@@ -176,20 +177,40 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) 
         }
     };
 
-    // prologue: step 0 entirely, the first half of step 1; wait for step 0 (all but the 4 newest)
+    // prologue: steps 0 .. NS-2 entirely, the A half of step NS-1; wait for step 0 (everything but the
+    // loads issued after it)
+    auto issue_step = [&](int kt, unsigned char *st, int first, int last) {
+        const int k = kt < nk ? kt : nk - 1;
 #pragma unroll
-    for (int i = 0; i < LA + LB; ++i) issue_one(0, lds0, i);
-#pragma unroll
-    for (int i = 0; i < LA; ++i) issue_one(nk > 1 ? 1 : 0, lds1, i);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(LA) : "memory");
+        for (int i = first; i < last; ++i) issue_one(k, st, i);
+    };
+    issue_step(0, stage(ic<0>()), 0, LA + LB);
+    if constexpr (NS == 4) {
+        issue_step(1, stage(ic<1>()), 0, LA + LB);
+        issue_step(2, stage(ic<2>()), 0, LA + LB);
+    }
+    issue_step(NS - 1, stage(ic<NS - 1>()), 0, LA);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((NS - 2) * (LA + LB) + LA) : "memory");
     read_frags(lds0, 0, af[0], bf[0]);
     __builtin_amdgcn_sched_barrier(0);
     int kt = 0;
-    for (; kt + 2 <= nk; kt += 2) {
-        step(kt, ic<0>());
-        step(kt + 1, ic<1>());
+    if constexpr (NS == 2) {
+        for (; kt + 2 <= nk; kt += 2) {
+            step(kt, ic<0>());
+            step(kt + 1, ic<1>());
+        }
+        if (kt < nk) step(kt, ic<0>());
+    } else {
+        for (; kt + 4 <= nk; kt += 4) {
+            step(kt, ic<0>());
+            step(kt + 1, ic<1>());
+            step(kt + 2, ic<2>());
+            step(kt + 3, ic<3>());
+        }
+        if (kt < nk) step(kt, ic<0>());
+        if (kt + 1 < nk) step(kt + 1, ic<1>());
+        if (kt + 2 < nk) step(kt + 2, ic<2>());
     }
-    if (kt < nk) step(kt, ic<0>());
     // the clamped prefetches of the last steps are still writing LDS: drain them
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
@@ -200,7 +221,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) 
     constexpr int EP = TN * 2 + 16;   // row pitch of the staging area
     constexpr int LPR = TN / 8;        // lanes per staged row (16 bytes each)
     constexpr int RPI = 64 / LPR;      // rows per store instruction
-    static_assert(NT / 64 * 32 * EP <= STAGE, "epilogue staging fits a stage");
+    static_assert(NT / 64 * 32 * EP <= NS * STAGE, "epilogue staging fits the stages");
     unsigned char *ep = lds0 + wave * (32 * EP);
     const int ep_row = lane / LPR, ep_chunk = lane % LPR;
     const int cw0 = c0 + wn * TN;
@@ -258,9 +279,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) 
 long long lq_gemm_i8_256_workgroups(int M, int N) { return (long long)((M + 255) / 256) * ((N + 255) / 256); }
 
 // Called by lq_a8w8_fwd (lq_gemm.hip) after argument validation: K % 128 == 0, N % 16 == 0.
-// tile = 256 or 128 (square tiles, 8 waves each).
+// tile = 256 or 128 (square tiles, 8 waves each); stages = 2, or 4 with the 128 tile.
 int lq_gemm_i8_tile_launch(const void *x8, const void *w8, const float *sx, const float *sw, const void *bias, void *y,
-                           int *acc_or_null, int M, int N, int K, int tile, hipStream_t st) {
+                           int *acc_or_null, int M, int N, int K, int tile, int stages, hipStream_t st) {
     I8Params p = {};
     p.x = (const unsigned char *)x8; p.w = (const unsigned char *)w8; p.sx = sx; p.sw = sw;
     p.bias = (const unsigned short *)bias; p.y = (unsigned short *)y; p.acc_out = acc_or_null;
@@ -271,7 +292,8 @@ int lq_gemm_i8_tile_launch(const void *x8, const void *w8, const float *sx, cons
     if (nwg > 0x7FFFFFFFll) return lq_fail(LQ_ERR_BAD_ARG, "lq_a8w8_fwd: problem too large");
     // the 32-bit lane offsets of the loads span up to 256 rows
     if (256ll * K >= (1ll << 32)) return lq_fail(LQ_ERR_BAD_ARG, "lq_a8w8_fwd: K too large");
-    if (tile == 256) hipLaunchKernelGGL((gemm_i8_tile_kernel<256, 256, 2, 4>), dim3((unsigned)nwg), dim3(512), 0, st, p);
-    else hipLaunchKernelGGL((gemm_i8_tile_kernel<128, 128, 2, 4>), dim3((unsigned)nwg), dim3(512), 0, st, p);
+    if (tile == 256) hipLaunchKernelGGL((gemm_i8_tile_kernel<256, 256, 2, 4, 2>), dim3((unsigned)nwg), dim3(512), 0, st, p);
+    else if (stages == 4) hipLaunchKernelGGL((gemm_i8_tile_kernel<128, 128, 2, 4, 4>), dim3((unsigned)nwg), dim3(512), 0, st, p);
+    else hipLaunchKernelGGL((gemm_i8_tile_kernel<128, 128, 2, 4, 2>), dim3((unsigned)nwg), dim3(512), 0, st, p);
     return lq_check_launch("lq_a8w8_fwd");
 }
