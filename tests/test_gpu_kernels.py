@@ -279,7 +279,10 @@ def test_a16w4_adjoint_identity(ops):
                                         # ragged and large enough for the weights-direct kernel; odd number of K steps
                                         (4100, 4112, 384, True),
                                         # one and two K steps through the 256 x 256 tile kernel
-                                        (3600, 3648, 128, False), (3330, 3840, 256, True)])
+                                        (3600, 3648, 128, False), (3330, 3840, 256, True),
+                                        # long reductions on small outputs: four stages, 49 / 50 / 51 / 52 steps
+                                        (300, 512, 6272, True), (129, 256, 6400, False), (520, 1040, 6528, True),
+                                        (64, 128, 6656, False)])
 def test_a8w8(ops, co, M, N, K, bias):
     g = torch.Generator().manual_seed(M + N + K)
     x8 = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
