@@ -6,7 +6,9 @@
  *   - every pointer is a DEVICE pointer on the current HIP device unless the
  *     parameter is documented as a host value;
  *   - the caller allocates every output; the library allocates nothing, never
- *     synchronises, keeps no mutable global state and is re-entrant;
+ *     synchronises and is re-entrant; the only state it keeps between calls is a
+ *     per-thread error text and a per-device cache of the compute-unit count
+ *     (one relaxed atomic each);
  *   - work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the
  *     default stream) and the call returns immediately;
  *   - return value: LQ_OK (0) on success, a negative LQ_ERR_* code otherwise;
@@ -51,26 +53,33 @@ const char *lq_last_error(void);
  * Replaces, on the latent-weight update path, the sequence
  *   DeQfunc_4bit_g -> (update) -> Qfunc_4bit_g_res -> python_compress
  * of the reference (utils/quant.py:1073, 1139-1144, 45-72), for the update
- * rule  code' = clamp(floor((deq(W) - lr*g)/s + z + u), 0, 15)  with
+ * rule  code' = clamp(floor((deq(W) - lr*g)/s + z + u), 0, 15)  evaluated as
  *   w  = bf16_rne( bf16_rne(q - z) * s )          (reference dequant arithmetic)
  *   t  = fma(-lr, g, w)                           (fp32, one rounding)
- *   v  = ((t / s) + z) + u                        (fp32, IEEE, left to right)
- *   code' = v<0 or NaN ? 0 : v>15 ? 15 : floor(v)
+ *   y  = fma(t, (1/s) * 65536, fma(z, 65536, 0.5))   (fp32; 1/s the IEEE quotient:
+ *                                                  (t/s + z) in 16.16 fixed point, plus one half)
+ *   X  = y as an unsigned 32-bit integer, truncated, saturated (NaN, negative -> 0)
+ *   code' = min( min(X + a, 2^32 - 1) >> 16, 15 )
+ * where a is a 16-bit uniform integer draw: the noise is u = (a + 1/2) * 2^-16, uniform on the
+ * centred 2^-16 grid, and x + u is formed exactly (integer addition), so that the expected new
+ * code equals x to within 2^-17 with no common drift.
  * codes_in / codes_out: N*K/2 bytes, native layout (may alias each other).
  * scales, zeros: bf16[N*K/128]. grad: bf16[N,K] row-major. lr: host float.
  * codes_in, codes_out, grad and u must be 16-byte aligned.
- * Noise: if u_or_null != NULL it is an fp32[N,K] array of u in [0,1);
- * otherwise u for flat element index i is word (i & 3) of
- * Philox4x32-10(counter = philox_offset + i/4 as a 128-bit little-endian
- * integer in the low 64 bits, key = philox_seed) mapped as (x >> 8) * 2^-24.
+ * Noise: if u_or_null != NULL it is an fp32[N,K] array of uniforms and a = floor(u * 65536)
+ * (only 16 fractional bits of u are used; u >= 1 counts as 65535, negative or NaN as 0);
+ * otherwise a for flat element index i is the 16-bit half i & 1 (1 = the high half) of word
+ * (i >> 1) & 3 of Philox4x32-10(counter = philox_offset + i/8 as a 128-bit little-endian
+ * integer in the low 64 bits, key = philox_seed). One call consumes N*K/8 counters.
  * ------------------------------------------------------------------------- */
 int lq_requant_sr(const void *codes_in, void *codes_out, const void *scales, const void *zeros,
                   const void *grad, float lr, int64_t N, int64_t K, int group,
                   const float *u_or_null, uint64_t philox_seed, uint64_t philox_offset,
                   void *stream);
 
-/* Materialise the same uniform stream lq_requant_sr draws from: out[i], i < n,
- * is the u that element i would receive. For exactness checks. */
+/* Materialise the uniform stream lq_requant_sr draws from: out[i] = (a_i + 1/2) * 2^-16, i < n,
+ * for the draw a_i that element i would receive; feeding out back as u_or_null reproduces the
+ * Philox-mode result bit for bit. For exactness checks. */
 int lq_philox_uniform(float *out, int64_t n, uint64_t philox_seed, uint64_t philox_offset,
                       void *stream);
 
@@ -84,8 +93,10 @@ int lq_philox_uniform(float *out, int64_t n, uint64_t philox_seed, uint64_t phil
  * QLinearFunctionW4.backward (utils/quant.py:136-140): dX[M,K] = dY[M,N] * deq(W).
  * x, y, dy, dx, bias: bf16 row-major; accumulation in fp32, output rounded to
  * bf16 (round-to-nearest-even). M <= 16 takes the wavefront GEMV path.
- * Requirements: K % 128 == 0, N % 16 == 0 (fwd), N % 16 == 0 (dx); all
- * pointers 16-byte aligned.
+ * The bias is added to the fp32 sum before that single rounding; the reference rounds the
+ * product to bf16 first and then adds (utils/quant.py:118-120), one bf16 rounding more.
+ * Requirements: K % 128 == 0; N % 16 == 0 for lq_a16w4_fwd, N % 64 == 0 for lq_a16w4_dx;
+ * x, dy, codes, y, dx 16-byte aligned; scales and zeros 2-byte aligned.
  * ------------------------------------------------------------------------- */
 int lq_a16w4_fwd(const void *x, const void *codes, const void *scales, const void *zeros,
                  const void *bias_or_null, void *y, int64_t M, int64_t N, int64_t K, int group,
@@ -137,7 +148,8 @@ int lq_a16w4_dequant(const void *codes, const void *scales, const void *zeros, v
  *   y[m,n]   = bf16_rne( (float(acc) * sx[m]) * sw[n] + bias[n] )
  * x: int8[M,K], w: int8[N,K] row-major; sx: fp32[M]; sw: fp32[N];
  * bias_or_null: bf16[N]; y: bf16[M,N]; acc_or_null: int32[M,N] (written when
- * non-NULL, for the bit-exact accumulator check). K % 64 == 0, N % 16 == 0.
+ * non-NULL, for the bit-exact accumulator check). K % 128 == 0, N % 16 == 0;
+ * x, w, y, acc 16-byte aligned, sx and sw 4-byte aligned.
  * ------------------------------------------------------------------------- */
 int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const float *sw,
                 const void *bias_or_null, void *y, int32_t *acc_or_null, int64_t M, int64_t N,

@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liblatentq_hip.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _vp, _i64, _i32, _u64, _f32, _f64 = C.c_void_p, C.c_int64, C.c_int, C.c_uint64, C.c_float, C.c_double
 

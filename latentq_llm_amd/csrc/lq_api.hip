@@ -1,6 +1,7 @@
 // Error plumbing and ABI version of liblatentq_hip.so.
 #include "lq_common.h"
 
+#include <atomic>
 #include <stdarg.h>
 #include <stdio.h>
 
@@ -22,6 +23,21 @@ int lq_check_launch(const char *what) {
     return LQ_OK;
 }
 
-extern "C" int lq_abi_version(void) { return 1; }
+// Compute units of the current device. The only state the library keeps between calls besides the
+// per-thread error text: one relaxed atomic per device ordinal, written with the value the runtime
+// reports (every thread that races here writes the same number).
+int lq_device_cu_count() {
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
+extern "C" int lq_abi_version(void) { return 2; }
 
 extern "C" const char *lq_last_error(void) { return g_err; }

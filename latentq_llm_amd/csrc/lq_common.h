@@ -7,6 +7,7 @@
 // ---- error plumbing (defined in lq_api.hip) --------------------------------
 int lq_fail(int code, const char *fmt, ...);
 int lq_check_launch(const char *what);
+int lq_device_cu_count();  // compute units of the current device (cached)
 
 #define LQ_REQUIRE(cond, ...)                          \
     do {                                               \

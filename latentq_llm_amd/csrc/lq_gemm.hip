@@ -583,19 +583,6 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
 
 }  // namespace
 
-// number of compute units of the current device (cached per device)
-static int lq_device_cu_count() {
-    static int cached[64];
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev] = n;
-    }
-    return cached[dev];
-}
-
 // 128 x 128 or 256 x 128 tiles. Measured: a workgroup alone on a compute unit takes ~0.54 us per
 // 64-deep step with the small tile and ~0.75 with the large one, and a second small-tile workgroup
 // on the same unit adds its full time, so a grid costs about (rounds of one workgroup per unit) x

@@ -811,7 +811,7 @@ class MyAdam(torch.optim.Adam):
     (dequantised codes + stored residual), stepped, and re-quantised; with ``lbit=0`` the whole
     rebuild/step/re-quantise tail is one call of the stochastic-rounding requantizer.
 
-    ``sr_seed`` seeds the Philox stream of that requantizer; every call consumes N*K/4 counters."""
+    ``sr_seed`` seeds the Philox stream of that requantizer; every call consumes N*K/8 counters."""
 
     def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), obit=8, mu_updata_f=20, cpu=False, sr_seed=0):
         super().__init__(params, lr=lr, betas=betas)
@@ -1037,7 +1037,7 @@ class MyAdam(torch.optim.Adam):
                 scales, zeros, shape = _flat_qparam(p.qparam)
                 p.data = ops.requant_sr(p.data, scales, zeros, direction.view(shape), step_size, shape,
                                         seed=self.sr_seed, offset=self.sr_offset)
-                self.sr_offset += (p.numel() + 3) // 4
+                self.sr_offset += (p.numel() + 7) // 8
             elif p.wbit == 8:
                 p.data = Qfunc_8bit_res(pdata, p.residual, qscales=p.qparam)
             elif p.wbit == 4:

@@ -167,18 +167,21 @@ void lqo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t ou
     out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
 }
 
-static inline float philox_u(int64_t i, uint64_t seed, uint64_t offset) {
-    uint64_t c = offset + (uint64_t)(i >> 2);
+/* 16-bit draw of flat element i: half (i & 1; 1 = the high half) of word (i >> 1) & 3 of the block
+ * Philox4x32-10(counter = offset + i / 8, key = seed). */
+static inline uint32_t philox_draw16(int64_t i, uint64_t seed, uint64_t offset) {
+    uint64_t c = offset + (uint64_t)(i >> 3);
     uint32_t ctr[4] = {(uint32_t)c, (uint32_t)(c >> 32), 0u, 0u};
     uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
     uint32_t o[4];
     lqo_philox4x32_10(ctr, key, o);
-    return (float)(o[i & 3] >> 8) * 0x1p-24f;
+    return (o[(i >> 1) & 3] >> (16 * (i & 1))) & 0xFFFFu;
 }
 
+/* The uniform the requantizer adds for element i: (a + 1/2) * 2^-16, on the centred 2^-16 grid. */
 void lqo_philox_uniform(float *out, int64_t n, uint64_t seed, uint64_t offset) {
 #pragma omp parallel for schedule(static)
-    for (int64_t i = 0; i < n; ++i) out[i] = philox_u(i, seed, offset);
+    for (int64_t i = 0; i < n; ++i) out[i] = ((float)philox_draw16(i, seed, offset) + 0.5f) * 0x1p-16f;
 }
 
 /* ------------------------------------------------------------ requant -- */
@@ -186,10 +189,18 @@ void lqo_philox_uniform(float *out, int64_t n, uint64_t seed, uint64_t offset) {
  * no function with this formula; its nearest relatives are Qfunc_4bit_g_res
  * (utils/quant.py:45-63, Z = t/s + z then round) and the stochastic rounding
  * round(x + U(-.5,.5)) of GradientQTensor.quant (utils/quant.py:867-871).
- * Operation order, all fp32, each line one IEEE rounding:
- *   w = bf16(bf16(q - z) * s);  t = fma(-lr, g, w);  v = t / s;  v = v + z;
- *   v = v + u;  code = NaN or v < 0 -> 0, v > 15 -> 15, else floor(v).
- * u == NULL selects the Philox stream. */
+ * Operation order, fp32, each line one IEEE rounding:
+ *   w = bf16(bf16(q - z) * s);  t = fma(-lr, g, w);  r16 = (1 / s) * 65536;  c16 = fma(z, 65536, 0.5);
+ *   y = fma(t, r16, c16);                       (t/s + z) in 16.16 fixed point plus one half
+ *   X = NaN or y < 0 -> 0, y >= 2^32 -> 2^32 - 1, else trunc(y);   S = min(X + a, 2^32 - 1);
+ *   code = min(S >> 16, 15)                     = clamp(floor(x + (a + 1/2) / 65536), 0, 15)
+ * with the 16-bit draw a from the Philox stream (u == NULL) or from an injected uniform:
+ * a = NaN or u < 0 -> 0, else min(trunc(u * 65536), 65535). */
+static inline uint32_t sat_u32(float y) {
+    if (!(y >= 0.0f)) return 0u;
+    if (y >= 4294967296.0f) return 0xFFFFFFFFu;
+    return (uint32_t)y;
+}
 void lqo_requant(const uint8_t *packed_in, uint8_t *packed_out, const uint16_t *scales, const uint16_t *zeros,
                  const uint16_t *grad, float lr, int64_t N, int64_t K, int group, const float *u, uint64_t seed,
                  uint64_t offset) {
@@ -202,11 +213,22 @@ void lqo_requant(const uint8_t *packed_in, uint8_t *packed_out, const uint16_t *
             float s = bf16_to_f32(scales[i / group]), z = bf16_to_f32(zeros[i / group]);
             float w = deq_elem(code_at(packed_in, i), s, z);
             float t = fmaf(-lr, bf16_to_f32(grad[i]), w);
-            volatile float v = t / s;
-            v = v + z;
-            v = v + (u ? u[i] : philox_u(i, seed, offset));
-            float f = floorf(v);
-            nib[h] = (f != f || f < 0.0f) ? 0u : (f > 15.0f ? 15u : (unsigned)f);
+            volatile float r = 1.0f / s;
+            volatile float r16 = r * 65536.0f;
+            float c16 = fmaf(z, 65536.0f, 0.5f);
+            float y = fmaf(t, r16, c16);
+            uint32_t a;
+            if (u) {
+                volatile float ua = u[i] * 65536.0f;
+                a = sat_u32(ua);
+                if (a > 65535u) a = 65535u;
+            } else {
+                a = philox_draw16(i, seed, offset);
+            }
+            uint64_t S = (uint64_t)sat_u32(y) + a;
+            if (S > 0xFFFFFFFFull) S = 0xFFFFFFFFull;
+            uint32_t c = (uint32_t)(S >> 16);
+            nib[h] = c > 15u ? 15u : c;
         }
         packed_out[b] = (uint8_t)((nib[0] << 4) | nib[1]);
     }
@@ -273,7 +295,8 @@ void lqo_native_to_gptq(const uint8_t *packed, int32_t *qweight, int64_t N, int6
 }
 
 /* ------------------------------------------------ reciprocal-based divide -- */
-/* The HIP requantizer replaces t / s by q0 = t*r, e = fma(-q0, s, t), q = fma(e, r, q0) with
+/* The HIP latent re-quantiser (lbit = 4) and the fused Adam kernels replace t / s by
+ * q0 = t*r, e = fma(-q0, s, t), q = fma(e, r, q0) with
  * r = RN(1/s) (Markstein's correction) whenever |s| is in [2^-40, 2^40] and |t| < 2^60. This
  * routine sweeps EVERY bf16 scale in that range (both signs) against `per_scale` pseudo-random
  * numerators and counts (a) quotients that differ from IEEE t/s when |t| >= 2^-60 and (b) final

@@ -8,9 +8,11 @@ for small cases (it runs at a few thousand elements per second).
 
 Formulas modelled:
   dequant  w = bf16(bf16(q - z) * s)                       (utils/quant.py:66-72)
-  requant  t = fma(-lr, g, w); v = t / s; v = v + z; v = v + u; code' = clamp(floor(v), 0, 15)
-           every operation rounded to fp32, NaN-free inputs only
-  uniform  u_i = (word[i & 3] of Philox(counter = offset + i // 4, key = seed) >> 8) * 2^-24
+  requant  t = fma(-lr, g, w); r16 = fl(fl(1/s) * 2^16); c16 = fl(z * 2^16 + 1/2); y = fl(t * r16 + c16);
+           X = trunc(max(y, 0)) saturated at 2^32 - 1; S = min(X + a, 2^32 - 1); code' = min(S >> 16, 15)
+           every fl() one rounding to fp32, NaN- and overflow-free inputs only
+  draw     a_i = 16-bit half (i & 1) of word (i >> 1) & 3 of Philox(counter = offset + i // 8, key = seed);
+           the uniform it stands for is u_i = (a_i + 1/2) * 2^-16
 """
 import struct
 from fractions import Fraction
@@ -66,15 +68,23 @@ def dequant_model(q: int, zb: int, sb: int) -> Fraction:
     return bf16(f32(bf16(f32(q - z)) * s))
 
 
-def requant_model(q: int, zb: int, sb: int, gb: int, lr_bits: int, u: Fraction) -> int:
+def requant_model(q: int, zb: int, sb: int, gb: int, lr_bits: int, a: int) -> int:
+    """New code of one element for the 16-bit draw a."""
     z, s, g = frac_of_bf16_bits(zb), frac_of_bf16_bits(sb), frac_of_bf16_bits(gb)
     w = dequant_model(q, zb, sb)
     t = f32(w - frac_of_f32_bits(lr_bits) * g)  # one rounding: fused multiply-add
-    v = f32(t / s)
-    v = f32(v + z)
-    v = f32(v + u)
-    fl = v.numerator // v.denominator
-    return min(max(fl, 0), 15)
+    r16 = f32(f32(1 / s) * 65536)
+    c16 = f32(z * 65536 + Fraction(1, 2))
+    y = f32(t * r16 + c16)
+    x = min(max(y.numerator // y.denominator, 0), 2 ** 32 - 1)  # floor == trunc for y >= 0
+    big = min(x + a, 2 ** 32 - 1)
+    return min(big >> 16, 15)
+
+
+def draw_of_uniform(u: Fraction) -> int:
+    """16-bit draw taken from an injected uniform in [0, 1): floor(fl(u * 2^16)), at most 65535."""
+    v = f32(u * 65536)
+    return min(max(v.numerator // v.denominator, 0), 65535)
 
 
 def philox4x32_10(ctr, key):
@@ -90,7 +100,7 @@ def philox4x32_10(ctr, key):
 
 
 def uniform_draw(i: int, seed: int, offset: int) -> int:
-    """24-bit integer m of element i; u = m * 2^-24."""
-    c = (offset + i // 4) & 0xFFFFFFFFFFFFFFFF
+    """16-bit integer a of element i; the uniform it stands for is (a + 1/2) * 2^-16."""
+    c = (offset + i // 8) & 0xFFFFFFFFFFFFFFFF
     w = philox4x32_10([c & 0xFFFFFFFF, c >> 32, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
-    return w[i & 3] >> 8
+    return (w[(i >> 1) & 3] >> (16 * (i & 1))) & 0xFFFF

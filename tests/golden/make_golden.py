@@ -41,11 +41,11 @@ def main():
     for k in out["philox_kat"]:
         assert em.philox4x32_10(k["ctr"], k["key"]) == k["out"]
 
-    # uniform stream: 24-bit draws of the first 24 elements for two (seed, offset) pairs,
+    # uniform stream: 16-bit draws of the first 24 elements for two (seed, offset) pairs,
     # the second one crossing the 32-bit boundary of the counter
     out["uniform"] = []
     for seed, offset in [(7, 0), (0x0123456789ABCDEF, 2 ** 32 - 2)]:
-        out["uniform"].append({"seed": seed, "offset": offset, "m24": [em.uniform_draw(i, seed, offset) for i in range(24)]})
+        out["uniform"].append({"seed": seed, "offset": offset, "a16": [em.uniform_draw(i, seed, offset) for i in range(24)]})
 
     # dequant: (code, zero bits, scale bits) -> weight bits
     cases = []
@@ -68,10 +68,10 @@ def main():
         zb = [bf16_bits(z) for z in zvals]
         gb = [bf16_bits(rnd.gauss(0, gstd)) for _ in range(N * K)]
         lrb = f32_bits(lr)
-        m24 = [em.uniform_draw(i, seed, offset) for i in range(N * K)]
-        new = [em.requant_model(codes[i], zb[i // K], sb[i // K], gb[i], lrb, Fraction(m24[i], 2 ** 24)) for i in range(N * K)]
+        a16 = [em.uniform_draw(i, seed, offset) for i in range(N * K)]
+        new = [em.requant_model(codes[i], zb[i // K], sb[i // K], gb[i], lrb, a16[i]) for i in range(N * K)]
         out["requant"].append({"N": N, "K": K, "lr_bits": lrb, "seed": seed, "offset": offset, "codes": codes,
-                               "scale_bits": sb, "zero_bits": zb, "grad_bits": gb, "m24": m24, "new_codes": new})
+                               "scale_bits": sb, "zero_bits": zb, "grad_bits": gb, "a16": a16, "new_codes": new})
 
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "hot_path_vectors.json")
     with open(path, "w") as f:

@@ -34,6 +34,11 @@ def _pack(codes):
     return ((c[:, 0] << 4) | c[:, 1]).astype(np.uint8)
 
 
+def _uniform_of(a16):
+    """The uniform a 16-bit draw stands for: (a + 1/2) * 2^-16, exact in fp32."""
+    return ((np.array(a16, np.float64) + 0.5) * 2.0 ** -16).astype(np.float32)
+
+
 def _lr(case):
     return float(np.array([case["lr_bits"]], np.uint32).view(np.float32)[0])
 
@@ -43,8 +48,8 @@ def test_oracle_philox_and_uniform(vec, co):
     for k in vec["philox_kat"]:
         assert list(co.philox4x32_10(k["ctr"], k["key"])) == k["out"]
     for s in vec["uniform"]:
-        u = co.philox_uniform(len(s["m24"]), s["seed"], s["offset"])
-        assert np.array_equal(u, (np.array(s["m24"], np.float64) * 2.0 ** -24).astype(np.float32))
+        u = co.philox_uniform(len(s["a16"]), s["seed"], s["offset"])
+        assert np.array_equal(u, _uniform_of(s["a16"]))
 
 
 def test_oracle_dequant(vec, co):
@@ -59,8 +64,7 @@ def test_oracle_requant(vec, co):
         args = (_pack(c["codes"]), np.array(c["scale_bits"], np.uint16), np.array(c["zero_bits"], np.uint16),
                 np.array(c["grad_bits"], np.uint16), _lr(c), N, K)
         want = _pack(c["new_codes"])
-        u = (np.array(c["m24"], np.float64) * 2.0 ** -24).astype(np.float32)
-        assert np.array_equal(co.requant(*args, u=u), want)
+        assert np.array_equal(co.requant(*args, u=_uniform_of(c["a16"])), want)
         assert np.array_equal(co.requant(*args, seed=c["seed"], offset=c["offset"]), want)
 
 
@@ -69,8 +73,8 @@ def test_oracle_requant(vec, co):
 def test_hip_uniform(vec):
     from latentq_llm_amd import ops
     for s in vec["uniform"]:
-        u = ops.philox_uniform(len(s["m24"]), s["seed"], s["offset"]).cpu().numpy()
-        assert np.array_equal(u, (np.array(s["m24"], np.float64) * 2.0 ** -24).astype(np.float32))
+        u = ops.philox_uniform(len(s["a16"]), s["seed"], s["offset"]).cpu().numpy()
+        assert np.array_equal(u, _uniform_of(s["a16"]))
 
 
 @pytest.mark.gpu
@@ -96,7 +100,7 @@ def test_hip_requant(vec):
         zeros = _bf16_tensor(c["zero_bits"], (N, 1)).cuda()
         grad = _bf16_tensor(c["grad_bits"], (N, K)).cuda()
         want = _pack(c["new_codes"])
-        u = torch.from_numpy((np.array(c["m24"], np.float64) * 2.0 ** -24).astype(np.float32)).reshape(N, K).cuda()
+        u = torch.from_numpy(_uniform_of(c["a16"])).reshape(N, K).cuda()
         got_u = ops.requant_sr(codes, scales, zeros, grad, _lr(c), (N, K), u=u)
         got_p = ops.requant_sr(codes, scales, zeros, grad, _lr(c), (N, K), seed=c["seed"], offset=c["offset"])
         assert np.array_equal(got_u.cpu().numpy().view(np.uint8), want)

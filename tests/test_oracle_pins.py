@@ -10,9 +10,10 @@ function is pinned by what the mathematics fixes:
                          the GPTQ identity (q - (z_stored + 1)) * s
   A16W4 fwd / dX         torch float64 matmul on the dequantised matrix, the adjoint identity,
                          identity activations, bf16 torch.mm (the reference's CPU path) to tolerance
-  Philox4x32-10          the three Random123 known-answer vectors; uniform mapping range/grid
+  Philox4x32-10          the three Random123 known-answer vectors; draw mapping (block, word, half), range, grid
   requant                exact rational model (fractions.Fraction, own RNE rounding), invariants
-                         (idempotence, floor at u = 0, saturation), unbiasedness
+                         (idempotence, floor / ceiling at the extreme draws, saturation, 16 bits of an
+                         injected uniform), unbiasedness incl. a sub-grid drift check
   reciprocal divide      exhaustive sweep over every bf16 scale (lqo_markstein_check)
   A8W8 int32             numpy int64 matmul; extreme value 127*127*8192
   A8W8 bf16 epilogue     "parity unpinned": the reference's epilogue lives in the external,
@@ -144,26 +145,36 @@ def test_philox_known_answers():
 
 
 def test_philox_uniform_mapping():
+    """Element i takes the 16-bit half (i & 1) of word (i >> 1) & 3 of block offset + i // 8; the
+    uniform is (a + 1/2) / 65536: inside (0, 1), on the centred 2^-16 grid, never 0 or 1."""
     seed, off = 0x0123456789ABCDEF, 2 ** 32 - 2
     u = co.philox_uniform(4096, seed, off)
-    assert u.min() >= 0 and u.max() < 1 and np.all(u * 2 ** 24 == np.floor(u * 2 ** 24))
-    for i in (0, 1, 5, 4095):
-        c = off + i // 4
+    a = u.astype(np.float64) * 65536 - 0.5
+    assert u.min() > 0 and u.max() < 1 and np.all(a == np.floor(a))
+    for i in (0, 1, 5, 8, 4095):
+        c = off + i // 8
         w = co.philox4x32_10([c & 0xFFFFFFFF, c >> 32, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
-        assert u[i] == np.float32((int(w[i % 4]) >> 8) * 2.0 ** -24)
+        half = (int(w[(i >> 1) & 3]) >> (16 * (i & 1))) & 0xFFFF
+        assert u[i] == np.float32((half + 0.5) * 2.0 ** -16)
     assert 0.48 < u.mean() < 0.52 and abs(np.corrcoef(u[:-1], u[1:])[0, 1]) < 0.05
+    # the two halves of a word and the four words of a block are all used: 8 distinct draws per block
+    blk = co.philox_uniform(8, 1, 0)
+    assert len(set(blk.tolist())) == 8
 
 
 # -------------------------------------------------------------------- requant --
 def requant_model(q, zb, sb, gb, lr, u):
+    """Exact rational restatement of the update rule (own rounding helper, no float arithmetic):
+    the 16.16 fixed-point sum floor(x * 2^16 + 1/2) + a with a = floor(u * 2^16)."""
     z, s, g = frac_of_bits(zb), frac_of_bits(sb), frac_of_bits(gb)
     w = bf16(f32(bf16(f32(q - z)) * s))
     t = f32(w - Fraction(float(np.float32(lr))) * g)
-    v = f32(t / s)
-    v = f32(v + z)
-    v = f32(v + Fraction(float(u)))
-    fl = v.numerator // v.denominator
-    return min(max(fl, 0), 15)
+    r16 = f32(f32(1 / s) * 65536)
+    y = f32(t * r16 + f32(z * 65536 + Fraction(1, 2)))
+    x = min(max(y.numerator // y.denominator, 0), 2 ** 32 - 1)
+    ua = f32(Fraction(float(u)) * 65536)
+    a = min(max(ua.numerator // ua.denominator, 0), 65535)
+    return min(min(x + a, 2 ** 32 - 1) >> 16, 15)
 
 
 @pytest.mark.parametrize("lr,gstd", [(1e-4, 1e-3), (1.0, 2e-3), (3e-2, 1.0)])
@@ -192,10 +203,27 @@ def test_requant_invariants():
     big = torch.full((N, K), 1e30, dtype=torch.bfloat16)
     assert np.all(co.requant(packed.numpy(), *args, bits(big), 1.0, N, K, u=half) == 0x00)
     assert np.all(co.requant(packed.numpy(), *args, bits(-big), 1.0, N, K, u=half) == 0xFF)
-    # u = 0 is a plain floor: with g = 0 the code can only stay or drop by one (bf16 rounding of w)
+    # the smallest draw (a = 0: u = 2^-17) is a floor: with g = 0 the code can only stay or drop by one
+    # (bf16 rounding of w); the largest (a = 65535) is a ceiling: stay or rise by one
     fl = co.unpack(co.requant(packed.numpy(), *args, bits(zero_g), 1e-4, N, K, u=np.zeros(N * K, np.float32)))
     d = codes.reshape(-1).numpy().astype(int) - fl.astype(int)
     assert set(np.unique(d)) <= {0, 1}
+    top = np.full(N * K, 1.0 - 2.0 ** -17, np.float32)
+    ce = co.unpack(co.requant(packed.numpy(), *args, bits(zero_g), 1e-4, N, K, u=top))
+    d = ce.astype(int) - codes.reshape(-1).numpy().astype(int)
+    assert set(np.unique(d)) <= {0, 1}
+    # only 16 bits of an injected uniform are used, out-of-range values saturate, NaN counts as 0
+    g2 = randn_bf16((N, K), 17, 1e-2)
+    base = np.random.default_rng(5).random(N * K, dtype=np.float32)
+    trunc = np.floor(base.astype(np.float64) * 65536) / 65536
+    ra = co.requant(packed.numpy(), *args, bits(g2), 0.05, N, K, u=base)
+    assert np.array_equal(ra, co.requant(packed.numpy(), *args, bits(g2), 0.05, N, K, u=trunc.astype(np.float32)))
+    odd = base.copy()
+    odd[::3], odd[1::3] = -1.0, 7.0
+    odd[2::3] = np.nan
+    ref = np.where(np.arange(N * K) % 3 == 1, np.float32(1 - 2.0 ** -16), np.float32(0)).astype(np.float32)
+    assert np.array_equal(co.requant(packed.numpy(), *args, bits(g2), 0.05, N, K, u=odd),
+                          co.requant(packed.numpy(), *args, bits(g2), 0.05, N, K, u=ref))
     # Philox mode == injected mode on the materialised stream
     g = randn_bf16((N, K), 14, 1e-2)
     a = co.requant(packed.numpy(), *args, bits(g), 0.05, N, K, seed=99, offset=5)
@@ -222,6 +250,36 @@ def test_requant_unbiased():
     inside = (target > 0.5) & (target < 14.5)
     assert inside.sum() > 100
     assert np.abs(acc / reps - target)[inside].max() < 0.12  # 4 sigma of a Bernoulli mean over 400 draws
+
+
+def test_requant_mean_over_all_65536_draws():
+    """Every 16-bit draw once per parameter set: the mean new code equals x = (w - lr g)/s + z to
+    within half a grid step (2^-17), and the centred grid leaves no common drift over sets whose x
+    falls at unrelated places inside a 2^-16 cell (an uncentred grid would show -2^-17)."""
+    sets, K = 24, 128
+    rows_per_set = 65536 // K
+    N = sets * rows_per_set
+    rng = np.random.default_rng(21)
+    q = rng.integers(2, 14, sets)
+    s_bits = bits(torch.tensor(np.abs(rng.normal(0, 0.02, sets)) / 7 + 1e-4).to(torch.bfloat16))
+    z_val = rng.integers(6, 10, sets).astype(np.float32)
+    g_bits = bits(torch.tensor(rng.normal(0, 1e-3, sets)).to(torch.bfloat16))
+    lr = np.float32(1e-4)
+    codes = np.repeat(q, 65536).astype(np.uint8)
+    packed = co.pack(codes)
+    scales = np.repeat(s_bits, rows_per_set).astype(np.uint16)
+    zeros = np.repeat(bits(torch.tensor(z_val).to(torch.bfloat16)), rows_per_set).astype(np.uint16)
+    grad = np.repeat(g_bits, 65536).astype(np.uint16)
+    u = np.tile((np.arange(65536, dtype=np.float64) + 0.5) / 65536, sets).astype(np.float32)
+    new = co.unpack(co.requant(packed, scales, zeros, grad, float(lr), N, K, u=u)).reshape(sets, 65536)
+    sf = co.bf16_bits_to_f32(s_bits).astype(np.float64)
+    gf = co.bf16_bits_to_f32(g_bits).astype(np.float64)
+    w = co.bf16_bits_to_f32(co.dequant(co.pack(np.repeat(q, K).astype(np.uint8)), s_bits, bits(torch.tensor(z_val).to(torch.bfloat16)),
+                                       sets, K)[:, 0]).astype(np.float64)
+    x = (w - float(lr) * gf) / sf + z_val
+    err = new.mean(axis=1) - x
+    assert np.abs(err).max() <= 2.0 ** -17 + 2.0 ** -20, err
+    assert abs(err.mean()) < 2.0 ** -18, err.mean()
 
 
 def test_reciprocal_divide_exhaustive_over_scales():
