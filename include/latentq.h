@@ -119,6 +119,23 @@ int lq_a16w4_fwd_ws(const void *x, const void *codes, const void *scales, const 
 int lq_a16w4_dx_ws(const void *dy, const void *codes, const void *scales, const void *zeros, void *dx, int64_t M,
                    int64_t N, int64_t K, int group, void *workspace, int64_t workspace_bytes, void *stream);
 
+/* lq_a16w4_fwd_ws with the library's own scratch instead of a caller's workspace: a static device
+ * array of LQ_STATIC_SCRATCH_BYTES that is part of the code object (every device the library runs
+ * on holds it until the process ends). No counterpart in the reference; it is for callers that
+ * cannot allocate device memory and have none to pass: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc. Neither this call nor anything it runs allocates or frees.
+ * Results equal lq_a16w4_fwd_ws called with a workspace of LQ_STATIC_SCRATCH_BYTES bytes bit for bit.
+ * For M > 16 the output must satisfy 8*M*N <= LQ_STATIC_SCRATCH_BYTES (two fp32 slices), otherwise
+ * LQ_ERR_BAD_ARG; M <= 16 (GEMV) uses no scratch. All calls on one device share that device's
+ * array: calls that may overlap on one device (different streams, different threads) race and must
+ * be ordered by the caller. Nothing in the array needs clearing between calls (every word that is
+ * read was written by the same call). The first call on a device looks the array's address up
+ * (hipGetSymbolAddress); make it outside graph capture. */
+#define LQ_STATIC_SCRATCH_BYTES (32 << 20)
+int lq_a16w4_fwd_static(const void *x, const void *codes, const void *scales, const void *zeros,
+                        const void *bias_or_null, void *y, int64_t M, int64_t N, int64_t K, int group,
+                        void *stream);
+
 /* Which kernel lq_a16w4_fwd(_ws) (backward = 0) or lq_a16w4_dx(_ws) (backward = 1) would run for a
  * shape and a workspace size, and how it would cut the reduction; launches nothing. *kernel is
  * one of LQ_PLAN_*; *splits > 1 means a split reduction of *steps_per_split 64-deep steps per slice

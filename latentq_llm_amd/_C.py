@@ -22,6 +22,7 @@ SIGNATURES = {
     "lq_philox_uniform": [_vp, _i64, _u64, _u64, _vp],
     "lq_a16w4_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
     "lq_a16w4_fwd_ws": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp],
+    "lq_a16w4_fwd_static": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
     "lq_a16w4_dx": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
     "lq_a16w4_dx_ws": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp],
     "lq_a16w4_plan": [_i32, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp],

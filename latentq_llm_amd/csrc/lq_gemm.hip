@@ -40,6 +40,8 @@
 // load never aliases the fragment reads it schedules next to it).
 #include "lq_common.h"
 
+#include <atomic>
+
 #include <type_traits>
 
 namespace {
@@ -807,6 +809,47 @@ static int a16w4_dx_impl(const char *who, const void *dy, const void *codes, con
                                            : launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
     if (rc || plan.splits < 2) return rc;
     return launch_split_reduce(p, plan.splits, (hipStream_t)stream, who);
+}
+
+// Scratch of the entry point that allocates nothing: one array per device, part of the code object,
+// held by every device the library runs on until the process ends.
+static __device__ __align__(256) unsigned char scratch[LQ_STATIC_SCRATCH_BYTES];
+
+// Device address of `scratch` on the current device; looked up once per device (the array's name is
+// only a host-side handle: each device has its own copy at its own address).
+static int lq_static_scratch(void **out) {
+    static std::atomic<void *> ptrs[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        return lq_fail(LQ_ERR_LAUNCH, "lq_a16w4_fwd_static: cannot identify the current device");
+    void *p = ptrs[dev].load(std::memory_order_acquire);
+    if (!p) {
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return lq_fail(LQ_ERR_LAUNCH, "lq_a16w4_fwd_static: hipGetSymbolAddress failed on device %d: %s", dev,
+                           hipGetErrorString(e));
+        ptrs[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return LQ_OK;
+}
+
+extern "C" int lq_a16w4_fwd_static(const void *x, const void *codes, const void *scales, const void *zeros,
+                                   const void *bias_or_null, void *y, int64_t M, int64_t N, int64_t K, int group,
+                                   void *stream) {
+    LQ_REQUIRE(M > 0 && N > 0, "lq_a16w4_fwd_static: M and N must be positive (M=%lld N=%lld)", (long long)M, (long long)N);
+    // two fp32 slices of the output are the least a split reduction takes
+    LQ_REQUIRE(M <= 16 || (M < (1ll << 31) && N < (1ll << 31) && 8 * M * N <= (int64_t)LQ_STATIC_SCRATCH_BYTES),
+               "lq_a16w4_fwd_static: an output of %lld x %lld needs %lld bytes for two fp32 slices, the static scratch holds %lld; "
+               "use lq_a16w4_fwd or lq_a16w4_fwd_ws",
+               (long long)M, (long long)N, (long long)(8 * M * N), (long long)LQ_STATIC_SCRATCH_BYTES);
+    void *ws = nullptr;
+    if (M > 16) {
+        const int rc = lq_static_scratch(&ws);
+        if (rc) return rc;
+    }
+    return a16w4_fwd_impl("lq_a16w4_fwd_static", x, codes, scales, zeros, bias_or_null, y, M, N, K, group, ws,
+                          ws ? (size_t)LQ_STATIC_SCRATCH_BYTES : 0, stream);
 }
 
 // The plan the two entry points above would follow, without launching anything.

@@ -118,6 +118,34 @@ def a16w4_forward(x, codes, scales, zeros, shape, bias=None, out=None):
     return y
 
 
+STATIC_SCRATCH_BYTES = 32 << 20
+
+
+def a16w4_forward_static(x, codes, scales, zeros, shape, out, bias=None):
+    """a16w4_forward through the entry point that allocates nothing (lq_a16w4_fwd_static): the split
+    reduction of skinny problems uses the library's static scratch array, and ``out`` is mandatory.
+    Raises LatentQError when M > 16 and 8*M*N exceeds STATIC_SCRATCH_BYTES."""
+    N, K = shape
+    _chk(x, torch.bfloat16, "x")
+    if x.dim() != 2 or x.shape[1] != K:
+        raise ValueError(f"x must be [M,{K}], got {tuple(x.shape)}")
+    _codes_ok(codes, N, K)
+    _qparam_ok(scales, zeros, N, K)
+    _chk(out, torch.bfloat16, "out")
+    M = x.shape[0]
+    if tuple(out.shape) != (M, N):
+        raise ValueError(f"out must be [{M},{N}]")
+    if bias is not None:
+        _chk(bias, torch.bfloat16, "bias")
+        if bias.numel() != N:
+            raise ValueError("bias must have N elements")
+    if M:
+        with torch.cuda.device(x.device):
+            _C.call("lq_a16w4_fwd_static", x.data_ptr(), codes.data_ptr(), scales.data_ptr(), zeros.data_ptr(),
+                    None if bias is None else bias.data_ptr(), out.data_ptr(), M, N, K, GROUP, _stream(x))
+    return out
+
+
 def a16w4_dx(dy, codes, scales, zeros, shape, out=None):
     """dX[M,K] = dY[M,N] . deq(W)[N,K]."""
     N, K = shape
