@@ -253,6 +253,22 @@ int lq_adam8_latent_w4_step(const void *grad, void *codes, int32_t *residual, co
                             double eps, double step_size, void *stream);
 
 /* ---------------------------------------------------------------------------
+ * 8-bit gradient accumulator: GradientQTensor.find_param / quant / dequant / set_value / add_ of
+ * the reference (utils/quant.py:856-898) for bit = 8 as one pass over the bf16 weight gradient,
+ * with the bf16 rounding of every tensor operation of that chain kept.
+ *   accumulate == 0 (set_value):  scale[n] = bf16(max(bf16(4 * max_k |dw[n,k]|), bf16(1e-5)) * (1/127))
+ *                                 is computed and written; x = dw
+ *   accumulate != 0 (add_):       scale[n] is read; x = bf16(bf16(q * scale[n]) + dw)
+ *   q[n,k] = clamp(rint(bf16(bf16(x / scale[n]) + noise[n,k])), -128, 127)        (written in place)
+ * dw: bf16[N,K]; q_inout: int8[N,K]; scale_inout: bf16[N]; K % 8 == 0; dw and noise 16-byte aligned,
+ * q 8-byte aligned. Noise: noise_or_null is a bf16[N,K] array (the reference draws it with
+ * uniform_(-0.5, 0.5)), otherwise noise = bf16((a + 1/2) * 2^-16 - 1/2) with the 16-bit Philox draw a
+ * of flat element n*K + k defined as for lq_requant_sr (N*K/8 counters per call).
+ * ------------------------------------------------------------------------- */
+int lq_gradq8_quant(const void *dw, int8_t *q_inout, void *scale_inout, int accumulate, int64_t N, int64_t K,
+                    const void *noise_or_null, uint64_t philox_seed, uint64_t philox_offset, void *stream);
+
+/* ---------------------------------------------------------------------------
  * Layout converters (device side).
  * GPTQ layout (reference PTQ/quant/quant_linear.py:343-389): qweight is
  * int32[K/8, N] with code(k, n) at bits 4*(k%8) of word [k/8, n].

@@ -69,24 +69,37 @@ def philox_uniform(n: int, seed: int, offset: int = 0, device="cuda"):
     return out
 
 
-# Scratch for the split-reduction GEMM of skinny problems (fp32 partial tiles): one buffer per device
-# and stream, allocated on first need and kept; the library itself never allocates.
+# Scratch for the split-reduction GEMM of skinny problems (fp32 partial tiles); the library itself
+# never allocates. Outside graph capture: one buffer of WORKSPACE_MAX_BYTES per (device, stream),
+# allocated on first need and never resized, so its address is stable; at most WORKSPACE_MAX_STREAMS
+# streams per device keep one (least recently used first out; a dropped buffer goes back to the
+# caching allocator's pool of the stream it was allocated on, which orders its reuse after the
+# kernels that still read it). Under graph capture: a buffer of the size the call needs from the
+# capturing graph's own memory pool, which lives as long as the graph and is reused by later
+# calls of the same capture.
 _WORKSPACE = {}
 WORKSPACE_MAX_BYTES = 64 << 20
+WORKSPACE_MAX_STREAMS = 8
 
 
 def _workspace(t, rows, cols):
-    """(pointer, bytes) of a scratch buffer for a rows x cols fp32 result cut into up to 8 slices, or
-    (None, 0) when the problem is not one the split reduction is meant for (more than 2048 rows)."""
+    """(tensor, pointer, bytes) of a scratch buffer for a rows x cols fp32 result cut into up to 8
+    slices, or (None, None, 0) when the problem is not one the split reduction is meant for (more than
+    2048 rows). The caller keeps the tensor referenced until its launch is enqueued."""
     if rows > 2048:
-        return None, 0
-    need = min(8 * rows * cols * 4, WORKSPACE_MAX_BYTES)
+        return None, None, 0
+    if torch.cuda.is_current_stream_capturing():
+        buf = torch.empty(min(8 * rows * cols * 4, WORKSPACE_MAX_BYTES), dtype=torch.uint8, device=t.device)
+        return buf, buf.data_ptr(), buf.numel()
     key = (t.device.index, _stream(t))
-    buf = _WORKSPACE.get(key)
-    if buf is None or buf.numel() < need:
-        buf = torch.empty(need, dtype=torch.uint8, device=t.device)
-        _WORKSPACE[key] = buf
-    return buf.data_ptr(), buf.numel()
+    buf = _WORKSPACE.pop(key, None)
+    if buf is None:
+        buf = torch.empty(WORKSPACE_MAX_BYTES, dtype=torch.uint8, device=t.device)
+        same_device = [k for k in _WORKSPACE if k[0] == key[0]]
+        for k in same_device[: max(0, len(same_device) - (WORKSPACE_MAX_STREAMS - 1))]:
+            del _WORKSPACE[k]
+    _WORKSPACE[key] = buf  # (re)inserted last: dict order is the recency order
+    return buf, buf.data_ptr(), buf.numel()
 
 
 def a16w4_forward(x, codes, scales, zeros, shape, bias=None, out=None):
@@ -112,9 +125,10 @@ def a16w4_forward(x, codes, scales, zeros, shape, bias=None, out=None):
     if M == 0:
         return y
     with torch.cuda.device(x.device):
-        ws, ws_bytes = _workspace(x, M, N) if M > 16 else (None, 0)
+        keep, ws, ws_bytes = _workspace(x, M, N) if M > 16 else (None, None, 0)
         _C.call("lq_a16w4_fwd_ws", x.data_ptr(), codes.data_ptr(), scales.data_ptr(), zeros.data_ptr(),
                 None if bias is None else bias.data_ptr(), y.data_ptr(), M, N, K, GROUP, ws, ws_bytes, _stream(x))
+        del keep
     return y
 
 
@@ -165,9 +179,10 @@ def a16w4_dx(dy, codes, scales, zeros, shape, out=None):
     if M == 0:
         return dx
     with torch.cuda.device(dy.device):
-        ws, ws_bytes = _workspace(dy, M, K)
+        keep, ws, ws_bytes = _workspace(dy, M, K)
         _C.call("lq_a16w4_dx_ws", dy.data_ptr(), codes.data_ptr(), scales.data_ptr(), zeros.data_ptr(), dx.data_ptr(),
                 M, N, K, GROUP, ws, ws_bytes, _stream(dy))
+        del keep
     return dx
 
 
@@ -299,6 +314,27 @@ def adam8_latent_w4_step(grad, codes, residual_int, scales, zeros, shape, state1
                 int(q[0]), float(q[1]), int(q[2]), float(q[3]), int(q[4]),
                 float(beta1), float(beta2), float(eps), float(step_size), _stream(grad))
     return codes
+
+
+def gradq8_quant(dw, q, scale, accumulate: bool, noise=None, seed: int = 0, offset: int = 0):
+    """The 8-bit gradient accumulator in one pass (lq_gradq8_quant): dw bf16 [N, K]; q int8 [N, K] and
+    scale bf16 [N, 1] are updated in place (scale only when ``accumulate`` is False). ``noise`` is an
+    optional bf16 [N, K] tensor of rounding noise; without it the Philox stream (seed, offset) is used."""
+    _chk(dw, torch.bfloat16, "dw")
+    _chk(q, torch.int8, "q")
+    _chk(scale, torch.bfloat16, "scale")
+    if dw.dim() != 2 or tuple(q.shape) != tuple(dw.shape) or scale.numel() != dw.shape[0]:
+        raise ValueError("dw and q must be [N, K] and scale must hold N entries")
+    if noise is not None:
+        _chk(noise, torch.bfloat16, "noise")
+        if tuple(noise.shape) != tuple(dw.shape):
+            raise ValueError("noise must have the shape of dw")
+    N, K = dw.shape
+    if N and K:
+        with torch.cuda.device(dw.device):
+            _C.call("lq_gradq8_quant", dw.data_ptr(), q.data_ptr(), scale.data_ptr(), int(bool(accumulate)), N, K,
+                    None if noise is None else noise.data_ptr(), seed & (2**64 - 1), offset & (2**64 - 1), _stream(dw))
+    return q
 
 
 def transpose_bf16(x):

@@ -14,9 +14,10 @@ Deliberate deviations from the reference, all on purpose:
     (utils/quant.py:200-201) are used: ``W8.to(bf16) * qscales``.
   * the dynamic A8W8 forward keeps ``clampv = input.max()`` on the device instead of ``.item()``
     (utils/quant.py:220, 320): same value, no host sync.
-  * ``lbit=0`` (the constructor default, which in the reference leaves an uninitialised fp32
-    latent copy) selects the stochastic-rounding latent requantizer: no stored residual, the
-    optimizer calls ``ops.requant_sr`` once per parameter (kernel 1).
+  * ``lbit=0`` on a 4-bit weight (the constructor default, which in the reference leaves an
+    uninitialised fp32 latent copy that main0.py never fills) selects the stochastic-rounding latent
+    requantizer: no stored residual, the optimizer calls ``ops.requant_sr`` once per parameter
+    (kernel 1). An 8-bit weight with ``lbit=0`` keeps the reference's fp32 latent copy.
   * ``MyAdam.step`` does not synchronise the device and empty the cache after every parameter
     (utils/quant.py:985, 1137).
 """
@@ -39,6 +40,9 @@ FUSED_LATENT = True
 # The Adam step on uint8 moments (dequantise both moments, update them, apply the update, re-quantise
 # them per block) as one HIP kernel; False runs the chain of tensor operations (same bits either way).
 FUSED_ADAM8 = True
+# The 8-bit gradient accumulator (row scales + stochastic rounding to int8, and the accumulate form) as
+# one HIP pass per micro-batch; False runs the reference's tensor operations with torch's uniform_ noise.
+FUSED_GRADQ = True
 EXT_type = torch.bfloat16  # utils/quant.py:722
 
 # dW travels from the autograd Functions to the full-backward hook through this list
@@ -541,8 +545,10 @@ class _LatentBase(object):
 
 class QuantTensor(_LatentBase):
     """Packed weight + latent information (utils/quant.py:606-663). ``lbit`` selects how the
-    sub-LSB part of the latent weight is kept: 4 -> ResidualTensor (4-bit codec), 16/32 -> a
-    bf16/fp32 copy, 0 -> nothing stored (stochastic-rounding requantizer)."""
+    sub-LSB part of the latent weight is kept: 4 -> ResidualTensor (4-bit codec), 16 -> a bf16 copy,
+    anything else -> an fp32 copy as in the reference, except that a 4-bit weight with lbit 0 stores
+    nothing (stochastic-rounding requantizer). An 8-bit weight always keeps a latent: main0.py:339-340
+    fills ``residual.data`` of a default-constructed QLinearA8W8."""
 
     def __init__(self, shape, wbit=8, gbit=8, lbit=4):
         self.shape = shape
@@ -555,7 +561,7 @@ class QuantTensor(_LatentBase):
             self.residual = ResidualTensor(qshape=[channels, prodx(shape) // channels], oshape=shape)
         elif lbit == 16:
             self.residual = torch.empty(shape, dtype=torch.bfloat16)
-        elif lbit == 0:
+        elif lbit == 0 and wbit == 4:
             self.residual = None
         else:
             self.residual = torch.empty(shape, dtype=torch.float32)
@@ -741,7 +747,18 @@ class ResidualTensor(object):
 
 
 class GradientQTensor(object):
-    """8-bit gradient accumulator with stochastic rounding (utils/quant.py:846-922)."""
+    """Gradient accumulator of a quantised weight (utils/quant.py:846-922): for ``bit <= 8`` an int8
+    tensor with one scale per output row and stochastic rounding, otherwise the plain tensor.
+
+    On the GPU with a bf16 gradient the 8-bit forms are one HIP pass each (``ops.gradq8_quant``):
+    ``set_value`` finds the row scales and quantises, ``add_`` quantises ``dequant() + fdata`` with
+    the scales of the first micro-batch, both with the bf16 rounding points of the reference's
+    tensor operations. The rounding noise comes from the library's Philox stream (``noise_seed`` and
+    a running counter shared by all instances); ``noise=`` injects a bf16 tensor instead. Anything
+    else (CPU tensors, other dtypes, FUSED_GRADQ off) runs the tensor-op chain with ``uniform_``."""
+
+    noise_seed = 0x6B0D
+    _noise_offset = 0  # Philox blocks consumed so far by all instances
 
     def __init__(self, shape, bit=8):
         self.acc_ite = 0
@@ -753,37 +770,61 @@ class GradientQTensor(object):
         self.fixscale = False
 
     def find_param(self, data):
+        """Row scale 4 * max|row| / 127, floored at 1e-5 / 127 (utils/quant.py:856-861; the factor 4
+        leaves head room for the micro-batches that add_ accumulates)."""
         self.vmax = data.abs().amax(dim=1, keepdim=True) * 4
         self.scale = (torch.clamp(self.vmax, min=1e-5) / (2 ** (self.bit - 1) - 1)).to(data.dtype)
 
-    def quant(self, fdata):
-        noise = torch.empty_like(fdata).uniform_(-0.5, 0.5)
+    def _hip_ok(self, fdata):
+        return (FUSED_GRADQ and self.bit == 8 and fdata.is_cuda and fdata.dtype == torch.bfloat16 and fdata.dim() == 2
+                and fdata.is_contiguous() and fdata.shape[1] % 8 == 0 and fdata.data_ptr() % 16 == 0)
+
+    def _hip_quant(self, fdata, accumulate, noise):
+        cls = GradientQTensor
+        if not accumulate:
+            self.qdata = torch.empty(fdata.shape, dtype=torch.int8, device=fdata.device)
+            self.scale = torch.empty((fdata.shape[0], 1), dtype=torch.bfloat16, device=fdata.device)
+        ops.gradq8_quant(fdata, self.qdata, self.scale, accumulate, noise=noise, seed=cls.noise_seed, offset=cls._noise_offset)
+        if noise is None:
+            cls._noise_offset += (fdata.numel() + 7) // 8
+
+    def quant(self, fdata, noise=None):
+        if noise is None:
+            noise = torch.empty_like(fdata).uniform_(-0.5, 0.5)
         q = torch.round(fdata / self.scale + noise)
         self.qdata = torch.clamp(q, -2 ** (self.bit - 1), 2 ** (self.bit - 1) - 1).to(torch.int8)
 
     def dequant(self):
         return self.qdata.to(self.fdtype) * self.scale
 
-    def set_value(self, fdata):
+    def set_value(self, fdata, noise=None):
         if self.bit > 8:
             self.qdata = fdata
             return
-        if not (self.fixscale and self.scale is None):
-            self.find_param(fdata)
-        self.quant(fdata)
         self.fdtype = fdata.dtype
+        if self._hip_ok(fdata) and not self.fixscale:
+            self._hip_quant(fdata, False, noise)
+        else:
+            if not (self.fixscale and self.scale is None):
+                self.find_param(fdata)
+            self.quant(fdata, noise)
         self.acc_ite = 1
 
     def zero(self):
         self.acc_ite = 0
         self.qdata = None
 
-    def add_(self, fdata):
+    def add_(self, fdata, noise=None):
         if self.bit > 8:
             self.qdata += fdata
+            return
+        self.acc_ite += 1
+        if (self._hip_ok(fdata) and isinstance(self.qdata, torch.Tensor) and self.qdata.is_cuda and self.qdata.is_contiguous()
+                and self.scale is not None and self.scale.dtype == torch.bfloat16 and self.scale.is_contiguous()
+                and self.fdtype == torch.bfloat16):
+            self._hip_quant(fdata, True, noise)
         else:
-            self.acc_ite += 1
-            self.quant(self.dequant() + fdata)
+            self.quant(self.dequant() + fdata, noise)
 
     def get_value(self):
         return self.qdata if self.bit > 8 else self.dequant()

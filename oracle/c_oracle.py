@@ -129,6 +129,18 @@ def requant(packed, scales, zeros, grad, lr, N, K, group=128, u=None, seed=0, of
     return out
 
 
+def gradq8(dw, q, scale, accumulate, N, K, noise=None, seed=0, offset=0):
+    """GradientQTensor (bit = 8) set_value / add_: returns (new int8 q [N*K], bf16 scale bits [N]).
+    dw, noise: bf16 bit patterns; q: int8 or None (set); scale: bf16 bits or None (set)."""
+    dw = _c(dw.reshape(-1), np.uint16)
+    qo = np.zeros(N * K, np.int8) if q is None else _c(q.reshape(-1), np.int8).copy()
+    so = np.zeros(N, np.uint16) if scale is None else _c(scale.reshape(-1), np.uint16).copy()
+    noise = None if noise is None else _c(noise.reshape(-1), np.uint16)
+    lib().lqo_gradq8(_p(dw), _p(qo), _p(so), C.c_int(1 if accumulate else 0), C.c_int64(N), C.c_int64(K), _p(noise),
+                     C.c_uint64(seed), C.c_uint64(offset))
+    return qo, so
+
+
 def a8w8(x, w, sx, sw, bias, M, N, K, want_y=True):
     x = _c(x.reshape(-1), np.int8)
     w = _c(w.reshape(-1), np.int8)

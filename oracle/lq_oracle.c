@@ -294,6 +294,51 @@ void lqo_native_to_gptq(const uint8_t *packed, int32_t *qweight, int64_t N, int6
         }
 }
 
+/* ------------------------------------------------- 8-bit gradient tensor -- */
+/* GradientQTensor for bit = 8, utils/quant.py:856-898, on a bf16 gradient, every tensor operation
+ * rounded to bf16 as torch does it (fp32 inside; x / python_scalar is x * (1.0f / scalar) in the
+ * tensor library's GPU kernels):
+ *   find_param :856-861  vmax = amax|dw| * 4;  scale = clamp(vmax, min=1e-5) / 127
+ *   quant      :864-868  q = clamp(round(fdata / scale + noise), -128, 127)      (round half to even)
+ *   dequant    :873-875  qdata.to(bf16) * scale
+ *   set_value  :877-885  find_param(fdata); quant(fdata)
+ *   add_       :891-898  quant(dequant() + fdata)
+ * noise == NULL: noise = bf16((a + 1/2) * 2^-16 - 1/2) with the requantizer's 16-bit Philox draw a. */
+void lqo_gradq8(const uint16_t *dw, int8_t *q, uint16_t *scale, int accumulate, int64_t N, int64_t K,
+                const uint16_t *noise, uint64_t seed, uint64_t offset) {
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; ++n) {
+        float s;
+        if (!accumulate) {
+            float m = 0.0f;
+            for (int64_t k = 0; k < K; ++k) {
+                float a = fabsf(bf16_to_f32(dw[n * K + k]));
+                if (a > m) m = a;
+            }
+            float vmax = bf16_round(m * 4.0f);
+            float lo = bf16_round(1e-5f);
+            volatile float inv = 1.0f / 127.0f;
+            s = bf16_round((vmax > lo ? vmax : lo) * inv);
+            scale[n] = f32_to_bf16(s);
+        } else {
+            s = bf16_to_f32(scale[n]);
+        }
+        for (int64_t k = 0; k < K; ++k) {
+            int64_t i = n * K + k;
+            float x = bf16_to_f32(dw[i]);
+            if (accumulate) x = bf16_round(bf16_round((float)q[i] * s) + x);
+            float nz = noise ? bf16_to_f32(noise[i])
+                             : bf16_round(((float)philox_draw16(i, seed, offset) + 0.5f) * 0x1p-16f - 0.5f);
+            volatile float quo = x / s;
+            float y = bf16_round(bf16_round(quo) + nz);
+            float r = nearbyintf(y);
+            if (!(r >= -128.0f)) r = -128.0f; /* also NaN */
+            if (r > 127.0f) r = 127.0f;
+            q[i] = (int8_t)r;
+        }
+    }
+}
+
 /* ------------------------------------------------ reciprocal-based divide -- */
 /* The HIP latent re-quantiser (lbit = 4) and the fused Adam kernels replace t / s by
  * q0 = t*r, e = fma(-q0, s, t), q = fma(e, r, q0) with
@@ -361,7 +406,10 @@ void lqo_markstein_check(uint32_t seed, int per_scale, int64_t *quot_mismatch, i
  * (mode 1). `round` is C's half-away-from-zero; the host-side random offset v0 is
  * `rand()%1000/1000`, an integer division, i.e. always 0. The reference is compiled by nvcc,
  * whose default (-fmad=true) contracts a*b+c into one FMA: fmaf is used where the source has
- * that shape. A float level below -8 converts to unsigned 0 (saturating conversion). */
+ * that shape. (On bf16 inputs the contracted and the uncontracted reading give the same level for
+ * every input of all four curves: tests/test_oracle_pins.py sweeps them against an exact rational
+ * transcription of the kernel, which is what pins this function.) A float level below -8 converts
+ * to unsigned 0 (saturating conversion). */
 static inline float residual_level(float x, int mode, float c1, float c2, float c3, float b1, float b2, int t1,
                                    int t2) {
     float S = fabsf(x);

@@ -183,3 +183,40 @@ def adam8_step(grad, state1, scale1, max1, state2, scale2, max2, beta1, beta2, e
     q1, sc1, mx1 = quant_8bit_opt(exp_avg.float(), nblk)
     q2, sc2, mx2 = quant_8bit_opt(exp_avg_sqrt.float(), nblk)
     return out, (q1, sc1, mx1, q2, sc2, mx2)
+
+
+# ------------------------------------------------------------------ A8W8 latent re-quantiser ---
+def quant_8bit_res(latent, qscales, carry=None):
+    """Qfunc_8bit_res, utils/quant.py:88-103, without the residual handle: q = round(latent / qscales)
+    (torch.round: half to even), plus the carry the residual codec returned (lbit = 4), clamped to
+    [-128, 127] as int8. Also returns the residual latent / qscales - q that the handle receives."""
+    q = latent / qscales
+    q = q.round()
+    res = latent / qscales - q
+    if carry is not None:
+        q = q + carry
+    return q.clamp(-128, 127).to(torch.int8), res
+
+
+# --------------------------------------------------------------- 8-bit gradient accumulator ---
+def gradq8_find_param(data):
+    """GradientQTensor.find_param, utils/quant.py:856-861 (bit = 8)."""
+    vmax = data.abs().amax(dim=1, keepdim=True) * 4
+    return (torch.clamp(vmax, min=1e-5) / 127).to(data.dtype)
+
+
+def gradq8_quant(fdata, scale, noise):
+    """GradientQTensor.quant, utils/quant.py:864-868, with the uniform_(-0.5, 0.5) noise injected."""
+    return torch.clamp(torch.round(fdata / scale + noise), -128, 127).to(torch.int8)
+
+
+def gradq8_set(fdata, noise):
+    """set_value, utils/quant.py:877-885: (qdata, scale)."""
+    scale = gradq8_find_param(fdata)
+    return gradq8_quant(fdata, scale, noise), scale
+
+
+def gradq8_add(qdata, scale, fdata, noise):
+    """add_, utils/quant.py:891-898: quant(dequant() + fdata) with the scale of the first micro-batch."""
+    odata = qdata.to(fdata.dtype) * scale
+    return gradq8_quant(odata + fdata, scale, noise)

@@ -73,6 +73,27 @@ def main():
         out["requant"].append({"N": N, "K": K, "lr_bits": lrb, "seed": seed, "offset": offset, "codes": codes,
                                "scale_bits": sb, "zero_bits": zb, "grad_bits": gb, "a16": a16, "new_codes": new})
 
+    # 4-bit residual codec: per companding curve (three_fold_curve_4bit, utils/quant.py:708-716) 96 bf16
+    # inputs in [-0.5, 0.5] with nibble and carry from the exact transcription of quant_kernel_bf, and
+    # the bf16 value of each of the 16 nibbles from dequant_kernel_bf (fused reading; the unfused one
+    # gives the same results on every bf16 input, see tests/test_oracle_pins.py)
+    curves = {0: (2, 0.125, 4, 0.25), 1: (2, 0.2666300266320331, 4, 0.375), 2: (2, 0.37272211741724515, 4, 0.4375),
+              3: (2, 0.4330623539159437, 4, 0.46875)}
+    out["residual_codec"] = []
+    for mu, (p1, y1, p2, y2) in curves.items():
+        k1, b1, k2, b2, k3 = p1, y1, p2 - p1, y2, 8 - p2
+        cst = em.codec_constants(k1, b1, k2, b2, k3)
+        xs = [bf16_bits(rnd.uniform(-0.5, 0.5)) for _ in range(88)] + [0x3F00, 0xBF00, 0, 0x8000, bf16_bits(b1), bf16_bits(-b1),
+                                                                        bf16_bits(b2), bf16_bits(-b2)]
+        nib, carry = [], []
+        for b in xs:
+            n, c = em.codec_nibble(em.codec_level(em.frac_of_bf16_bits(b), cst, True))
+            nib.append(n)
+            carry.append(c)
+        values = [em.bf16_bits_of_frac(em.codec_value(n, cst, True)) for n in range(16)]
+        out["residual_codec"].append({"mu": mu, "k1": k1, "b1": b1, "k2": k2, "b2": b2, "k3": k3, "x_bits": xs,
+                                      "nibble": nib, "carry": carry, "value_bits": values})
+
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "hot_path_vectors.json")
     with open(path, "w") as f:
         json.dump(out, f, separators=(",", ":"))

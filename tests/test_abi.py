@@ -75,6 +75,59 @@ def test_bad_arguments_are_rejected_without_a_gpu(hip_lib):
         _C.call("lq_a16w4_dequant", None, None, None, None, 1, 128, 128, None)
 
 
+def header_divisibility_constraints():
+    """{entry point: {dimension: modulus}} from the 'X % n == 0 [for lq_name]' statements in the comment
+    that precedes each declaration in include/latentq.h."""
+    text = open(os.path.join(ROOT, "include", "latentq.h")).read()
+    out = {}
+    for m in re.finditer(r"/\*(.*?)\*/\s*((?:int\s+lq_[a-z0-9_]+\s*\([^;]*;\s*)+)", text, flags=re.S):
+        comment, decls = m.group(1), m.group(2)
+        names = re.findall(r"int\s+(lq_[a-z0-9_]+)\s*\(", decls)
+        for dim, mod, only in re.findall(r"\b([MNK]) % (\d+) == 0(?: for (lq_[a-z0-9_]+))?", comment):
+            for n in ([only] if only else names):
+                out.setdefault(n, {})[dim] = int(mod)
+    return out
+
+
+def test_header_divisibility_constraints_are_the_ones_enforced(hip_lib):
+    """The header is the contract: every 'X % n == 0' it states is what the entry point enforces.
+    Shapes that miss a stated modulus by one (and by half of it) are rejected with a message naming
+    that modulus; only rejected shapes are passed, so nothing is ever launched."""
+    lib = hip_lib
+    cons = header_divisibility_constraints()
+    assert cons["lq_a16w4_fwd"] == {"K": 128, "N": 16} and cons["lq_a16w4_dx"] == {"K": 128, "N": 64}
+    assert cons["lq_a8w8_fwd"] == {"K": 128, "N": 16} and cons["lq_gradq8_quant"] == {"K": 8}
+    buf = (C.c_char * 4096)()
+    p = C.cast(buf, C.c_void_p)
+
+    def call(name, M, N, K):
+        if name == "lq_a16w4_fwd":
+            return lib.lq_a16w4_fwd(p, p, p, p, None, p, M, N, K, 128, None)
+        if name == "lq_a16w4_dx":
+            return lib.lq_a16w4_dx(p, p, p, p, p, M, N, K, 128, None)
+        if name == "lq_a8w8_fwd":
+            return lib.lq_a8w8_fwd(p, p, p, p, None, p, None, M, N, K, None)
+        if name == "lq_gradq8_quant":
+            return lib.lq_gradq8_quant(p, p, p, 0, N, K, None, 0, 0, None)
+        raise KeyError(name)
+
+    for name in ("lq_a16w4_fwd", "lq_a16w4_dx", "lq_a8w8_fwd", "lq_gradq8_quant"):
+        good = {"M": 32, "N": 256, "K": 1024}
+        for dim, mod in cons[name].items():
+            for bad in (good[dim] + 1, good[dim] - 1, good[dim] + mod // 2):
+                dims = dict(good, **{dim: bad})
+                assert call(name, dims["M"], dims["N"], dims["K"]) == -1, (name, dims)
+                assert f"multiple of {mod}".encode() in lib.lq_last_error(), (name, dims, lib.lq_last_error())
+    # the plan query launches nothing and accepts exactly the stated multiples
+    from latentq_llm_amd import ops
+    from latentq_llm_amd._C import LatentQError
+    for backward, name in ((False, "lq_a16w4_fwd"), (True, "lq_a16w4_dx")):
+        n = cons[name]["N"]
+        ops.a16w4_plan(32, (3 * n, 1024), backward=backward, compute_units=256)
+        with pytest.raises(LatentQError, match=f"multiple of {n}"):
+            ops.a16w4_plan(32, (3 * n + n // 2, 1024), backward=backward, compute_units=256)
+
+
 def test_ops_refuse_cpu_tensors(hip_lib):
     import torch
     from latentq_llm_amd import _C, ops

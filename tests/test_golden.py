@@ -68,7 +68,37 @@ def test_oracle_requant(vec, co):
         assert np.array_equal(co.requant(*args, seed=c["seed"], offset=c["offset"]), want)
 
 
+def _codec_words(nibbles):
+    n = np.array(nibbles, np.uint32).reshape(-1, 8)
+    return sum(n[:, k] << (28 - 4 * k) for k in range(8)).astype(np.uint32)
+
+
+def test_oracle_residual_codec(vec, co):
+    for c in vec["residual_codec"]:
+        args = (0, c["k1"], c["b1"], c["k2"], c["b2"], c["k3"])
+        q, carry = co.residual_quant(np.array(c["x_bits"], np.uint16), *args)
+        assert np.array_equal(q, _codec_words(c["nibble"]))
+        assert np.array_equal(carry, np.where(np.array(c["carry"]) == 1, 0x3F80, 0).astype(np.uint16))
+        vals = co.residual_dequant(np.array([0x01234567, 0x89ABCDEF], np.uint32), *args)
+        assert list(vals) == c["value_bits"]
+
+
 # ------------------------------------------------------------------ HIP kernels --
+@pytest.mark.gpu
+def test_hip_residual_codec(vec):
+    from latentq_llm_amd import ops
+    for c in vec["residual_codec"]:
+        args = (0, c["k1"], c["b1"], c["k2"], c["b2"], c["k3"])
+        x = _bf16_tensor(c["x_bits"], (len(c["x_bits"]),)).cuda()
+        q = torch.empty(len(c["x_bits"]) // 8, dtype=torch.int32, device="cuda")
+        ops.residual_quant(x, q, *args)
+        assert np.array_equal(q.cpu().numpy().view(np.uint32), _codec_words(c["nibble"]))
+        assert np.array_equal(bits(x.cpu()), np.where(np.array(c["carry"]) == 1, 0x3F80, 0).astype(np.uint16))
+        words = torch.from_numpy(np.array([0x01234567, 0x89ABCDEF], np.uint32).view(np.int32)).cuda()
+        assert list(bits(ops.residual_dequant(words, *args).cpu()).reshape(-1)) == c["value_bits"]
+
+
+
 @pytest.mark.gpu
 def test_hip_uniform(vec):
     from latentq_llm_amd import ops

@@ -44,8 +44,8 @@ class _Mlp:
         o.a16w4_forward(self.h, *self.down, (hid, ffn), out=self.y)
 
 
-# M = 4: the GEMV; M = 48: the GEMV in chunks or the split reduction; M = 200: split reduction with the
-# scratch buffer (allocated by the eager warm-up, before the capture); M = 640: plain GEMM kernels
+# M = 4: the GEMV; M = 48: the GEMV in chunks or the split reduction; M = 200: split reduction (its
+# scratch buffer comes from the graph's memory pool while capturing); M = 640: plain GEMM kernels
 @pytest.mark.parametrize("M,hid,ffn", [(4, 512, 1408), (48, 1024, 2816), (200, 1024, 2816), (640, 512, 1408)])
 def test_mlp_forward_replays_match_eager(ops, M, hid, ffn):
     blk = _Mlp(ops, M, hid, ffn)
@@ -75,6 +75,53 @@ def test_mlp_forward_replays_match_eager(ops, M, hid, ffn):
             blk.step()
             torch.cuda.synchronize()
             assert torch.equal(blk.y, want[0])
+
+
+def test_graphs_of_growing_token_counts_keep_their_own_scratch(ops):
+    """Graphs captured one after another on one stream for 48, 200 and then 400 tokens (each needing
+    more split-reduction scratch than the one before), eager calls of other sizes in between: every
+    graph still gives the eager result when replayed afterwards, in any order. The scratch a captured
+    call uses comes from its graph's memory pool, and the eager buffer of a stream never moves."""
+    hid, ffn = 1024, 2816
+    s = torch.cuda.Stream()
+    blocks, graphs, wants, xs = [], [], [], []
+    for i, M in enumerate((48, 200, 400)):
+        blk = _Mlp(ops, M, hid, ffn)
+        x = dev(randn_bf16((M, hid), 30 + i))
+        blk.x.copy_(x)
+        blk.step()
+        wants.append(blk.y.clone())
+        torch.cuda.synchronize()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            blk.step()
+        torch.cuda.current_stream().wait_stream(s)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            blk.step()
+        blocks.append(blk); graphs.append(g); xs.append(x)
+        # eager traffic of a larger shape on the capture stream and on the default stream
+        big = _Mlp(ops, 512, hid, ffn)
+        with torch.cuda.stream(s):
+            big.step()
+        big.step()
+        torch.cuda.synchronize()
+    for order in ((0, 1, 2), (2, 0, 1), (1, 1, 0)):
+        for k in order:
+            blocks[k].y.zero_()
+            blocks[k].x.copy_(xs[k])
+            graphs[k].replay()
+            # allocations between replays may land where a freed eager scratch buffer was
+            junk = [torch.full((1 << 20,), 7.0, device="cuda") for _ in range(8)]
+            torch.cuda.synchronize()
+            assert torch.equal(blocks[k].y, wants[k]), (order, k)
+            del junk
+    before = {k: v.data_ptr() for k, v in ops._WORKSPACE.items()}
+    _Mlp(ops, 300, hid, ffn).step()
+    torch.cuda.synchronize()
+    assert all(ops._WORKSPACE[k].data_ptr() == p for k, p in before.items())
+    dev0 = [k for k in ops._WORKSPACE if k[0] == torch.cuda.current_device()]
+    assert len(dev0) <= ops.WORKSPACE_MAX_STREAMS
 
 
 def test_requant_and_a8w8_replay(ops):

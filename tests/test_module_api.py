@@ -123,3 +123,31 @@ def test_forward_requires_gpu(Q):
     m.weight.set_value(torch.zeros(16 * 64, dtype=torch.int8), [m.scales, m.zeros, m.wshape])
     with pytest.raises(LatentQError):
         m(torch.zeros(2, 128, dtype=torch.bfloat16))
+
+
+def test_a8w8_default_lbit_keeps_a_latent_copy_like_the_reference():
+    """main0.py:329-340 builds QLinearA8W8(..., lbit=args.lbit) and, for lbit != 4, writes the
+    dequantised weight into weight.residual.data: an 8-bit weight always has a latent tensor (fp32
+    for the default lbit = 0, utils/quant.py:606-627); only a 4-bit weight with lbit = 0 has none."""
+    import torch
+    from latentq_llm_amd import convert, quant as Q
+    N, K = 16, 128
+    layer = Q.QLinearA8W8(K, N, bias=True)  # constructor defaults: lbit = 0, gbit = 8
+    assert isinstance(layer.weight.residual, torch.Tensor) and layer.weight.residual.dtype == torch.float32
+    assert isinstance(layer.weight.grad, Q.GradientQTensor)
+    g = torch.Generator().manual_seed(0)
+    ckt = {"l.qweight": torch.randint(0, 256, (N, K), generator=g, dtype=torch.uint8),
+           "l.scales": torch.rand(N, 1, generator=g) * 0.01 + 1e-3,
+           "l.inp_absmax": torch.rand(K, generator=g) * 4,
+           "l.bias": torch.randn(N, generator=g)}
+    # the reference's own statements (main0.py:331-340), then the loader that wraps them
+    ii = ckt["l.qweight"].to(torch.int32) - 128
+    layer.qscales.data = ckt["l.scales"].to(torch.bfloat16)
+    aa = (ii * layer.qscales).to(torch.bfloat16)
+    layer.weight.set_value(ii.to(torch.int8), layer.qscales)
+    layer.weight.residual.data = aa
+    assert torch.equal(layer.weight.residual.data, aa)
+    other = convert.load_a8w8(Q.QLinearA8W8(K, N, bias=True), ckt, "l")
+    assert torch.equal(other.weight.residual.data.float(), aa.float())
+    assert torch.equal(other.weight.data, ii.to(torch.int8))
+    assert Q.QuantTensor([N, K], wbit=4, gbit=16, lbit=0).residual is None

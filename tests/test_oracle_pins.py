@@ -387,3 +387,91 @@ def test_quotient_of_bf16_rounds_the_same_within_three_ulps():
         assert np.array_equal(_bf16_rne_bits(near), want), d
     frac = q.view(np.uint32) & 0xFFFF
     assert int(np.abs(frac.astype(np.int64) - 0x8000).min()) > 16  # distance to a tie, in fp32 ulps
+
+
+# ------------------------------------------------------- 8-bit gradient accumulator --
+@pytest.mark.parametrize("N,K,std", [(5, 64, 1e-3), (17, 264, 3.0), (3, 4096, 1e-6)])
+def test_gradq8_oracle_matches_torch_bf16_tensor_ops(N, K, std):
+    """The C restatement of GradientQTensor (bit = 8) against the chain of torch bf16 tensor
+    operations the reference runs (oracle/torch_ref.py spells them as utils/quant.py:856-898 does),
+    with the same injected noise: row scales and int8 values, for set_value and two add_ calls."""
+    g = torch.Generator().manual_seed(N * 1000 + K)
+    dws = [(torch.randn(N, K, generator=g) * std).to(torch.bfloat16) for _ in range(3)]
+    dws[0][1] = 0  # an all-zero row takes the 1e-5 floor of the scale
+    noises = [(torch.rand(N, K, generator=g) - 0.5).to(torch.bfloat16) for _ in range(3)]
+    want_q, want_s = tr.gradq8_set(dws[0], noises[0])
+    q, s = co.gradq8(bits(dws[0]), None, None, False, N, K, noise=bits(noises[0]))
+    assert np.array_equal(s, bits(want_s).reshape(-1))
+    assert np.array_equal(q, want_q.numpy().reshape(-1))
+    for dw, nz in zip(dws[1:], noises[1:]):
+        want_q = tr.gradq8_add(want_q, want_s, dw, nz)
+        q, s2 = co.gradq8(bits(dw), q, s, True, N, K, noise=bits(nz))
+        assert np.array_equal(s2, s) and np.array_equal(q, want_q.numpy().reshape(-1))
+    assert np.abs(q.astype(int)).max() <= 128 and (q != 0).mean() > 0.5
+
+
+def test_gradq8_philox_noise_is_the_requantizer_stream():
+    """Without injected noise element i draws bf16((a_i + 1/2) / 65536 - 1/2) from the stream that
+    lqo_philox_uniform materialises; the noise is centred and reaches +-0.5 only after rounding."""
+    N, K, seed, off = 4, 128, 99, 3
+    dw = randn_bf16((N, K), 1, 0.01)
+    u = co.philox_uniform(N * K, seed, off)
+    noise = torch.from_numpy(u - np.float32(0.5)).to(torch.bfloat16)
+    a, sa = co.gradq8(bits(dw), None, None, False, N, K, seed=seed, offset=off)
+    b, sb = co.gradq8(bits(dw), None, None, False, N, K, noise=bits(noise))
+    assert np.array_equal(a, b) and np.array_equal(sa, sb)
+    assert float(noise.float().abs().max()) <= 0.5 and abs(float(noise.float().mean())) < 0.05
+
+
+# ------------------------------------------------------------- 4-bit residual codec --
+CURVES = {0: (2, 0.125, 4, 0.25), 1: (2, 0.2666300266320331, 4, 0.375), 2: (2, 0.37272211741724515, 4, 0.4375),
+          3: (2, 0.4330623539159437, 4, 0.46875)}  # three_fold_curve_4bit, utils/quant.py:708-716
+
+
+@pytest.mark.parametrize("mu", [0, 1, 2, 3])
+def test_residual_codec_against_an_exact_transcription_of_the_kernel(mu):
+    """Every bf16 input with 2^-14 <= |x| <= 0.5 (and a sample of smaller ones) through a rational-
+    arithmetic transcription of quant_kernel_bf, in both readings of `a*b + c` (fused, as nvcc
+    compiles it by default, and unfused): the C oracle must equal the fused reading everywhere; the
+    inputs on which the two readings differ are counted (a sign or centring mistake in the dither term
+    would move thousands of levels, not a handful of ties). Dequantised values: all 16 nibbles."""
+    from tests.golden import exact_model as em
+    p1, y1, p2, y2 = CURVES[mu]
+    k1, b1, k2, b2, k3 = p1, y1, p2 - p1, y2, 8 - p2
+    cst = em.codec_constants(k1, b1, k2, b2, k3)
+    mags = [b for b in range(0x3880, 0x3F01)] + [0, 1, 0x0080, 0x1234, 0x3000, 0x387F]  # 2^-14 .. 0.5, then small ones
+    xb = np.array([m | sgn for m in mags for sgn in (0, 0x8000)], np.uint16)
+    xb = np.concatenate([xb, np.zeros((-len(xb)) % 8, np.uint16)])
+    q, carry = co.residual_quant(xb.copy(), 0, k1, b1, k2, b2, k3)
+    nib = np.array([(int(w) >> (28 - 4 * k)) & 0xF for w in q for k in range(8)])
+    differ = 0
+    for i, b in enumerate(xb):
+        x = em.frac_of_bf16_bits(int(b))
+        lf = em.codec_level(x, cst, True)
+        want_nib, want_carry = em.codec_nibble(lf)
+        assert (nib[i], int(carry[i] == 0x3F80)) == (want_nib, want_carry), (hex(int(b)), lf)
+        differ += em.codec_level(x, cst, False) != lf
+    assert differ <= len(xb) // 100, differ  # the two readings part only where x*c + v sits on a rounding edge
+    print(f"mu={mu}: fused and unfused readings differ on {differ} of {len(xb)} inputs")
+    vals = co.residual_dequant(np.array([0x01234567, 0x89ABCDEF], np.uint32), 0, k1, b1, k2, b2, k3)
+    for n in range(16):
+        assert int(vals[n]) == em.bf16_bits_of_frac(em.codec_value(n, cst, True)), n
+    # the dither v = S*499 - round(S*499) lies in [-1/2, 1/2]: it moves a level by at most one and in both
+    # directions equally often (a dropped or one-sided dither term would show here)
+    moved = []
+    for m in range(0x3C00, 0x3F01, 3):
+        for sgn in (0, 0x8000):
+            x = em.frac_of_bf16_bits(m | sgn)
+            plain = dict(cst)
+            S = abs(x)
+            if S < cst["b1"]:
+                base = em.cround(f32(x * cst["c1"]))
+            elif S < cst["b2"]:
+                base = em.cround(f32(f32(S - cst["b1"]) * cst["c2"])) + cst["t1"]
+                base = -base if x < 0 else base
+            else:
+                base = em.cround(f32(f32(S - cst["b2"]) * cst["c3"])) + cst["t2"]
+                base = -base if x < 0 else base
+            moved.append(em.codec_level(x, cst, True) - base)
+    moved = np.array(moved)
+    assert np.abs(moved).max() <= 1 and (moved != 0).mean() > 0.1 and abs(moved.mean()) < 0.08, (moved.mean(),)
