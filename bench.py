@@ -115,38 +115,75 @@ class MLPBlock:
 
 MLP_FLOP = 6 * 2 * TOKENS * HID * FFN  # 1 108.1 GFLOP
 
-# HBM traffic per GEMM launch in MB (read, written), from two counter runs of
+# HBM traffic per GEMM launch: read from profiles/gemm_a16w4_c2_counters.json, which is written together
+# with profiles/gemm_a16w4_c2_counters.md from two counter runs of
 #   rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --profile-target gemm     (then WRITE_SIZE)
-# each scaled by what the same counter reads for the 256 MiB calibration copy of the same run
-# (FETCH_SIZE reads half the bytes fetched: factor 2.000; WRITE_SIZE factor 1.000).
-PMC_GEMM_MB = {
-    "fwd_gate_up": (224.16, 45.09), "fwd_down": (190.66, 16.78),
-    "dx_gate_up": (191.95, 16.78), "dx_down": (279.10, 45.09),
-}
+# each scaled by what the same counter reads for the 256 MiB calibration copy of the same run.
 PMC_LAUNCHES = {"fwd_gate_up": 2, "fwd_down": 1, "dx_gate_up": 2, "dx_down": 1}  # per MLP step
 
 
 def gemm_traffic_bytes():
-    """Launch-weighted mean HBM bytes (read + written) per GEMM launch of the MLP step."""
-    tot = sum(n * sum(PMC_GEMM_MB[k]) for k, n in PMC_LAUNCHES.items())
+    """Launch-weighted mean HBM bytes (read + written) per GEMM launch of the MLP step, or None when
+    the counter summary is missing."""
+    path = os.path.join(ROOT, "profiles", "gemm_a16w4_c2_counters.json")
+    try:
+        with open(path) as f:
+            mb = json.load(f)["hbm_MB_per_launch"]
+        tot = sum(n * (mb[k]["read"] + mb[k]["written"]) for k, n in PMC_LAUNCHES.items())
+    except (OSError, KeyError, ValueError):
+        return None
     return tot * 1e6 / sum(PMC_LAUNCHES.values())
 
 
-def bench_requant(device):
-    from latentq_llm_amd import ops
-    N, K = 8192, 2048
-    nb = 8  # 8 x 50 MB of distinct buffers > 256 MB of last-level cache
+def _requant_sets(device, N, K, nb, seed0):
     sets = []
     for i in range(nb):
-        p, s, z = synth_w4(N, K, 10 + i, device)
+        p, s, z = synth_w4(N, K, seed0 + i, device)
         g = (torch.randn(N, K, device=device) * 1e-3).to(torch.bfloat16)
         sets.append((p, s, z, g, torch.empty_like(p)))
+    return sets
+
+
+def bench_requant(device):
+    from latentq_llm_amd import _C, ops
+    N, K = 8192, 2048
+    nb = 8  # 8 x 50 MB of distinct buffers > 256 MB of last-level cache
+    sets = _requant_sets(device, N, K, nb, 10)
     calls = [(lambda t=t, i=i: ops.requant_sr(t[0], t[1], t[2], t[3], 1e-4, (N, K), seed=7, offset=i, out=t[4]))
              for i, t in enumerate(sets)]
     sec = graph_time(calls)
     nbytes = N * K // 2 * 2 + N * K * 2 + 4 * N * K // GROUP
+    # a plain copy that moves the same number of bytes (half read, half written), same rotation
+    half = (nbytes // 2) // 16 * 16
+    bufs = [(torch.empty(half, dtype=torch.uint8, device=device).random_(0, 256), torch.empty(half, dtype=torch.uint8, device=device))
+            for _ in range(nb)]
+    for src, dst in bufs:
+        assert src.numel() == half and dst.numel() == half and src.data_ptr() % 16 == 0 and dst.data_ptr() % 16 == 0
+    copies = [(lambda b=b: _C.call("lq_calib_copy", b[0].data_ptr(), b[1].data_ptr(), half,
+                                   torch.cuda.current_stream().cuda_stream)) for b in bufs]
+    sec_copy = graph_time(copies)
+    del bufs
     return {"shape": [N, K], "us": sec * 1e6, "GB/s": nbytes / sec / 1e9, "frac_hbm": nbytes / sec / PEAK_HBM,
-            "bytes": nbytes, "noise": "in-kernel Philox4x32-10"}
+            "bytes": nbytes, "noise": "in-kernel Philox4x32-10, 16-bit draws",
+            "copy_same_bytes_us": sec_copy * 1e6, "frac_of_copy": sec_copy / sec}
+
+
+def bench_gradq8(device):
+    """The 8-bit gradient accumulator on a dW of the MLP (11008 x 4096): set_value and add_ forms."""
+    from latentq_llm_amd import ops
+    N, K = FFN, HID
+    sets = []
+    for i in range(4):
+        dw = (torch.randn(N, K, device=device) * 1e-3).to(torch.bfloat16)
+        sets.append((dw, torch.empty((N, K), dtype=torch.int8, device=device),
+                     torch.empty((N, 1), dtype=torch.bfloat16, device=device)))
+    out = {"shape": [N, K]}
+    for name, acc, nbytes in (("set", False, 3 * N * K), ("add", True, 4 * N * K)):
+        for t in sets:
+            ops.gradq8_quant(t[0], t[1], t[2], False, seed=1, offset=0)
+        sec = graph_time([(lambda t=t, i=i: ops.gradq8_quant(t[0], t[1], t[2], acc, seed=1, offset=i)) for i, t in enumerate(sets)])
+        out[name] = {"us": sec * 1e6, "GB/s": nbytes / sec / 1e9, "frac_hbm": nbytes / sec / PEAK_HBM, "bytes": nbytes}
+    return out
 
 
 def bench_latent(device):
@@ -267,6 +304,88 @@ def bench_dw(device):
     return out
 
 
+def _clock_ghz(clocks, n):
+    """Median over n records (cycles start, cycles end, 100 MHz ticks start, ticks end) of the shader clock."""
+    c = clocks[: 4 * n].view(n, 4).double()
+    ticks = (c[:, 3] - c[:, 2]).clamp_min(1)
+    return float(((c[:, 1] - c[:, 0]) / ticks * 0.1).median())
+
+
+def mfma_loop(device, zero_operands, wgs_per_cu=2, seconds=0.004):
+    """The MFMA-only loop (lq_calib_mfma_loop) under sustained load: (TFLOP/s, granted shader clock in GHz)."""
+    import ctypes
+    from latentq_llm_amd import _C
+    n = 1 << 20
+    if zero_operands:
+        a = torch.zeros(n, dtype=torch.bfloat16, device=device)
+        b = torch.zeros(n, dtype=torch.bfloat16, device=device)
+    else:
+        a = torch.randn(n, device=device).to(torch.bfloat16)
+        b = (torch.randn(n, device=device) * 0.02).to(torch.bfloat16)
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    waves = 4 * cus * wgs_per_cu
+    clocks = torch.zeros(4 * waves, dtype=torch.int64, device=device)
+    sink = torch.zeros(waves, dtype=torch.float32, device=device)
+    nw = ctypes.c_int64()
+    st = torch.cuda.current_stream().cuda_stream
+
+    def run(iters):
+        _C.call("lq_calib_mfma_loop", a.data_ptr(), b.data_ptr(), n, iters, wgs_per_cu, clocks.data_ptr(), clocks.numel(),
+                sink.data_ptr(), ctypes.addressof(nw), st)
+    iters = 20000
+    sec = event_time(lambda: run(iters), 5, warm=3, warm_seconds=0.1)
+    flop = waves * iters * 8 * 32768.0
+    return flop / sec / 1e12, _clock_ghz(clocks, waves)
+
+
+def gemm_clock(device, backward, a, w, shape):
+    """Shader clock granted to the dequant-GEMM under sustained load: 40 plain launches, then one that records
+    each workgroup's cycle and real-time counters."""
+    import ctypes
+    from latentq_llm_amd import _C, ops
+    N, K = shape
+    M = a.shape[0]
+    out = torch.empty((M, K if backward else N), dtype=torch.bfloat16, device=device)
+    fn = (lambda: ops.a16w4_dx(a, *w, shape, out=out)) if backward else (lambda: ops.a16w4_forward(a, *w, shape, out=out))
+    event_time(fn, 10)
+    clocks = torch.zeros(4 * 4096, dtype=torch.int64, device=device)
+    nwg = ctypes.c_int64()
+    for _ in range(40):
+        fn()
+    _C.call("lq_calib_gemm_clocks", int(backward), a.data_ptr(), w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(),
+            out.data_ptr(), M, N, K, GROUP, clocks.data_ptr(), clocks.numel(), ctypes.addressof(nwg),
+            torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return _clock_ghz(clocks, nwg.value)
+
+
+def bench_ceiling(device, blk, h):
+    """What the matrix pipes deliver with nothing else in the loop, at the clock the chip grants for it, next
+    to the clock it grants the two dequant-GEMM kernels and to the vendor's dense bf16 GEMM on the same shapes."""
+    out = {}
+    for name, zero in (("random_operands", False), ("zero_operands", True)):
+        for wgs in (2, 1):
+            tf, ghz = mfma_loop(device, zero, wgs)
+            out[f"mfma_loop_{name}_{wgs}wg_per_cu"] = {"TFLOP/s": tf, "clock_GHz": ghz}
+    out["clock_GHz"] = {
+        "fwd_gate_up": gemm_clock(device, False, blk.x, blk.gate, (FFN, HID)),
+        "fwd_down": gemm_clock(device, False, h, blk.down, (HID, FFN)),
+        "dx_gate_up": gemm_clock(device, True, h, blk.gate, (FFN, HID)),
+        "dx_down": gemm_clock(device, True, blk.dy, blk.down, (HID, FFN)),
+    }
+    # vendor dense bf16 GEMM (torch.mm -> hipBLASLt) on the four shapes, weights N(0, 0.02^2), no dequantisation
+    wg = (torch.randn(FFN, HID, device=device) * 0.02).to(torch.bfloat16)
+    wd = (torch.randn(HID, FFN, device=device) * 0.02).to(torch.bfloat16)
+    flop = 2 * TOKENS * HID * FFN
+    vend = {}
+    for name, fn in (("fwd_gate_up", lambda: blk.x.mm(wg.t())), ("fwd_down", lambda: h.mm(wd.t())),
+                     ("dx_gate_up", lambda: h.mm(wg)), ("dx_down", lambda: blk.dy.mm(wd))):
+        sec = event_time(fn, 30)
+        vend[name] = {"us": sec * 1e6, "TFLOP/s": flop / sec / 1e12}
+    out["vendor_dense_bf16_mm"] = vend
+    return out
+
+
 def bench_copy(device):
     """Plain streaming copy (lq_calib_copy) over buffers larger than the last-level cache: the
     HBM rate this device sustains for read + write traffic, for comparison with the 8 TB/s peak."""
@@ -302,11 +421,26 @@ def profile_target(device, which, launches=10):
         for _ in range(launches):
             o.a16w4_dx(blk.dy, *blk.down, (HID, FFN))
     elif which == "requant":
-        N, K = 8192, 2048
+        # the benchmark size (8192 x 2048), then 4 and 16 times as many rows: steady state against launch cost
+        for rows in (8192, 4 * 8192, 16 * 8192):
+            N, K = rows, 2048
+            for i in range(launches if rows == 8192 else 4):
+                p, s, z = synth_w4(N, K, 10 + i, device)
+                g = (torch.randn(N, K, device=device) * 1e-3).to(torch.bfloat16)
+                o.requant_sr(p, s, z, g, 1e-4, (N, K), seed=7, offset=i)
+                del p, s, z, g
+    elif which == "gradq8":
+        N, K = FFN, HID
         for i in range(launches):
-            p, s, z = synth_w4(N, K, 10 + i, device)
-            g = (torch.randn(N, K, device=device) * 1e-3).to(torch.bfloat16)
-            o.requant_sr(p, s, z, g, 1e-4, (N, K), seed=7, offset=i)
+            dw = (torch.randn(N, K, device=device) * 1e-3).to(torch.bfloat16)
+            q8 = torch.empty((N, K), dtype=torch.int8, device=device)
+            sc = torch.empty((N, 1), dtype=torch.bfloat16, device=device)
+            o.gradq8_quant(dw, q8, sc, False, seed=1, offset=i)
+            o.gradq8_quant(dw, q8, sc, True, seed=1, offset=i + 100)
+    elif which == "ceiling":
+        blk = MLPBlock(device)
+        h = torch.randn(TOKENS, FFN, device=device).to(torch.bfloat16)
+        print(json.dumps(bench_ceiling(device, blk, h)))
     elif which == "latent":
         N, K = 8192, 2048
         curve = (2, 0.125, 2, 0.25, 4)
@@ -349,11 +483,29 @@ def profile_target(device, which, launches=10):
     torch.cuda.synchronize()
 
 
+def _cpu_time(fn, budget_s, min_runs=1, max_runs=7):
+    """Median seconds per call after one warm-up, within a time budget."""
+    fn()
+    ts, t_start = [], time.time()
+    while len(ts) < min_runs or (time.time() - t_start < budget_s and len(ts) < max_runs):
+        t0 = time.time()
+        fn()
+        ts.append(time.time() - t0)
+    ts.sort()
+    return ts[len(ts) // 2], len(ts)
+
+
 def cpu_baseline():
     """The reference's CPU path (nibble unpack -> bf16 group dequant -> bf16 torch.mm), restated in
-    oracle/torch_ref.py, on the host cores: the whole MLP step at 2048 tokens, fwd + dX."""
+    oracle/torch_ref.py, and the requant oracle (oracle/lq_oracle.c), on the host cores: the whole MLP
+    step at 2048 tokens (the headline workload), and bounded samples of the OPT-125m layer (fwd + dX),
+    the requantizer at its benchmark size and the decode shapes."""
+    import numpy as np
+    from oracle import c_oracle as co
     from oracle import torch_ref as tr
-    cores = min(os.cpu_count() or 1, 16)
+    from tests.util import bits
+    os_cores = os.cpu_count() or 1
+    cores = min(os_cores, 16)  # the box's share of the host; OMP_NUM_THREADS is set to the same there
     torch.set_num_threads(cores)
     gate = [t.cpu() for t in synth_w4(FFN, HID, 1, "cpu")] + [(FFN, HID)]
     up = [t.cpu() for t in synth_w4(FFN, HID, 2, "cpu")] + [(FFN, HID)]
@@ -370,16 +522,45 @@ def cpu_baseline():
         dx = dg.mm(tr.dequant_4bit_g(*gate)) + du.mm(tr.dequant_4bit_g(*up))
         return y, dx
 
-    step()  # warm-up (thread pool, allocator)
-    runs, t0 = 0, time.time()
-    while runs < 3 or (time.time() - t0 < 10.0 and runs < 10):
-        step()
-        runs += 1
-    sec = (time.time() - t0) / runs
-    return {"value": MLP_FLOP / sec / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": f"whole workload ({TOKENS} tokens, fwd + dX of the MLP block), 1 warm-up + {runs} timed runs, "
-                      f"torch {torch.__version__} CPU bf16 mm, {sec:.2f} s per step",
-            "cpu": _cpu_model()}
+    sec, runs = _cpu_time(step, 8.0, min_runs=3, max_runs=10)
+    out = {"value": MLP_FLOP / sec / 1e12, "unit": "TFLOP/s", "cores": cores, "os_cpu_count": os_cores,
+           "torch_num_threads": torch.get_num_threads(), "kind": "port",
+           "sample": f"whole workload ({TOKENS} tokens, fwd + dX of the MLP block), 1 warm-up + {runs} timed runs (median), "
+                     f"torch {torch.__version__} CPU bf16 mm, {sec:.2f} s per step",
+           "cpu": _cpu_model()}
+    # configs[0]: OPT-125m fc1 (3072 x 768) at 1024 tokens, forward + dX
+    N0, K0, M0 = 3072, 768, 1024
+    w0 = [t.cpu() for t in synth_w4(N0, K0, 5, "cpu")]
+    x0 = torch.randn(M0, K0, generator=g).to(torch.bfloat16)
+    dy0 = torch.randn(M0, N0, generator=g).to(torch.bfloat16)
+
+    def c0():
+        y = tr.w4_forward(x0, *w0, (N0, K0))
+        dx = dy0.mm(tr.dequant_4bit_g(*w0, (N0, K0)))
+        return y, dx
+    sec, runs = _cpu_time(c0, 2.0, min_runs=3)
+    out["c0"] = {"workload": "configs[0]: 3072x768 at 1024 tokens, fwd + dX", "TFLOP/s": 2 * 2 * M0 * N0 * K0 / sec / 1e12,
+                 "ms": sec * 1e3, "runs": runs}
+    # configs[1]: the requantizer at 8192 x 2048 (C oracle, OpenMP over the same cores)
+    N1, K1 = 8192, 2048
+    p1, s1, z1 = [t.cpu() for t in synth_w4(N1, K1, 10, "cpu")]
+    g1 = (torch.randn(N1, K1, generator=g) * 1e-3).to(torch.bfloat16)
+    a1 = (p1.numpy().view(np.uint8), bits(s1), bits(z1), bits(g1))
+    sec, runs = _cpu_time(lambda: co.requant(*a1, 1e-4, N1, K1, seed=7, offset=0), 3.0, min_runs=3)
+    nbytes = N1 * K1 // 2 * 2 + N1 * K1 * 2 + 4 * N1 * K1 // GROUP
+    out["c1"] = {"workload": "configs[1]: requant 8192x2048, Philox mode, C oracle", "GB/s": nbytes / sec / 1e9, "ms": sec * 1e3,
+                 "runs": runs, "omp_threads": os.environ.get("OMP_NUM_THREADS", "unset")}
+    # configs[4]: decode shapes, the reference's dequantise-then-mm path
+    c4 = []
+    for (N, K) in [(4096, 4096), (11008, 4096), (4096, 11008)]:
+        w = [t.cpu() for t in synth_w4(N, K, 20, "cpu")]
+        for M in (1, 4, 16):
+            xm = torch.randn(M, K, generator=g).to(torch.bfloat16)
+            sec, runs = _cpu_time(lambda: tr.w4_forward(xm, *w, (N, K)), 0.6, min_runs=1, max_runs=3)
+            nb = N * K // 2 + 4 * N * K // GROUP + 2 * M * K + 2 * M * N
+            c4.append({"N": N, "K": K, "M": M, "ms": sec * 1e3, "GB/s": nb / sec / 1e9})
+    out["c4"] = c4
+    return out
 
 
 def _cpu_model():
@@ -398,10 +579,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--settle-ms", type=float, default=150.0, help="untimed steps run for at least this long before the warm-up")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-mlp", action="store_true", help="skip the side measurements (requant, GEMV, A8W8)")
-    ap.add_argument("--profile-target", choices=["gemm", "requant", "gemv", "a8w8", "latent", "adam8"],
-                    help="run only a short fixed launch sequence of one kernel family (for rocprofv3), print nothing")
+    ap.add_argument("--profile-target", choices=["gemm", "requant", "gemv", "a8w8", "latent", "adam8", "gradq8", "ceiling"],
+                    help="run only a short fixed launch sequence of one kernel family (for rocprofv3); prints nothing except for 'ceiling'")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no sharding, no collectives); use --gpus 1")
@@ -417,6 +599,15 @@ def main():
         return
 
     blk = MLPBlock(dev)
+    # Settle the clock first: after an idle period the device takes tens of milliseconds of load to reach the
+    # clock it sustains (a step timed in the first milliseconds reads ~5-10 % low), so run untimed steps for
+    # at least --settle-ms, then the --warmup steps asked for.
+    t_settle = time.perf_counter()
+    while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
+        for _ in range(5):
+            blk.step()
+        torch.cuda.synchronize()
+    settle_ms = (time.perf_counter() - t_settle) * 1e3
     for _ in range(args.warmup):
         blk.step()
     torch.cuda.synchronize()
@@ -450,7 +641,7 @@ def main():
 
     line = {
         "metric": "A16W4 GEMM TFLOP/s (7B MLP, 2048 tok)", "value": value, "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3,
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_ms": settle_ms, "ms_per_step": dt * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[2]: A16W4 Llama-2-7B MLP block, 4x512=2048 bf16 tokens, forward + dX "
                                "through gate/up (11008x4096) and down (4096x11008), int4 group 128",
@@ -459,9 +650,15 @@ def main():
         "gemm_kernels": kern,
     }
     if not args.only_mlp:
+        ceil = bench_ceiling(dev, blk, h)
+        loop = ceil["mfma_loop_random_operands_2wg_per_cu"]["TFLOP/s"]
+        roofline["ceiling"] = {"what": "MFMA-only loop (lq_calib_mfma_loop), random bf16 operands, the forward kernel's 2 x 4 waves per compute unit",
+                               "TFLOP/s": loop, "achieved_over_ceiling": achieved / loop}
+        line["ceiling"] = ceil
         del blk
         torch.cuda.empty_cache()
         line["requant"] = bench_requant(dev)
+        line["gradq8"] = bench_gradq8(dev)
         line["latent_lbit4"] = bench_latent(dev)
         line["gemv"] = bench_gemv(dev)
         line["a8w8"] = bench_a8w8(dev)

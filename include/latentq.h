@@ -294,6 +294,25 @@ int lq_transpose_bf16(const void *src, void *dst, int64_t R, int64_t C, void *st
  * ------------------------------------------------------------------------- */
 int lq_calib_copy(const void *src, void *dst, int64_t nbytes, void *stream);
 
+/* Measurement aids for the GEMM's ceiling, no counterpart in the reference.
+ * lq_calib_mfma_loop: nothing but matrix instructions in the forward GEMM's shape: workgroups of 4
+ * waves (workgroups_per_cu = 1 or 2 per compute unit), each wave 8 accumulator tiles of 32 x 32 and the
+ * 8 MFMAs (32x32x16 bf16) of one reduction slice per iteration, operand fragments loaded once from
+ * a and b (bf16, n_elems each: zeros and random data draw different power). Every wave writes the
+ * shader-cycle counter at the start and end of its loop and the 100 MHz real-time counter at the same
+ * two points to clocks[4 w .. 4 w + 3] and a checksum to sink[w]; *waves receives the wave count
+ * (4 x workgroups). Work per wave: iters x 8 x 32768 flop.
+ * lq_calib_gemm_clocks: one lq_a16w4_fwd (backward = 0, bias-free) or lq_a16w4_dx (backward = 1)
+ * launch, M > 16, without workspace, in which every workgroup writes the same four counters at its
+ * start and end to clocks[4 g .. 4 g + 3]; *workgroups receives their number. Shader clock granted
+ * to a workgroup = (cycles end - start) / (real time end - start) x 100 MHz.
+ * ------------------------------------------------------------------------- */
+int lq_calib_mfma_loop(const void *a, const void *b, int64_t n_elems, int64_t iters, int workgroups_per_cu,
+                       uint64_t *clocks, int64_t clocks_capacity, float *sink, int64_t *waves, void *stream);
+int lq_calib_gemm_clocks(int backward, const void *a, const void *codes, const void *scales, const void *zeros,
+                         void *out, int64_t M, int64_t N, int64_t K, int group, uint64_t *clocks,
+                         int64_t clocks_capacity, int64_t *workgroups, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

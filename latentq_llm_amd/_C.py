@@ -35,6 +35,8 @@ SIGNATURES = {
     "lq_repack_gptq_to_native": [_vp, _vp, _i64, _i64, _vp],
     "lq_repack_native_to_gptq": [_vp, _vp, _i64, _i64, _vp],
     "lq_calib_copy": [_vp, _vp, _i64, _vp],
+    "lq_calib_mfma_loop": [_vp, _vp, _i64, _i64, _i32, _vp, _i64, _vp, _vp, _vp],
+    "lq_calib_gemm_clocks": [_i32, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp, _vp],
     "lq_transpose_bf16": [_vp, _vp, _i64, _i64, _vp],
     "lq_latent_w4_reconstruct": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],
     "lq_latent_w4_requant": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],

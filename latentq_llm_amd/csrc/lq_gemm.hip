@@ -67,6 +67,9 @@ struct GemmParams {
     // blockIdx.y * steps_per_split and writes its fp32 partial tile to partial[blockIdx.y][M][C]
     int steps_per_split;
     float *partial;
+    // measurement aid (null in normal use): workgroup w writes the shader-cycle counter and the
+    // 100 MHz real-time counter at its start and end to clk[4 w .. 4 w + 3]
+    unsigned long long *clk;
 };
 
 typedef __attribute__((address_space(3))) void lds_void;
@@ -130,6 +133,11 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
     // wave index as a scalar, so that the role split is a uniform branch and LDS-direct
     // destinations are wave-uniform
     const int wave_all = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    unsigned long long clk_t0 = 0, clk_r0 = 0;
+    if (p.clk) {
+        clk_t0 = __builtin_amdgcn_s_memtime();
+        clk_r0 = __builtin_amdgcn_s_memrealtime();
+    }
     const bool is_weight_wave = wave_all >= WM * WN;
     const int wave = wave_all % (WM * WN);
     const int lane = threadIdx.x & 63;
@@ -546,6 +554,10 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             if (mm < p.M && c_lane < p.C) *reinterpret_cast<u32x4_t *>(out + (long long)mm * p.C + c_lane) = o;
         }
     }
+    if (p.clk && threadIdx.x == 0) {
+        unsigned long long *c = p.clk + 4ll * (blockIdx.x + (long long)blockIdx.y * gridDim.x);
+        c[0] = clk_t0; c[1] = __builtin_amdgcn_s_memtime(); c[2] = clk_r0; c[3] = __builtin_amdgcn_s_memrealtime();
+    }
 }
 
 template <int MODE, int BM, int BN, int WM, int WN>
@@ -599,7 +611,7 @@ static bool small_tiles(const GemmParams &p) {
 // weights-direct forward GEMM (lq_gemm_fwd.hip)
 long long lq_gemm_fwd_direct_workgroups(int M, int N);
 int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
-                              void *y, int M, int N, int K, hipStream_t st);
+                              void *y, int M, int N, int K, hipStream_t st, unsigned long long *clk);
 
 // int8 GEMM with 256 x 256 tiles (lq_gemm_i8.hip)
 long long lq_gemm_i8_256_workgroups(int M, int N);
@@ -742,7 +754,7 @@ static int launch_split_reduce(const GemmParams &p, int splits, hipStream_t st, 
 
 static int a16w4_fwd_impl(const char *who, const void *x, const void *codes, const void *scales, const void *zeros,
                           const void *bias_or_null, void *y, int64_t M, int64_t N, int64_t K, int group, void *workspace,
-                          size_t ws_bytes, void *stream) {
+                          size_t ws_bytes, void *stream, unsigned long long *clk = nullptr) {
     int rc = check_w4_common(who, x, codes, scales, zeros, y, M, N, K, group);
     if (rc) return rc;
     LQ_REQUIRE(N % 16 == 0, "%s: N=%lld must be a multiple of 16", who, (long long)N);
@@ -761,8 +773,9 @@ static int a16w4_fwd_impl(const char *who, const void *x, const void *codes, con
         return LQ_OK;
     }
     if (plan.kernel == LQ_PLAN_DIRECT)
-        return lq_gemm_fwd_direct_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream);
+        return lq_gemm_fwd_direct_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream, clk);
     GemmParams p = {};
+    p.clk = clk;
     p.a = x; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.bias = (const unsigned short *)bias_or_null; p.c = y;
     p.M = (int)M; p.C = (int)N; p.R = (int)K; p.Kw = (int)K;
@@ -791,12 +804,13 @@ extern "C" int lq_a16w4_fwd_ws(const void *x, const void *codes, const void *sca
 
 static int a16w4_dx_impl(const char *who, const void *dy, const void *codes, const void *scales, const void *zeros,
                          void *dx, int64_t M, int64_t N, int64_t K, int group, void *workspace, size_t ws_bytes,
-                         void *stream) {
+                         void *stream, unsigned long long *clk = nullptr) {
     int rc = check_w4_common(who, dy, codes, scales, zeros, dx, M, N, K, group);
     if (rc) return rc;
     LQ_REQUIRE(N % 64 == 0, "%s: N=%lld must be a multiple of 64", who, (long long)N);
     LQ_REQUIRE(!workspace || lq_aligned(workspace, 16), "%s: the workspace must be 16-byte aligned", who);
     GemmParams p = {};
+    p.clk = clk;
     p.a = dy; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.c = dx;
     p.M = (int)M; p.C = (int)K; p.R = (int)N; p.Kw = (int)K;
@@ -850,6 +864,33 @@ extern "C" int lq_a16w4_fwd_static(const void *x, const void *codes, const void 
     }
     return a16w4_fwd_impl("lq_a16w4_fwd_static", x, codes, scales, zeros, bias_or_null, y, M, N, K, group, ws,
                           ws ? (size_t)LQ_STATIC_SCRATCH_BYTES : 0, stream);
+}
+
+// Measurement aid: lq_a16w4_fwd / lq_a16w4_dx with every workgroup recording its start and end on the
+// shader-cycle counter and on the 100 MHz real-time counter (4 values per workgroup).
+extern "C" int lq_calib_gemm_clocks(int backward, const void *a, const void *codes, const void *scales, const void *zeros,
+                                    void *out, int64_t M, int64_t N, int64_t K, int group, uint64_t *clocks,
+                                    int64_t clocks_capacity, int64_t *workgroups, void *stream) {
+    LQ_REQUIRE(clocks && workgroups && lq_aligned(clocks, 8), "lq_calib_gemm_clocks: clocks and workgroups must be given");
+    LQ_REQUIRE(M > 16, "lq_calib_gemm_clocks: needs M > 16 (the GEMM kernels)");
+    LQ_REQUIRE(N > 0 && K > 0 && K % LQ_GROUP == 0 && M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) &&
+                   (backward ? N % 64 == 0 : N % 16 == 0),
+               "lq_calib_gemm_clocks: bad shape");
+    const long long cus = lq_device_cu_count();
+    const W4Plan plan = backward ? plan_dx(M, N, K, 0, cus) : plan_fwd(M, N, K, 0, cus);
+    LQ_REQUIRE(plan.kernel != LQ_PLAN_GEMV_CHUNKS, "lq_calib_gemm_clocks: this shape runs as GEMV chunks");
+    const long long cols = backward ? K : N;
+    const long long wg = plan.kernel == LQ_PLAN_DIRECT ? lq_gemm_fwd_direct_workgroups((int)M, (int)N)
+                         : plan.kernel == LQ_PLAN_STAGED_256 ? ((M + 255) / 256) * ((cols + 127) / 128)
+                                                             : ((M + 127) / 128) * ((cols + 127) / 128);
+    LQ_REQUIRE(4 * wg <= clocks_capacity, "lq_calib_gemm_clocks: clocks must hold %lld values, holds %lld", 4 * wg,
+               (long long)clocks_capacity);
+    *workgroups = wg;
+    if (backward)
+        return a16w4_dx_impl("lq_calib_gemm_clocks", a, codes, scales, zeros, out, M, N, K, group, nullptr, 0, stream,
+                             (unsigned long long *)clocks);
+    return a16w4_fwd_impl("lq_calib_gemm_clocks", a, codes, scales, zeros, nullptr, out, M, N, K, group, nullptr, 0, stream,
+                          (unsigned long long *)clocks);
 }
 
 // The plan the two entry points above would follow, without launching anything.

@@ -57,6 +57,9 @@ struct FwdParams {
     unsigned short *y;           // bf16 [M, N]
     int M, N, K;
     int tiles_m, tiles_n;
+    // measurement aid (null in normal use): workgroup w writes the shader-cycle counter and the
+    // 100 MHz real-time counter at its start and end to clk[4 w .. 4 w + 3]
+    unsigned long long *clk;
 };
 
 typedef __attribute__((address_space(3))) void lds_void;
@@ -86,6 +89,11 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
     const int r = lane & 31, h = lane >> 5;
+    unsigned long long clk_t0 = 0, clk_r0 = 0;
+    if (p.clk) {
+        clk_t0 = __builtin_amdgcn_s_memtime();
+        clk_r0 = __builtin_amdgcn_s_memrealtime();
+    }
 
     // Workgroup ids are dealt round-robin over the 8 XCDs (id % 8): give each XCD a contiguous
     // range of the tile sequence, ordered in bands of GN tile columns walked row by row, so the
@@ -372,6 +380,10 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
             if (mm < p.M && c_lane < p.N) *reinterpret_cast<u32x4_t *>(p.y + (long long)mm * p.N + c_lane) = o;
         }
     }
+    if (p.clk && threadIdx.x == 0) {
+        unsigned long long *c = p.clk + 4ll * blockIdx.x;
+        c[0] = clk_t0; c[1] = __builtin_amdgcn_s_memtime(); c[2] = clk_r0; c[3] = __builtin_amdgcn_s_memrealtime();
+    }
 }
 
 }  // namespace
@@ -393,8 +405,9 @@ static int launch_direct(FwdParams p, hipStream_t st, const char *who) {
 
 // Called by lq_a16w4_fwd (lq_gemm.hip) after argument validation: K % 256 == 0, N % 16 == 0, M > 16.
 int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
-                              void *y, int M, int N, int K, hipStream_t st) {
+                              void *y, int M, int N, int K, hipStream_t st, unsigned long long *clk) {
     FwdParams p = {};
+    p.clk = clk;
     p.x = (const unsigned char *)x; p.w = (const unsigned char *)codes;
     p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.bias = (const unsigned short *)bias; p.y = (unsigned short *)y;

@@ -148,6 +148,65 @@ __global__ __launch_bounds__(256) void calib_copy_kernel(const u32x4_t *__restri
         __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
+// Measurement aid: nothing but matrix instructions, in the forward GEMM's shape. A workgroup is 4 waves
+// (one per SIMD), each holding 4 + 2 operand fragments loaded once from the caller's buffers and 8
+// accumulator tiles of 32 x 32; an iteration issues the 8 MFMAs (32x32x16 bf16) of one reduction
+// slice of that kernel. Every wave records the shader-cycle counter and the 100 MHz real-time
+// counter around its loop.
+__global__ __launch_bounds__(256, 2) void mfma_loop_kernel(const u32x4_t *__restrict__ a, const u32x4_t *__restrict__ b,
+                                                           long long n16, long long iters, unsigned long long *__restrict__ clk,
+                                                           float *__restrict__ sink) {
+    const int lane = threadIdx.x & 63;
+    const long long wv = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    u32x4_t af[4], bf[2];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) af[j] = a[((wv * 4 + j) * 64 + lane) % n16];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) bf[i] = b[((wv * 2 + i) * 64 + lane) % n16];
+    f32x16_t acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0;
+    const unsigned long long t0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+    for (long long it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[i]),
+                                                                   __builtin_bit_cast(bf16x8_t, af[j]), acc[i][j], 0, 0, 0);
+    }
+    const unsigned long long t1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) s += acc[i][j][q];
+    if (lane == 0) {
+        clk[4 * wv] = t0; clk[4 * wv + 1] = t1; clk[4 * wv + 2] = r0; clk[4 * wv + 3] = r1;
+        sink[wv] = s;
+    }
+}
+
+extern "C" int lq_calib_mfma_loop(const void *a, const void *b, int64_t n_elems, int64_t iters, int workgroups_per_cu,
+                                  uint64_t *clocks, int64_t clocks_capacity, float *sink, int64_t *waves, void *stream) {
+    LQ_REQUIRE(a && b && clocks && sink && waves, "lq_calib_mfma_loop: null pointer argument");
+    LQ_REQUIRE(n_elems >= 512 && n_elems % 8 == 0 && lq_aligned(a, 16) && lq_aligned(b, 16) && lq_aligned(clocks, 8),
+               "lq_calib_mfma_loop: operands need at least 512 elements, a multiple of 8, 16-byte aligned");
+    LQ_REQUIRE(iters > 0 && (workgroups_per_cu == 1 || workgroups_per_cu == 2), "lq_calib_mfma_loop: iters > 0, 1 or 2 workgroups per unit");
+    const long long wgs = (long long)lq_device_cu_count() * workgroups_per_cu;
+    LQ_REQUIRE(16 * wgs <= clocks_capacity, "lq_calib_mfma_loop: clocks must hold %lld values", 16 * wgs);
+    *waves = 4 * wgs;
+    hipLaunchKernelGGL(mfma_loop_kernel, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream, (const u32x4_t *)a,
+                       (const u32x4_t *)b, (long long)(n_elems / 8), (long long)iters, (unsigned long long *)clocks, sink);
+    return lq_check_launch("lq_calib_mfma_loop");
+}
+
 extern "C" int lq_calib_copy(const void *src, void *dst, int64_t nbytes, void *stream) {
     LQ_REQUIRE(src && dst, "lq_calib_copy: null pointer argument");
     LQ_REQUIRE(nbytes >= 0 && nbytes % 16 == 0, "lq_calib_copy: nbytes must be a non-negative multiple of 16");
