@@ -199,6 +199,16 @@ int lq_residual_quant(void *x_inout, int32_t *q_out, int64_t n_words, int mode, 
 int lq_residual_dequant(const int32_t *q, void *x_out, int64_t n_words, int mode, int k1, float b1, int k2,
                         float b2, int k3, void *stream);
 
+/* The reference's deterministic uniform quantiser, pybind name `uniform_quant_s`
+ * (utils/cuda_src/multi_random_quant.cpp:33-36, 48-50; kernel quant_kernel0,
+ * multi_random_quant_kernel.cu:219-239; launcher :376-381): level = roundf(float(x) * 8) with halves
+ * away from zero and no dither, nibble and carry as in lq_residual_quant, carries written back over
+ * x in x's own type. The reference dispatches it for fp32, fp16 and fp64 tensors (dtype 0, 1, 2; a
+ * double is converted to float first, as its kernel does); dtype 3 = bf16 is an addition. Nothing in the
+ * reference calls it. x_inout: 8 * n_words elements of that type, 16-byte aligned. Levels below -8
+ * (|x| > 1, undefined in the reference) store nibble 0. */
+int lq_residual_quant_s(void *x_inout, int32_t *q_out, int64_t n_words, int dtype, void *stream);
+
 /* ---------------------------------------------------------------------------
  * Fused latent-weight passes of the A16W4 layer in its 4-bit-residual mode (lbit = 4), three-segment
  * codec with the parameters of lq_residual_quant. Each is one pass instead of a chain of bf16

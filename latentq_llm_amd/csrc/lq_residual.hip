@@ -57,6 +57,44 @@ __global__ __launch_bounds__(256) void residual_dequant_kernel(const unsigned *_
     x[w] = out;
 }
 
+// Deterministic uniform quantiser (the reference's quant_kernel0): level = roundf(float(x) * 8), no dither.
+// T is the tensor's element type; a thread converts 8 consecutive elements and writes the carries back in T.
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static __device__ __forceinline__ float load(const float *p) { return *p; }
+    static __device__ __forceinline__ void store(float *p, float v) { *p = v; }
+};
+template <> struct Elem<double> {
+    static __device__ __forceinline__ float load(const double *p) { return (float)*p; }
+    static __device__ __forceinline__ void store(double *p, float v) { *p = (double)v; }
+};
+template <> struct Elem<_Float16> {
+    static __device__ __forceinline__ float load(const _Float16 *p) { return (float)*p; }
+    static __device__ __forceinline__ void store(_Float16 *p, float v) { *p = (_Float16)v; }
+};
+template <> struct Elem<unsigned short> {  // bf16 bit patterns
+    static __device__ __forceinline__ float load(const unsigned short *p) { return lq_bf16_bits_to_f32(*p); }
+    static __device__ __forceinline__ void store(unsigned short *p, float v) { *p = lq_f32_to_bf16_bits(v); }
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void residual_quant_s_kernel(T *__restrict__ x, unsigned *__restrict__ q, long long n_words) {
+    const long long w = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (w >= n_words) return;
+    struct alignas(8 * sizeof(T) > 16 ? 16 : 8 * sizeof(T)) Pack { T v[8]; };
+    Pack in = *reinterpret_cast<const Pack *>(x + 8 * w), out;
+    unsigned word = 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        bool carry;
+        const unsigned nib = nibble_of(roundf(Elem<T>::load(&in.v[k]) * 8.0f), carry);
+        word = (word << 4) | nib;
+        Elem<T>::store(&out.v[k], carry ? 1.0f : 0.0f);
+    }
+    q[w] = word;
+    *reinterpret_cast<Pack *>(x + 8 * w) = out;
+}
+
 int check(const char *who, const void *x, const void *q, int64_t n_words, int mode, int k1, float b1, int k2, float b2,
           int k3) {
     LQ_REQUIRE(x && q, "%s: null pointer argument", who);
@@ -85,6 +123,23 @@ extern "C" int lq_residual_quant(void *x_inout, int32_t *q_out, int64_t n_words,
         hipLaunchKernelGGL(residual_quant_kernel<1>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (u32x4_t *)x_inout,
                            (unsigned *)q_out, (long long)n_words, p);
     return lq_check_launch("lq_residual_quant");
+}
+
+extern "C" int lq_residual_quant_s(void *x_inout, int32_t *q_out, int64_t n_words, int dtype, void *stream) {
+    LQ_REQUIRE(x_inout && q_out, "lq_residual_quant_s: null pointer argument");
+    LQ_REQUIRE(n_words > 0 && n_words <= (0x7FFFFFFFll * 256), "lq_residual_quant_s: bad word count %lld", (long long)n_words);
+    LQ_REQUIRE(dtype >= 0 && dtype <= 3, "lq_residual_quant_s: dtype must be 0 (fp32), 1 (fp16), 2 (fp64) or 3 (bf16), got %d", dtype);
+    LQ_REQUIRE(lq_aligned(x_inout, 16) && lq_aligned(q_out, 4), "lq_residual_quant_s: x must be 16-byte and q 4-byte aligned");
+    const dim3 grid((unsigned)((n_words + 255) / 256)), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    unsigned *q = (unsigned *)q_out;
+    switch (dtype) {
+        case 0: hipLaunchKernelGGL(residual_quant_s_kernel<float>, grid, block, 0, st, (float *)x_inout, q, (long long)n_words); break;
+        case 1: hipLaunchKernelGGL(residual_quant_s_kernel<_Float16>, grid, block, 0, st, (_Float16 *)x_inout, q, (long long)n_words); break;
+        case 2: hipLaunchKernelGGL(residual_quant_s_kernel<double>, grid, block, 0, st, (double *)x_inout, q, (long long)n_words); break;
+        default: hipLaunchKernelGGL(residual_quant_s_kernel<unsigned short>, grid, block, 0, st, (unsigned short *)x_inout, q, (long long)n_words); break;
+    }
+    return lq_check_launch("lq_residual_quant_s");
 }
 
 extern "C" int lq_residual_dequant(const int32_t *q, void *x_out, int64_t n_words, int mode, int k1, float b1, int k2,

@@ -389,6 +389,22 @@ def residual_quant(x, q, mode: int, k1=0, b1=0.0, k2=0, b2=0.0, k3=0):
     return x
 
 
+_QUANT_S_DTYPES = {torch.float32: 0, torch.float16: 1, torch.float64: 2, torch.bfloat16: 3}
+
+
+def residual_quant_s(x, q):
+    """Deterministic uniform 4-bit quantiser (round(x * 8), no dither): packed words into q, carries over x."""
+    if x.dtype not in _QUANT_S_DTYPES:
+        raise TypeError(f"x must be float32, float16, float64 or bfloat16, got {x.dtype}")
+    _chk(x, x.dtype, "x")
+    _chk(q, torch.int32, "q")
+    if x.numel() != 8 * q.numel():
+        raise ValueError("x must have 8 elements per word of q")
+    with torch.cuda.device(x.device):
+        _C.call("lq_residual_quant_s", x.data_ptr(), q.data_ptr(), q.numel(), _QUANT_S_DTYPES[x.dtype], _stream(x))
+    return x
+
+
 def residual_dequant(q, mode: int, k1=0, b1=0.0, k2=0, b2=0.0, k3=0):
     """4-bit residual codec, dequantise: int32[n_words] -> bf16[n_words, 8]."""
     _chk(q, torch.int32, "q")

@@ -628,8 +628,8 @@ class _ResidualCodec(object):
 
     @staticmethod
     def uniform_quant_s(fp, q):
-        raise NotImplementedError("uniform_quant_s is not dispatched for bf16 in the reference either "
-                                  "(multi_random_quant_kernel.cu:376-381) and nothing calls it")
+        """multi_random_quant.cpp:33-36: fp32 / fp16 / fp64 as the reference dispatches it, bf16 in addition."""
+        ops.residual_quant_s(fp, q.view(-1))
 
     @staticmethod
     def uniform_dequant(q, fp):

@@ -190,6 +190,15 @@ def residual_quant(x_bits, mode, k1=0, b1=0.0, k2=0, b2=0.0, k3=0):
     return q, x
 
 
+def residual_quant_s(x_f32):
+    """Deterministic uniform quantiser on float32 values -> (words uint32[n/8], carries uint8[n])."""
+    x = _c(x_f32.reshape(-1), np.float32)
+    q = np.empty(x.size // 8, np.uint32)
+    carry = np.empty(x.size, np.uint8)
+    lib().lqo_residual_quant_s(_p(x), _p(q), _p(carry), C.c_int64(q.size))
+    return q, carry
+
+
 def residual_dequant(q, mode, k1=0, b1=0.0, k2=0, b2=0.0, k3=0):
     q = _c(q.reshape(-1).view(np.uint32), np.uint32)
     x = np.empty(q.size * 8, np.uint16)

@@ -450,6 +450,29 @@ void lqo_residual_quant(uint16_t *x, uint32_t *q, int64_t n_words, int mode, int
     }
 }
 
+/* Deterministic uniform quantiser, utils/cuda_src/multi_random_quant_kernel.cu:219-239 (quant_kernel0): the element
+ * is read into a float, level = roundf(x * 8), level > 7.5 stores nibble 1 and carry 1, otherwise nibble level + 8
+ * and carry 0. x: the elements already converted to float (the conversion of the tensor's type is the caller's);
+ * carry: 0 / 1 per element. */
+void lqo_residual_quant_s(const float *x, uint32_t *q, uint8_t *carry, int64_t n_words) {
+    for (int64_t w = 0; w < n_words; ++w) {
+        uint32_t word = 0;
+        for (int k = 0; k < 8; ++k) {
+            float lv = roundf(x[8 * w + k] * 8.0f);
+            word <<= 4;
+            if (lv > 7.5f) {
+                word += 1u;
+                carry[8 * w + k] = 1;
+            } else {
+                float t = lv + 8.0f;
+                word |= (t > 0.0f) ? ((uint32_t)t & 0xFu) : 0u;
+                carry[8 * w + k] = 0;
+            }
+        }
+        q[w] = word;
+    }
+}
+
 void lqo_residual_dequant(const uint32_t *q, uint16_t *x, int64_t n_words, int mode, int k1, float b1, int k2,
                           float b2, int k3) {
     float ic1 = 0, ic2 = 0, ic3 = 0;

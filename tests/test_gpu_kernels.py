@@ -196,6 +196,58 @@ def test_a16w4_fwd_gemv_many_tokens_staged_scales(ops, co, M, N, K):
     _fwd_case(ops, co, M, N, K, seed=M + N + K, with_bias=(M % 2 == 0))
 
 
+def test_gemv_and_gemm_agree_on_the_same_tokens_within_the_documented_bound(ops, co):
+    """Up to 16 tokens take the GEMV, which multiplies s * sum((q - z) x) in fp32; more tokens take kernels that
+    round the dequantised weight to bf16 first, as the reference does. The same token therefore gets slightly
+    different outputs depending on how many tokens ride along: at most 2^-9 relative per weight, i.e. well
+    inside the parity bar. Measured here between M = 16 (GEMV), M = 17 (GEMV chunks or GEMM) and M = 256 (GEMM)."""
+    N, K = 4096, 4096
+    codes, packed, scales, zeros = make_w4(N, K, 77)
+    x = randn_bf16((256, K), 78)
+    w = (dev(packed), dev(scales), dev(zeros))
+    xd = dev(x)
+    y16 = ops.a16w4_forward(xd[:16].contiguous(), *w, (N, K)).float()
+    y17 = ops.a16w4_forward(xd[:17].contiguous(), *w, (N, K)).float()[:16]
+    y256 = ops.a16w4_forward(xd, *w, (N, K)).float()[:16]
+    _, want64 = co.a16w4_fwd(bits(x[:16]), packed.numpy(), bits(scales), bits(zeros), None, 16, N, K, want_f64=True)
+    want = torch.from_numpy(want64)
+    for name, y in (("M=16", y16), ("M=17", y17), ("M=256", y256)):
+        print(f"{name}: rel_l2 vs float64 {rel_l2(y.cpu(), want):.3e}")
+    d = rel_l2(y16, y256)
+    print(f"GEMV(16) vs GEMM(256) on the same 16 tokens: rel_l2 {d:.3e}, max abs {float((y16 - y256).abs().max()):.3e}; "
+          f"M=17 vs M=256: {rel_l2(y17, y256):.3e}")
+    assert 0 < d <= 5e-3 and rel_l2(y17, y256) <= 5e-3
+    # the output scale is |y| ~ sqrt(K) * |w| ~ 0.1: no element moves by more than a few bf16 ulps of that
+    assert float((y16 - y256).abs().max()) <= 2.0 ** -7 * float(y256.abs().max())
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 640), (4, 4096, 4096), (16, 8192, 1536), (17, 16, 128), (300, 272, 512),
+                                   (2048, 512, 512)])
+def test_scales_and_zeros_need_only_2_byte_alignment(ops, co, M, N, K):
+    """Scales and zeros handed over at an address that is 2 bytes past a 256-byte boundary (a view into a larger
+    checkpoint tensor): forward (GEMV, staged and weights-direct GEMM), dX, dequant and the requantizer give
+    the same bits as with aligned copies."""
+    codes, packed, scales, zeros = make_w4(N, K, M + N + K)
+    x = dev(randn_bf16((M, K), 5))
+    dy = dev(randn_bf16((M, N), 6))
+    grad = dev(randn_bf16((N, K), 7, 1e-2))
+    G = N * K // 128
+    hold_s = torch.zeros(G + 1, 1, dtype=torch.bfloat16, device="cuda")
+    hold_z = torch.zeros(G + 1, 1, dtype=torch.bfloat16, device="cuda")
+    s_off, z_off = hold_s[1:], hold_z[1:]
+    s_off.copy_(scales)
+    z_off.copy_(zeros)
+    assert s_off.data_ptr() % 4 == 2 and z_off.data_ptr() % 4 == 2
+    p, s_al, z_al = dev(packed), dev(scales), dev(zeros)
+    assert torch.equal(ops.a16w4_forward(x, p, s_off, z_off, (N, K)), ops.a16w4_forward(x, p, s_al, z_al, (N, K)))
+    assert torch.equal(ops.a16w4_dequant(p, s_off, z_off, (N, K)), ops.a16w4_dequant(p, s_al, z_al, (N, K)))
+    if N % 64 == 0:
+        assert torch.equal(ops.a16w4_dx(dy, p, s_off, z_off, (N, K)), ops.a16w4_dx(dy, p, s_al, z_al, (N, K)))
+    a = ops.requant_sr(p, s_off, z_off, grad, 1e-2, (N, K), seed=3, offset=9)
+    b = ops.requant_sr(p, s_al, z_al, grad, 1e-2, (N, K), seed=3, offset=9)
+    assert torch.equal(a, b)
+
+
 def test_a16w4_fwd_identity_is_exact_dequant(ops, co):
     """X = identity: every output is a single dequantised weight, so the GEMM result must equal
     the reference dequantisation bit for bit (checks unpack + bf16 rounding through the kernel)."""

@@ -101,3 +101,27 @@ def test_optimizer_steps_fused_equals_unfused(hip_lib, monkeypatch):
         Q.FUSED_LATENT = True
     assert torch.equal(c1, c0) and torch.equal(r1, r0)
     assert not torch.equal(c1, make_w4(128, 256, 9)[1])  # the steps did move the weights
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.float64, torch.bfloat16])
+def test_deterministic_uniform_quantiser_bit_exact(dtype):
+    """cuda_module.uniform_quant_s (no dither) on every tensor type the reference dispatches it for, and on bf16:
+    words and carries equal the C restatement fed with the same values converted to float."""
+    from latentq_llm_amd import quant as Q
+    from oracle import c_oracle as co
+    g = torch.Generator().manual_seed(11)
+    n = 8 * 1000 + 8
+    x = (torch.rand(n, generator=g, dtype=torch.float64) * 2.2 - 1.1)
+    x[:9] = torch.tensor([0.0, 0.0625, -0.0625, 0.9375, 0.93749, -0.5, 0.5, 1.0, -1.0], dtype=torch.float64)
+    x = x.to(dtype)
+    want_q, want_c = co.residual_quant_s(x.to(torch.float32).numpy())
+    xd = x.cuda()
+    q = torch.empty(n // 8, dtype=torch.int32, device="cuda")
+    Q.cuda_module.uniform_quant_s(xd, q)
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy().view(np.uint32), want_q)
+    assert xd.dtype == dtype and np.array_equal(xd.cpu().to(torch.float32).numpy(), want_c.astype(np.float32))
+    # what the uniform dequantiser makes of the words is within half a step of the input where no carry was taken
+    deq = Q.cuda_dequant_linear(q).reshape(-1).float().cpu()
+    keep = (want_c == 0) & (x.abs().to(torch.float32).numpy() <= 1.0)
+    assert float((deq.numpy()[keep] - x.to(torch.float32).numpy()[keep]).__abs__().max()) <= 0.0625 + 1e-6

@@ -475,3 +475,24 @@ def test_residual_codec_against_an_exact_transcription_of_the_kernel(mu):
             moved.append(em.codec_level(x, cst, True) - base)
     moved = np.array(moved)
     assert np.abs(moved).max() <= 1 and (moved != 0).mean() > 0.1 and abs(moved.mean()) < 0.08, (moved.mean(),)
+
+
+def test_deterministic_uniform_quantiser_known_answers():
+    """quant_kernel0 (multi_random_quant_kernel.cu:219-239): level = round-half-away(x * 8); levels above 7.5
+    store nibble 1 and a carry, otherwise nibble level + 8. Known answers by hand, then every multiple of 1/64
+    in [-1, 1] against exact rational arithmetic."""
+    from fractions import Fraction
+    import math
+    x = np.array([0.0, 0.0625, -0.0625, 0.93, 0.9375, -0.5, 0.5, 0.124], np.float32)
+    q, carry = co.residual_quant_s(x)
+    #        0 -> 8   .5 -> 1 -> 9   -.5 -> -1 -> 7   7.44 -> 7 -> F   7.5 -> 8 -> carry   -4 -> 4   4 -> C   .992 -> 1 -> 9
+    assert int(q[0]) == 0x897F14C9 and list(carry) == [0, 0, 0, 0, 1, 0, 0, 0]
+    xs = np.arange(-64, 65, dtype=np.float32) / 64
+    xs = np.concatenate([xs, np.zeros((-len(xs)) % 8, np.float32)])
+    q, carry = co.residual_quant_s(xs)
+    nib = [(int(w) >> (28 - 4 * k)) & 0xF for w in q for k in range(8)]
+    for i, v in enumerate(xs):
+        t = Fraction(float(v)) * 8
+        lv = int(math.floor(abs(t) + Fraction(1, 2))) * (1 if t >= 0 else -1)
+        want = (1, 1) if lv > 7 else (lv + 8, 0)
+        assert (nib[i], int(carry[i])) == want, (float(v), lv)
