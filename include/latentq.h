@@ -270,10 +270,11 @@ int lq_adam8_latent_w4_step(const void *grad, void *codes, int32_t *residual, co
  *                                 is computed and written; x = dw
  *   accumulate != 0 (add_):       scale[n] is read; x = bf16(bf16(q * scale[n]) + dw)
  *   q[n,k] = clamp(rint(bf16(bf16(x / scale[n]) + noise[n,k])), -128, 127)        (written in place)
- * dw: bf16[N,K]; q_inout: int8[N,K]; scale_inout: bf16[N]; K % 8 == 0; dw and noise 16-byte aligned,
- * q 8-byte aligned. Noise: noise_or_null is a bf16[N,K] array (the reference draws it with
- * uniform_(-0.5, 0.5)), otherwise noise = bf16((a + 1/2) * 2^-16 - 1/2) with the 16-bit Philox draw a
- * of flat element n*K + k defined as for lq_requant_sr (N*K/8 counters per call).
+ * dw: bf16[N,K]; q_inout: int8[N,K]; scale_inout: bf16[N]; K % 16 == 0; dw, q and noise 16-byte
+ * aligned. Noise: noise_or_null is a bf16[N,K] array (the reference draws it with
+ * uniform_(-0.5, 0.5)), otherwise noise = (2b - 255) / 512 with the 8-bit Philox draw b of flat element
+ * i = n*K + k: byte i & 3 of word (i >> 2) & 3 of Philox4x32-10(counter = philox_offset + i / 16,
+ * key = philox_seed); a call consumes N*K/16 counters.
  * ------------------------------------------------------------------------- */
 int lq_gradq8_quant(const void *dw, int8_t *q_inout, void *scale_inout, int accumulate, int64_t N, int64_t K,
                     const void *noise_or_null, uint64_t philox_seed, uint64_t philox_offset, void *stream);

@@ -6,8 +6,9 @@
 //   add:  x = bf16(bf16(q * scale) + dW);   q = clamp(rint(bf16(bf16(x / scale) + noise)), -128, 127)
 // (a division by a Python scalar is a multiplication by its fp32 reciprocal inside the tensor
 // library's GPU kernels; tensor / tensor is the IEEE quotient). The reference draws the noise with
-// uniform_(-0.5, 0.5); here it is either injected (bf16) or bf16((a + 1/2) * 2^-16 - 1/2) for the
-// 16-bit Philox draw a of the element (the requantizer's stream: one block per 8 elements).
+// uniform_(-0.5, 0.5); here it is either injected (bf16) or (2b - 255) / 512 for the 8-bit Philox
+// draw b of the element: byte i & 3 of word (i >> 2) & 3 of Philox4x32-10(counter = offset + i / 16,
+// key = seed), i the flat element index. The 256 values are bf16 numbers, symmetric about zero.
 //
 // One workgroup per row: the row's absolute maximum needs the whole row before its first element can
 // be quantised, and a second read of an 8-22 KB row by the workgroup that just read it stays in L2.
@@ -17,34 +18,104 @@ namespace {
 
 __device__ __forceinline__ float bf16r(float v) { return lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(v)); }
 
-// IEEE x / s from the correctly rounded reciprocal r = RN(1/s) when fast (2^-40 <= s <= 2^40): q0 = x r,
-// e = x - q0 s exactly, q = q0 + e r; |x| is clamped to 2^60 first (the quotient then saturates the
-// int8 range anyway), a NaN takes the true division.
-__device__ __forceinline__ float div_by_scale(float x, float s, float r, bool fast) {
-    if (fast && x == x) {
-        const float xc = __builtin_amdgcn_fmed3f(x, -0x1p60f, 0x1p60f);
-        const float q0 = xc * r;
-        return fmaf(fmaf(-q0, s, xc), r, q0);
-    }
-    return x / s;
+// byte SEL of `old` replaced by sat_u8(rne(v)) (v_cvt_pk_u8_f32: saturates to 0..255, NaN -> 0)
+template <int SEL>
+__device__ __forceinline__ unsigned cvt_pk_u8(float v, unsigned old) {
+    unsigned r;
+    asm("v_cvt_pk_u8_f32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "n"(SEL), "v"(old));
+    return r;
 }
 
-template <bool kPhilox>
+__device__ __forceinline__ float bf16_of(const u32x4_t v, int j) { return (j & 1) ? lq_bf16_hi(v[j >> 1]) : lq_bf16_lo(v[j >> 1]); }
+
+// 16 consecutive elements (two 16-byte pieces of dW, 16 old int8, one Philox block or two pieces of noise).
+//
+// kFast (2^-40 <= s <= 2^40): only bf16(x / s) is needed, x and s are bf16 numbers, and the quotient of two
+// 8-bit significands is never closer than 2^-17 (relative) to a bf16 rounding tie (a tie has a 9-bit odd
+// significand t, and s t = x has no solution with x below 2^8), while x RN(1/s) is within 2^-23 of it: the
+// product rounds to the same bf16 number as the IEEE quotient. Where the quotient is a bf16 subnormal that
+// argument fails, and there the sum with the noise and the final code are the same for both anyway. Infinities
+// and NaN go the same way through the product as through the quotient.
+// clamp(rint(y), -128, 127) is taken as sat_u8(rne(y + 128)) - 128: y is a bf16 number, so y + 128 is exact
+// in fp32 whenever |y| >= 2^-8, below that both forms give 0, and ties keep their parity. NaN -> -128.
+template <bool kPhilox, bool kAcc, bool kFast>
+__device__ __forceinline__ u32x4_t quant16(const u32x4_t v0, const u32x4_t v1, const u32x4_t old, const u32x4_t n0,
+                                           const u32x4_t n1, float s, float r, unsigned long long counter,
+                                           unsigned long long seed) {
+    unsigned w[4] = {0u, 0u, 0u, 0u};
+    if (kPhilox) {
+        const lq_u4 A = lq_philox4x32_10((unsigned)counter, (unsigned)(counter >> 32), 0u, 0u, (unsigned)seed,
+                                         (unsigned)(seed >> 32));
+        w[0] = A.x; w[1] = A.y; w[2] = A.z; w[3] = A.w;
+    }
+    unsigned o[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        float x = j < 8 ? bf16_of(v0, j) : bf16_of(v1, j - 8);
+        if (kAcc) {
+            const int qi = (int)(signed char)((old[j >> 2] >> (8 * (j & 3))) & 0xFFu);
+            x = bf16r(bf16r((float)qi * s) + x);
+        }
+        float nz;
+        if (kPhilox) nz = fmaf((float)((w[j >> 2] >> (8 * (j & 3))) & 0xFFu), 0x1p-8f, 0x1p-9f - 0.5f);  // (2b - 255) / 512
+        else nz = j < 8 ? bf16_of(n0, j) : bf16_of(n1, j - 8);
+        const float q = kFast ? x * r : x / s;
+        const float y = bf16r(bf16r(q) + nz) + 128.0f;
+        switch (j & 3) {
+            case 0: o[j >> 2] = cvt_pk_u8<0>(y, o[j >> 2]); break;
+            case 1: o[j >> 2] = cvt_pk_u8<1>(y, o[j >> 2]); break;
+            case 2: o[j >> 2] = cvt_pk_u8<2>(y, o[j >> 2]); break;
+            default: o[j >> 2] = cvt_pk_u8<3>(y, o[j >> 2]); break;
+        }
+    }
+    return u32x4_t{o[0] ^ 0x80808080u, o[1] ^ 0x80808080u, o[2] ^ 0x80808080u, o[3] ^ 0x80808080u};
+}
+
+__device__ __forceinline__ float absmax8(const u32x4_t v, float m) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) m = fmaxf(m, fmaxf(fabsf(lq_bf16_lo(v[j])), fabsf(lq_bf16_hi(v[j]))));
+    return m;
+}
+
+// One workgroup per row, a thread takes 16 consecutive elements per step of 4096. kPieces > 0: the row has at
+// most kPieces * 4096 elements and a thread keeps its pieces in registers between the maximum and the
+// quantisation; 0: any K, the row is read a second time (from L2).
+template <bool kPhilox, bool kAcc, int kPieces>
 __global__ __launch_bounds__(256) void gradq8_kernel(const unsigned short *__restrict__ dw, signed char *__restrict__ q,
                                                      unsigned short *__restrict__ scale, const unsigned short *__restrict__ noise,
-                                                     int accumulate, long long K, unsigned long long seed,
-                                                     unsigned long long offset) {
+                                                     long long K, unsigned long long seed, unsigned long long offset) {
     __shared__ float red[4];
     const long long n = blockIdx.x;
     const unsigned short *row = dw + n * K;
     const int tid = threadIdx.x;
-    float s;
-    if (!accumulate) {
-        float m = 0.0f;
-        for (long long k = (long long)tid * 8; k < K; k += 256 * 8) {
-            const u32x4_t v = *reinterpret_cast<const u32x4_t *>(row + k);
+    const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+    constexpr int kHeld = kPieces > 0 ? kPieces : 1;
+    u32x4_t h0[kHeld], h1[kHeld], old[kHeld], z0[kHeld], z1[kHeld];
+    if (kPieces > 0) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) m = fmaxf(m, fmaxf(fabsf(lq_bf16_lo(v[j])), fabsf(lq_bf16_hi(v[j]))));
+        for (int i = 0; i < kPieces; ++i) {
+            const long long k = (long long)tid * 16 + (long long)i * 4096;
+            h0[i] = h1[i] = old[i] = z0[i] = z1[i] = zero4;
+            if (k < K) {
+                h0[i] = *reinterpret_cast<const u32x4_t *>(row + k);
+                h1[i] = *reinterpret_cast<const u32x4_t *>(row + k + 8);
+                if (kAcc) old[i] = *reinterpret_cast<const u32x4_t *>(q + n * K + k);
+                if (!kPhilox) {
+                    z0[i] = *reinterpret_cast<const u32x4_t *>(noise + n * K + k);
+                    z1[i] = *reinterpret_cast<const u32x4_t *>(noise + n * K + k + 8);
+                }
+            }
+        }
+    }
+    float s;
+    if (!kAcc) {
+        float m = 0.0f;
+        if (kPieces > 0) {
+#pragma unroll
+            for (int i = 0; i < kPieces; ++i) m = absmax8(h1[i], absmax8(h0[i], m));
+        } else {
+            for (long long k = (long long)tid * 16; k < K; k += 4096)
+                m = absmax8(*reinterpret_cast<const u32x4_t *>(row + k + 8), absmax8(*reinterpret_cast<const u32x4_t *>(row + k), m));
         }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
@@ -58,44 +129,52 @@ __global__ __launch_bounds__(256) void gradq8_kernel(const unsigned short *__res
     } else {
         s = lq_bf16_bits_to_f32(scale[n]);
     }
-    const bool fast = s >= 0x1p-40f && s <= 0x1p40f;
+    // the scale is the same for the whole workgroup, so this branch does not diverge
+    const bool fast = __builtin_amdgcn_readfirstlane((int)(s >= 0x1p-40f && s <= 0x1p40f)) != 0;
     const float r = 1.0f / s;
-    for (long long k = (long long)tid * 8; k < K; k += 256 * 8) {
-        const long long e0 = n * K + k;  // flat index of the first of 8 elements
-        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(row + k);
-        float x[8];
+    if (kPieces > 0) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) x[j] = (j & 1) ? lq_bf16_hi(v[j >> 1]) : lq_bf16_lo(v[j >> 1]);
-        if (accumulate) {
-            const u32x2_t old = *reinterpret_cast<const u32x2_t *>(q + e0);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int qi = (int)(signed char)((old[j >> 2] >> (8 * (j & 3))) & 0xFFu);
-                x[j] = bf16r(bf16r((float)qi * s) + x[j]);
+        for (int i = 0; i < kPieces; ++i) {
+            const long long k = (long long)tid * 16 + (long long)i * 4096;
+            if (k < K) {
+                const long long e0 = n * K + k;
+                const unsigned long long c = offset + (unsigned long long)(e0 >> 4);
+                const u32x4_t o = fast ? quant16<kPhilox, kAcc, true>(h0[i], h1[i], old[i], z0[i], z1[i], s, r, c, seed)
+                                       : quant16<kPhilox, kAcc, false>(h0[i], h1[i], old[i], z0[i], z1[i], s, r, c, seed);
+                *reinterpret_cast<u32x4_t *>(q + e0) = o;
             }
         }
-        float nz[8];
-        if (kPhilox) {
-            const unsigned long long c = offset + (unsigned long long)(e0 >> 3);
-            const lq_u4 A = lq_philox4x32_10((unsigned)c, (unsigned)(c >> 32), 0u, 0u, (unsigned)seed, (unsigned)(seed >> 32));
-            const unsigned w[4] = {A.x, A.y, A.z, A.w};
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                nz[j] = bf16r(((float)((w[j >> 1] >> (16 * (j & 1))) & 0xFFFFu) + 0.5f) * 0x1p-16f - 0.5f);
-        } else {
-            const u32x4_t nv = *reinterpret_cast<const u32x4_t *>(noise + e0);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) nz[j] = (j & 1) ? lq_bf16_hi(nv[j >> 1]) : lq_bf16_lo(nv[j >> 1]);
+    } else {
+        for (long long k = (long long)tid * 16; k < K; k += 4096) {
+            const long long e0 = n * K + k;
+            const u32x4_t v0 = *reinterpret_cast<const u32x4_t *>(row + k);
+            const u32x4_t v1 = *reinterpret_cast<const u32x4_t *>(row + k + 8);
+            u32x4_t ol = zero4, a0 = zero4, a1 = zero4;
+            if (kAcc) ol = *reinterpret_cast<const u32x4_t *>(q + e0);
+            if (!kPhilox) {
+                a0 = *reinterpret_cast<const u32x4_t *>(noise + e0);
+                a1 = *reinterpret_cast<const u32x4_t *>(noise + e0 + 8);
+            }
+            const unsigned long long c = offset + (unsigned long long)(e0 >> 4);
+            const u32x4_t o = fast ? quant16<kPhilox, kAcc, true>(v0, v1, ol, a0, a1, s, r, c, seed)
+                                   : quant16<kPhilox, kAcc, false>(v0, v1, ol, a0, a1, s, r, c, seed);
+            *reinterpret_cast<u32x4_t *>(q + e0) = o;
         }
-        unsigned o[2] = {0u, 0u};
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float y = bf16r(bf16r(div_by_scale(x[j], s, r, fast)) + nz[j]);
-            const float c = __builtin_amdgcn_fmed3f(rintf(y), -128.0f, 127.0f);  // NaN -> -128
-            o[j >> 2] |= ((unsigned)(int)c & 0xFFu) << (8 * (j & 3));
-        }
-        *reinterpret_cast<u32x2_t *>(q + e0) = u32x2_t{o[0], o[1]};
     }
+}
+
+template <bool kPhilox, bool kAcc>
+void launch_gradq8(const void *dw, int8_t *q, void *scale, const void *noise, int64_t N, int64_t K, uint64_t seed,
+                   uint64_t offset, hipStream_t st) {
+    const dim3 grid((unsigned)N), block(256);
+#define LQ_GRADQ8_LAUNCH(P)                                                                                         \
+    hipLaunchKernelGGL((gradq8_kernel<kPhilox, kAcc, P>), grid, block, 0, st, (const unsigned short *)dw,           \
+                       (signed char *)q, (unsigned short *)scale, (const unsigned short *)noise, (long long)K,      \
+                       (unsigned long long)seed, (unsigned long long)offset)
+    if (K <= 4096) LQ_GRADQ8_LAUNCH(1);
+    else if (K <= 3 * 4096) LQ_GRADQ8_LAUNCH(3);
+    else LQ_GRADQ8_LAUNCH(0);
+#undef LQ_GRADQ8_LAUNCH
 }
 
 }  // namespace
@@ -103,19 +182,18 @@ __global__ __launch_bounds__(256) void gradq8_kernel(const unsigned short *__res
 extern "C" int lq_gradq8_quant(const void *dw, int8_t *q_inout, void *scale_inout, int accumulate, int64_t N, int64_t K,
                                const void *noise_or_null, uint64_t philox_seed, uint64_t philox_offset, void *stream) {
     LQ_REQUIRE(dw && q_inout && scale_inout, "lq_gradq8_quant: null pointer argument");
-    LQ_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && N < (1ll << 31), "lq_gradq8_quant: need N > 0 and K a positive multiple of 8 (N=%lld K=%lld)",
+    LQ_REQUIRE(N > 0 && K > 0 && K % 16 == 0 && N < (1ll << 31), "lq_gradq8_quant: need N > 0 and K a positive multiple of 16 (N=%lld K=%lld)",
                (long long)N, (long long)K);
-    LQ_REQUIRE(lq_aligned(dw, 16) && lq_aligned(q_inout, 8) && lq_aligned(scale_inout, 2) &&
+    LQ_REQUIRE(lq_aligned(dw, 16) && lq_aligned(q_inout, 16) && lq_aligned(scale_inout, 2) &&
                    (!noise_or_null || lq_aligned(noise_or_null, 16)),
-               "lq_gradq8_quant: dw and noise need 16-byte alignment, q 8-byte alignment");
-    const dim3 grid((unsigned)N), block(256);
-    if (noise_or_null)
-        hipLaunchKernelGGL((gradq8_kernel<false>), grid, block, 0, (hipStream_t)stream, (const unsigned short *)dw,
-                           (signed char *)q_inout, (unsigned short *)scale_inout, (const unsigned short *)noise_or_null,
-                           accumulate, (long long)K, 0ull, 0ull);
-    else
-        hipLaunchKernelGGL((gradq8_kernel<true>), grid, block, 0, (hipStream_t)stream, (const unsigned short *)dw,
-                           (signed char *)q_inout, (unsigned short *)scale_inout, (const unsigned short *)nullptr, accumulate,
-                           (long long)K, (unsigned long long)philox_seed, (unsigned long long)philox_offset);
+               "lq_gradq8_quant: dw, q and noise need 16-byte alignment");
+    hipStream_t st = (hipStream_t)stream;
+    if (noise_or_null) {
+        if (accumulate) launch_gradq8<false, true>(dw, q_inout, scale_inout, noise_or_null, N, K, 0, 0, st);
+        else launch_gradq8<false, false>(dw, q_inout, scale_inout, noise_or_null, N, K, 0, 0, st);
+    } else {
+        if (accumulate) launch_gradq8<true, true>(dw, q_inout, scale_inout, nullptr, N, K, philox_seed, philox_offset, st);
+        else launch_gradq8<true, false>(dw, q_inout, scale_inout, nullptr, N, K, philox_seed, philox_offset, st);
+    }
     return lq_check_launch("lq_gradq8_quant");
 }

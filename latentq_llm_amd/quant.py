@@ -777,7 +777,7 @@ class GradientQTensor(object):
 
     def _hip_ok(self, fdata):
         return (FUSED_GRADQ and self.bit == 8 and fdata.is_cuda and fdata.dtype == torch.bfloat16 and fdata.dim() == 2
-                and fdata.is_contiguous() and fdata.shape[1] % 8 == 0 and fdata.data_ptr() % 16 == 0)
+                and fdata.is_contiguous() and fdata.shape[1] % 16 == 0 and fdata.data_ptr() % 16 == 0)
 
     def _hip_quant(self, fdata, accumulate, noise):
         cls = GradientQTensor
@@ -786,7 +786,7 @@ class GradientQTensor(object):
             self.scale = torch.empty((fdata.shape[0], 1), dtype=torch.bfloat16, device=fdata.device)
         ops.gradq8_quant(fdata, self.qdata, self.scale, accumulate, noise=noise, seed=cls.noise_seed, offset=cls._noise_offset)
         if noise is None:
-            cls._noise_offset += (fdata.numel() + 7) // 8
+            cls._noise_offset += (fdata.numel() + 15) // 16
 
     def quant(self, fdata, noise=None):
         if noise is None:

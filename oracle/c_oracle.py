@@ -129,6 +129,13 @@ def requant(packed, scales, zeros, grad, lr, N, K, group=128, u=None, seed=0, of
     return out
 
 
+def gradq8_noise(n, seed, offset=0):
+    """The noise lqo_gradq8 draws for flat elements 0..n-1 when none is injected (float32)."""
+    out = np.empty(n, np.float32)
+    lib().lqo_gradq8_noise(_p(out), C.c_int64(n), C.c_uint64(seed), C.c_uint64(offset))
+    return out
+
+
 def gradq8(dw, q, scale, accumulate, N, K, noise=None, seed=0, offset=0):
     """GradientQTensor (bit = 8) set_value / add_: returns (new int8 q [N*K], bf16 scale bits [N]).
     dw, noise: bf16 bit patterns; q: int8 or None (set); scale: bf16 bits or None (set)."""

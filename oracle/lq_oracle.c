@@ -178,6 +178,23 @@ static inline uint32_t philox_draw16(int64_t i, uint64_t seed, uint64_t offset) 
     return (o[(i >> 1) & 3] >> (16 * (i & 1))) & 0xFFFFu;
 }
 
+/* 8-bit draw of flat element i (gradient accumulator): byte i & 3 of word (i >> 2) & 3 of the block
+ * Philox4x32-10(counter = offset + i / 16, key = seed). */
+static inline uint32_t philox_draw8(int64_t i, uint64_t seed, uint64_t offset) {
+    uint64_t c = offset + (uint64_t)(i >> 4);
+    uint32_t ctr[4] = {(uint32_t)c, (uint32_t)(c >> 32), 0u, 0u};
+    uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    uint32_t o[4];
+    lqo_philox4x32_10(ctr, key, o);
+    return (o[(i >> 2) & 3] >> (8 * (i & 3))) & 0xFFu;
+}
+
+/* The noise the gradient accumulator adds for element i when none is injected: (2b - 255) / 512 for the 8-bit
+ * draw b, i.e. 256 equally spaced bf16 numbers symmetric about zero, as fp32. */
+void lqo_gradq8_noise(float *out, int64_t n, uint64_t seed, uint64_t offset) {
+    for (int64_t i = 0; i < n; ++i) out[i] = (2.0f * (float)philox_draw8(i, seed, offset) - 255.0f) / 512.0f;
+}
+
 /* The uniform the requantizer adds for element i: (a + 1/2) * 2^-16, on the centred 2^-16 grid. */
 void lqo_philox_uniform(float *out, int64_t n, uint64_t seed, uint64_t offset) {
 #pragma omp parallel for schedule(static)
@@ -303,7 +320,7 @@ void lqo_native_to_gptq(const uint8_t *packed, int32_t *qweight, int64_t N, int6
  *   dequant    :873-875  qdata.to(bf16) * scale
  *   set_value  :877-885  find_param(fdata); quant(fdata)
  *   add_       :891-898  quant(dequant() + fdata)
- * noise == NULL: noise = bf16((a + 1/2) * 2^-16 - 1/2) with the requantizer's 16-bit Philox draw a. */
+ * noise == NULL: noise = (2b - 255) / 512 with the element's 8-bit Philox draw b (lqo_gradq8_noise). */
 void lqo_gradq8(const uint16_t *dw, int8_t *q, uint16_t *scale, int accumulate, int64_t N, int64_t K,
                 const uint16_t *noise, uint64_t seed, uint64_t offset) {
 #pragma omp parallel for schedule(static)
@@ -328,7 +345,7 @@ void lqo_gradq8(const uint16_t *dw, int8_t *q, uint16_t *scale, int accumulate, 
             float x = bf16_to_f32(dw[i]);
             if (accumulate) x = bf16_round(bf16_round((float)q[i] * s) + x);
             float nz = noise ? bf16_to_f32(noise[i])
-                             : bf16_round(((float)philox_draw16(i, seed, offset) + 0.5f) * 0x1p-16f - 0.5f);
+                             : (2.0f * (float)philox_draw8(i, seed, offset) - 255.0f) / 512.0f;
             volatile float quo = x / s;
             float y = bf16_round(bf16_round(quo) + nz);
             float r = nearbyintf(y);

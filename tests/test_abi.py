@@ -96,7 +96,7 @@ def test_header_divisibility_constraints_are_the_ones_enforced(hip_lib):
     lib = hip_lib
     cons = header_divisibility_constraints()
     assert cons["lq_a16w4_fwd"] == {"K": 128, "N": 16} and cons["lq_a16w4_dx"] == {"K": 128, "N": 64}
-    assert cons["lq_a8w8_fwd"] == {"K": 128, "N": 16} and cons["lq_gradq8_quant"] == {"K": 8}
+    assert cons["lq_a8w8_fwd"] == {"K": 128, "N": 16} and cons["lq_gradq8_quant"] == {"K": 16}
     buf = (C.c_char * 4096)()
     p = C.cast(buf, C.c_void_p)
 

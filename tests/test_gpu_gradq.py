@@ -33,7 +33,8 @@ def _noise(shape, seed):
     return (torch.rand(shape, generator=torch.Generator().manual_seed(seed)) - 0.5).to(torch.bfloat16)
 
 
-@pytest.mark.parametrize("N,K,std", [(1, 8, 1.0), (7, 136, 1e-3), (33, 2048, 0.02), (16, 4104, 5.0), (4, 11008, 1e-6)])
+@pytest.mark.parametrize("N,K,std", [(1, 16, 1.0), (7, 144, 1e-3), (33, 2048, 0.02), (16, 4112, 5.0), (4, 11008, 1e-6),
+                                     (3, 12304, 0.3)])
 @pytest.mark.parametrize("mode", ["inject", "philox"])
 def test_gradq8_set_and_add_bit_exact(ops, N, K, std, mode):
     dws = [randn_bf16((N, K), 50 + i, std) for i in range(3)]
@@ -51,6 +52,39 @@ def test_gradq8_set_and_add_bit_exact(ops, N, K, std, mode):
         assert np.array_equal(bits(s).reshape(-1), want_s), f"scales differ at micro-batch {i}"
         mism = int((q.cpu().numpy().reshape(-1) != want_q).sum())
         assert mism == 0, f"{mism} of {N * K} int8 values differ at micro-batch {i}"
+
+
+@pytest.mark.parametrize("mode", ["inject", "philox"])
+def test_gradq8_edge_values_and_scales(ops, mode):
+    """NaN, infinities and huge or tiny magnitudes in dW; scales outside the range in which the kernel replaces the
+    division (2^-40 .. 2^40), given to the accumulate form by hand and produced by a row of 1e20-sized values."""
+    N, K = 8, 4112
+    dw = randn_bf16((N, K), 70, 0.05)
+    dw[0, 5] = float("nan")
+    dw[1, 6] = float("inf")
+    dw[1, 7] = float("-inf")
+    dw[2] *= 1e20
+    dw[3] *= 1e-30
+    dw[4, 100] = 3e38
+    dw[5, 9] = -1e-38
+    kw_o = {"noise": bits(_noise((N, K), 71))} if mode == "inject" else {"seed": 9, "offset": 2 ** 40}
+    kw_h = {"noise": _noise((N, K), 71).cuda()} if mode == "inject" else {"seed": 9, "offset": 2 ** 40}
+    q = torch.empty((N, K), dtype=torch.int8, device="cuda")
+    s = torch.empty((N, 1), dtype=torch.bfloat16, device="cuda")
+    want_q, want_s = co.gradq8(bits(dw), None, None, False, N, K, **kw_o)
+    ops.gradq8_quant(dw.cuda(), q, s, False, **kw_h)
+    assert np.array_equal(bits(s).reshape(-1), want_s)
+    assert np.array_equal(q.cpu().numpy().reshape(-1), want_q)
+    # accumulate onto hand-made state with scales from 2^-60 to 2^60
+    g = torch.Generator().manual_seed(72)
+    q0 = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+    s0 = torch.tensor([2.0 ** e for e in (-60, -41, -40, -1, 7, 40, 41, 60)], dtype=torch.bfloat16).reshape(N, 1)
+    dw2 = randn_bf16((N, K), 73, 1.0) * s0.float().to(torch.bfloat16) * 30
+    want_q, want_s = co.gradq8(bits(dw2), q0.numpy().reshape(-1).copy(), bits(s0).reshape(-1).copy(), True, N, K, **kw_o)
+    qd, sd = q0.cuda(), s0.cuda()
+    ops.gradq8_quant(dw2.cuda(), qd, sd, True, **kw_h)
+    assert np.array_equal(bits(sd).reshape(-1), want_s)
+    assert np.array_equal(qd.cpu().numpy().reshape(-1), want_q)
 
 
 def test_gradq8_module_path_equals_the_tensor_op_chain_on_the_gpu(Q):
@@ -87,7 +121,7 @@ def test_gradq8_philox_rounding_is_unbiased(ops):
     acc = torch.zeros((N, K), device="cuda")
     reps = 300
     for r in range(reps):
-        ops.gradq8_quant(dw, q, s, False, seed=1234, offset=r * (N * K // 8))
+        ops.gradq8_quant(dw, q, s, False, seed=1234, offset=r * (N * K // 16))
         acc += q.float() * s.float()
     err = (acc / reps - dw.float()).abs() / s.float()
     assert float(err.max()) < 0.2  # in units of a quantisation step; a biased rounding would sit near 0.5
@@ -121,7 +155,7 @@ def test_qlinear_a16w4_with_8bit_gradient_accumulation(Q):
         assert got.dtype == torch.bfloat16
         # each micro-batch adds at most one rounding step (|noise| <= 1/2 plus the bf16 roundings)
         assert float(((got.float() - want).abs() / g.scale.float()).max()) <= 1.5 * (i + 1)
-    assert Q.GradientQTensor._noise_offset == used0 + 2 * (N * K // 8)
+    assert Q.GradientQTensor._noise_offset == used0 + 2 * (N * K // 16)
     assert rel_l2(g.get_value().float(), want) < 0.05
     # the optimizer consumes the dequantised value and resets the accumulator
     opt = Q.MyAdam([{"params": [m.weight], "weight_decay": 0.0}], lr=1e-3, betas=(0.9, 0.95), obit=8)

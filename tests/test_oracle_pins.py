@@ -410,17 +410,57 @@ def test_gradq8_oracle_matches_torch_bf16_tensor_ops(N, K, std):
     assert np.abs(q.astype(int)).max() <= 128 and (q != 0).mean() > 0.5
 
 
-def test_gradq8_philox_noise_is_the_requantizer_stream():
-    """Without injected noise element i draws bf16((a_i + 1/2) / 65536 - 1/2) from the stream that
-    lqo_philox_uniform materialises; the noise is centred and reaches +-0.5 only after rounding."""
+def test_gradq8_philox_noise_definition():
+    """Without injected noise element i draws (2 b_i - 255) / 512, b_i = byte i & 3 of word (i >> 2) & 3 of the
+    Philox block with counter offset + i / 16 (recomputed here from the pinned block function): 256 equally
+    spaced bf16 numbers, symmetric about zero; the oracle's result equals the one with that noise injected."""
     N, K, seed, off = 4, 128, 99, 3
+    nz = co.gradq8_noise(N * K, seed, off)
+    for i in (0, 1, 3, 4, 15, 16, 17, 200, 511):
+        c = off + i // 16
+        blk = co.philox4x32_10([c & 0xFFFFFFFF, c >> 32, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
+        b = (int(blk[(i >> 2) & 3]) >> (8 * (i & 3))) & 0xFF
+        assert float(nz[i]) == (2 * b - 255) / 512
+    noise = torch.from_numpy(nz).to(torch.bfloat16)
+    assert np.array_equal(noise.float().numpy(), nz)  # every value is a bf16 number
     dw = randn_bf16((N, K), 1, 0.01)
-    u = co.philox_uniform(N * K, seed, off)
-    noise = torch.from_numpy(u - np.float32(0.5)).to(torch.bfloat16)
     a, sa = co.gradq8(bits(dw), None, None, False, N, K, seed=seed, offset=off)
     b, sb = co.gradq8(bits(dw), None, None, False, N, K, noise=bits(noise))
     assert np.array_equal(a, b) and np.array_equal(sa, sb)
-    assert float(noise.float().abs().max()) <= 0.5 and abs(float(noise.float().mean())) < 0.05
+    big = co.gradq8_noise(1 << 16, 7, 0)
+    assert float(np.abs(big).max()) == 255 / 512 and abs(float(big.mean())) < 0.005 and len(np.unique(big)) == 256
+
+
+def test_bf16_quotient_of_bf16_numbers_from_the_reciprocal_product():
+    """The gradient accumulator needs bf16(x / s) for bf16 numbers x and s and takes bf16(fl(x * RN(1/s))).
+    Every pair of 8-bit significands (the exponents only shift the result): the product rounds to the same bf16
+    number as the exact quotient, and the exact quotient keeps a relative distance of at least 2^-17 from
+    every bf16 rounding tie, far more than the product's error of at most 2^-23."""
+    from fractions import Fraction
+    xs = np.arange(128, 256, dtype=np.float32)
+    for e in (-20, 0, 13):
+        S, X = np.meshgrid(xs * np.float32(2.0 ** e), xs, indexing="ij")
+        r = (np.float32(1.0) / S).astype(np.float32)  # correctly rounded
+        prod = (X * r).astype(np.float32)
+        quo = (X.astype(np.float64) / S.astype(np.float64))  # 8-bit / 8-bit: the double is within 2^-53 of exact
+        def bf16_rne(a32):
+            u = a32.astype(np.float32).view(np.uint32).astype(np.uint64)
+            return (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) & 0xFFFF).astype(np.uint16)
+        assert np.array_equal(bf16_rne(prod), bf16_rne(quo.astype(np.float32)))
+    worst = 1.0
+    for x in range(128, 256):
+        for s_ in range(128, 256):
+            qv = Fraction(x, s_)
+            while qv < 256:
+                qv *= 2
+            while qv >= 512:
+                qv /= 2
+            # qv in [256, 512): bf16 ties are the odd integers here (9 significant bits)
+            lo = (qv.numerator // qv.denominator)
+            for t in (lo, lo + 1):
+                if t % 2 == 1:
+                    worst = min(worst, abs(qv - t) / qv)
+    assert worst >= Fraction(1, 2 ** 17), float(worst)
 
 
 # ------------------------------------------------------------- 4-bit residual codec --
