@@ -386,6 +386,24 @@ def bench_ceiling(device, blk, h):
     return out
 
 
+def bench_gate_up(device, blk):
+    """silu(gate(x)) * up(x) of the 7B MLP as one launch (lq_a16w4_gate_up_silu, the inference-side fused product)
+    against the same result from two forward GEMMs and torch's bf16 silu and product, over the token count."""
+    from latentq_llm_amd import ops
+    out = []
+    for M in (256, 512, 1024, 2048, 4096):
+        g = torch.Generator(device="cpu").manual_seed(40 + M)
+        x = torch.randn(M, HID, generator=g).to(torch.bfloat16).to(device)
+        h = torch.empty((M, FFN), dtype=torch.bfloat16, device=device)
+        t_fused = event_time(lambda: ops.a16w4_gate_up_silu(x, blk.gate, blk.up, (FFN, HID), out=h), 30)
+        t_parts = event_time(lambda: torch.nn.functional.silu(ops.a16w4_forward(x, *blk.gate, (FFN, HID)))
+                             * ops.a16w4_forward(x, *blk.up, (FFN, HID)), 30)
+        flop = 4.0 * M * HID * FFN
+        out.append({"M": M, "fused_us": t_fused * 1e6, "fused_TFLOP/s": flop / t_fused / 1e12,
+                    "two_gemms_silu_mul_us": t_parts * 1e6, "two_gemms_silu_mul_TFLOP/s": flop / t_parts / 1e12})
+    return out
+
+
 def bench_copy(device):
     """Plain streaming copy (lq_calib_copy) over buffers larger than the last-level cache: the
     HBM rate this device sustains for read + write traffic, for comparison with the 8 TB/s peak."""
@@ -634,7 +652,7 @@ def main():
     tot = 2 * kern["fwd_gate_up"]["us"] + kern["fwd_down"]["us"] + 2 * kern["dx_gate_up"]["us"] + kern["dx_down"]["us"]
     avg_us = tot / 6
     achieved = 2 * TOKENS * HID * FFN / (avg_us * 1e-6) / 1e12
-    roofline = {"bound": "mfma", "kernel": "A16W4 dequant-GEMM: gemm_fwd_direct_kernel (forward), gemm_kernel<1> (dX)",
+    roofline = {"bound": "mfma", "kernel": "A16W4 dequant-GEMM: gemm_fwd_direct_kernel<false> (forward), gemm_kernel<1> (dX)",
                 "achieved": achieved, "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": achieved * 1e12 / PEAK_BF16,
                 "avg_launch_us": avg_us, "flop_per_launch": 2 * TOKENS * HID * FFN, "traffic": gemm_traffic_bytes(),
                 "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated on a copy)"}
@@ -659,6 +677,7 @@ def main():
         torch.cuda.empty_cache()
         line["requant"] = bench_requant(dev)
         line["gradq8"] = bench_gradq8(dev)
+        line["gate_up_silu"] = bench_gate_up(dev, blk)
         line["latent_lbit4"] = bench_latent(dev)
         line["gemv"] = bench_gemv(dev)
         line["a8w8"] = bench_a8w8(dev)

@@ -136,6 +136,18 @@ int lq_a16w4_fwd_static(const void *x, const void *codes, const void *scales, co
                         const void *bias_or_null, void *y, int64_t M, int64_t N, int64_t K, int group,
                         void *stream);
 
+/* Gate / up pair of a gated MLP in one launch: h[M,N] = silu(X . deq(Wgate)^T) * (X . deq(Wup)^T) with
+ * silu(v) = v / (1 + exp(-v)), both products accumulated in fp32 and the result rounded to bf16 once.
+ * Replaces the fused product of the reference's GPTQ-side MLP (PTQ/quant/fused_mlp.py:85-168,
+ * fusedmatmul_248_kernel: "C = silu(A * B1) * (A * B2)", called from QuantLlamaMLP.triton_llama_mlp
+ * :206-218), on the native code layout. Neither product is rounded on its own, so h differs from
+ * running lq_a16w4_fwd twice and multiplying in bf16 by the roundings that path adds.
+ * Both matrices [N,K] with their own scales and zeros; no bias. K % 256 == 0; N % 16 == 0; M > 16
+ * (LQ_ERR_BAD_ARG otherwise: a caller with fewer tokens runs the two products through lq_a16w4_fwd). */
+int lq_a16w4_gate_up_silu(const void *x, const void *codes_gate, const void *scales_gate, const void *zeros_gate,
+                          const void *codes_up, const void *scales_up, const void *zeros_up, void *h, int64_t M,
+                          int64_t N, int64_t K, int group, void *stream);
+
 /* Which kernel lq_a16w4_fwd(_ws) (backward = 0) or lq_a16w4_dx(_ws) (backward = 1) would run for a
  * shape and a workspace size, and how it would cut the reduction; launches nothing. *kernel is
  * one of LQ_PLAN_*; *splits > 1 means a split reduction of *steps_per_split 64-deep steps per slice

@@ -612,6 +612,9 @@ static bool small_tiles(const GemmParams &p) {
 long long lq_gemm_fwd_direct_workgroups(int M, int N);
 int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
                               void *y, int M, int N, int K, hipStream_t st, unsigned long long *clk);
+int lq_gemm_fwd_gate_up_launch(const void *x, const void *codes_g, const void *scales_g, const void *zeros_g,
+                               const void *codes_u, const void *scales_u, const void *zeros_u, void *h, int M, int N, int K,
+                               hipStream_t st);
 
 // int8 GEMM with 256 x 256 tiles (lq_gemm_i8.hip)
 long long lq_gemm_i8_256_workgroups(int M, int N);
@@ -787,6 +790,22 @@ static int a16w4_fwd_impl(const char *who, const void *x, const void *codes, con
                                            : launch_gemm<MODE_W4_FWD, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
     if (rc || plan.splits < 2) return rc;
     return launch_split_reduce(p, plan.splits, (hipStream_t)stream, who);
+}
+
+extern "C" int lq_a16w4_gate_up_silu(const void *x, const void *codes_gate, const void *scales_gate, const void *zeros_gate,
+                                     const void *codes_up, const void *scales_up, const void *zeros_up, void *h, int64_t M,
+                                     int64_t N, int64_t K, int group, void *stream) {
+    const char *who = "lq_a16w4_gate_up_silu";
+    int rc = check_w4_common(who, x, codes_gate, scales_gate, zeros_gate, h, M, N, K, group);
+    if (rc) return rc;
+    rc = check_w4_common(who, x, codes_up, scales_up, zeros_up, h, M, N, K, group);
+    if (rc) return rc;
+    LQ_REQUIRE(N % 16 == 0, "%s: N=%lld must be a multiple of 16", who, (long long)N);
+    LQ_REQUIRE(K % 256 == 0, "%s: K=%lld must be a multiple of 256", who, (long long)K);
+    LQ_REQUIRE(M > 16, "%s: needs more than 16 tokens (M=%lld); below that run the two products through lq_a16w4_fwd", who,
+               (long long)M);
+    return lq_gemm_fwd_gate_up_launch(x, codes_gate, scales_gate, zeros_gate, codes_up, scales_up, zeros_up, h, (int)M, (int)N,
+                                      (int)K, (hipStream_t)stream);
 }
 
 extern "C" int lq_a16w4_fwd(const void *x, const void *codes, const void *scales, const void *zeros,

@@ -1,5 +1,9 @@
 // Weights-direct forward GEMM for gfx950:
 //   A16W4, M > 16:  Y[M,N] = X[M,K] . deq(W)[N,K]^T (+ bias), bf16 MFMA
+//   and, from the same loop, H[M,N] = silu(X . deq(Wg)^T) * (X . deq(Wu)^T) for the gate / up pair of a
+//   gated MLP (the fused product of the reference's PTQ/quant/fused_mlp.py:85-168): a wave's two column
+//   tiles then are the same 32 output columns of the two matrices, and the product is formed on the fp32
+//   accumulators in the epilogue.
 //
 // The weights never pass through LDS. An MFMA B-side lane needs 8 consecutive k of one weight
 // row, and 8 consecutive k of a row are exactly one 32-bit word of packed codes: every lane
@@ -54,6 +58,10 @@ struct FwdParams {
     const unsigned short *scales;
     const unsigned short *zeros;
     const unsigned short *bias;  // bf16 [N] or null
+    // gate / up mode: the second matrix (w, scales, zeros are the gate's; no bias)
+    const unsigned char *w2;
+    const unsigned short *scales2;
+    const unsigned short *zeros2;
     unsigned short *y;           // bf16 [M, N]
     int M, N, K;
     int tiles_m, tiles_n;
@@ -71,7 +79,12 @@ constexpr int BM = 128, BN = 256;
 constexpr int ROWB = 128;            // bytes of A per tile row and step: 64 bf16
 constexpr int STAGE = BM * ROWB;     // 16 KB per A stage
 
+// GU: gate / up mode. The workgroup then covers 128 output columns (both matrices' rows c0 .. c0 + 127)
+// instead of 256.
+template <bool GU>
 __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
+    constexpr int BNO = GU ? BN / 2 : BN;  // output columns per workgroup
+    constexpr int WN = BNO / 4;            // output columns per wave
     constexpr int ESZ = 2;    // bytes per A element
     constexpr int WROW = 32;  // bytes of one weight row consumed per step
     // 16-byte weight loads per lane and column tile in one batch: the pieces of two consecutive
@@ -110,7 +123,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     const int rest = p.tiles_n - band * GN;
     const int bw = rest < GN ? rest : GN;
     const int tile_m = within / bw, tile_n = band * GN + within % bw;
-    const int m0 = tile_m * BM, c0 = tile_n * BN;
+    const int m0 = tile_m * BM, c0 = tile_n * BNO;
     const int nk = p.K * ESZ / ROWB;
     const long long lda = (long long)p.K * ESZ;
 
@@ -145,20 +158,24 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     // ---- B: buffer descriptors over this workgroup's weight rows (rows past N read as zero), the
     // lane's two rows as 32-bit offsets, the reduction step as the scalar offset
     const int groups_per_row = p.K / LQ_GROUP;
-    const int rows_here = p.N - c0 < BN ? p.N - c0 : BN;
+    const int rows_here = p.N - c0 < BNO ? p.N - c0 : BNO;
     auto make_rsrc = [](const void *base, unsigned bytes) {
         const unsigned long long a = (unsigned long long)base;
         u32x4_t d = {(unsigned)a, (unsigned)(a >> 32) & 0xFFFFu, bytes, 0x00020000u};
         return d;
     };
     const unsigned wpitch = (unsigned)(p.K / 2);  // bytes per weight row
-    const u32x4_t w_rsrc = make_rsrc(p.w + (long long)c0 * wpitch, (unsigned)rows_here * wpitch);
-    const u32x4_t s_rsrc = make_rsrc(p.scales + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u);
-    const u32x4_t z_rsrc = make_rsrc(p.zeros + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u);
+    const u32x4_t w_rsrc0 = make_rsrc(p.w + (long long)c0 * wpitch, (unsigned)rows_here * wpitch);
+    const u32x4_t s_rsrc0 = make_rsrc(p.scales + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u);
+    const u32x4_t z_rsrc0 = make_rsrc(p.zeros + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u);
+    // column tile 1 reads the second matrix in gate / up mode, the same one otherwise
+    const u32x4_t w_rsrc1 = GU ? make_rsrc(p.w2 + (long long)c0 * wpitch, (unsigned)rows_here * wpitch) : w_rsrc0;
+    const u32x4_t s_rsrc1 = GU ? make_rsrc(p.scales2 + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u) : s_rsrc0;
+    const u32x4_t z_rsrc1 = GU ? make_rsrc(p.zeros2 + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u) : z_rsrc0;
     unsigned w_off[2], q_off[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        const unsigned n = wave * 64 + i * 32 + r;
+        const unsigned n = GU ? wave * 32 + r : wave * 64 + i * 32 + r;
         w_off[i] = n * wpitch + h * (WROW / 2);
         q_off[i] = n * (unsigned)groups_per_row * 2u;
     }
@@ -181,6 +198,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     u32x2_t qs[2], qz[2];
     float s[2], nzs[2];
     auto load_codes_one = [&](int kt, u32x4_t (*c)[NB], int i) {
+        const u32x4_t w_rsrc = i == 0 ? w_rsrc0 : w_rsrc1;
         asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(c[i][0]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
         asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:32" : "=v"(c[i][1]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
     };
@@ -191,6 +209,8 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     // Called on the even step two steps before group g starts; loads when g opens a quad.
     auto load_qparams_one = [&](int g, int i) {
         if ((g & 3) != 0) return;
+        const u32x4_t s_rsrc = i == 0 ? s_rsrc0 : s_rsrc1;
+        const u32x4_t z_rsrc = i == 0 ? z_rsrc0 : z_rsrc1;
         asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "=v"(qs[i]) : "v"(q_off[i]), "s"(s_rsrc), "s"(g * 2));
         asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "=v"(qz[i]) : "v"(q_off[i]), "s"(z_rsrc), "s"(g * 2));
     };
@@ -332,6 +352,38 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     // the clamped prefetches of the last two steps are still writing LDS: drain them
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
+    __syncthreads();
+    if constexpr (GU) {
+        // ---- gate / up epilogue: acc[0] and acc[1] hold the same output element of the two products,
+        // column c0 + 32*wave + 8*(q/4) + 4h + q%4, row m0 + 32j + r. H = silu(gate) * up on the fp32
+        // accumulators, rounded once. A wave's 32 rows x 32 columns pass through LDS (row pitch 80
+        // bytes) and leave as 16 bytes per lane, 4 lanes on the 64 contiguous bytes of a row.
+        constexpr int EP = 80;
+        unsigned char *ep = ((wave & 2) ? lds_a1 : lds_a0) + (wave & 1) * (32 * EP);
+        const int ep_row = lane >> 2, ep_chunk = lane & 3;
+        const int c_lane = c0 + wave * WN + ep_chunk * 8;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float g = acc[0][j][4 * q + e];
+                    v[e] = g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * acc[1][j][4 * q + e];
+                }
+                u32x2_t o = {lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3])};
+                *reinterpret_cast<u32x2_t *>(ep + r * EP + (8 * q + 4 * h) * 2) = o;
+            }
+#pragma unroll
+            for (int it = 0; it < 2; ++it) {
+                const int row = it * 16 + ep_row;
+                const u32x4_t o = *reinterpret_cast<const u32x4_t *>(ep + row * EP + ep_chunk * 16);
+                const int mm = m0 + j * 32 + row;
+                if (mm < p.M && c_lane < p.N) *reinterpret_cast<u32x4_t *>(p.y + (long long)mm * p.N + c_lane) = o;
+            }
+        }
+    } else {
     // ---- epilogue: acc[i][j][q]: column c0 + 64*wave + 32i + 8*(q/4) + 4h + q%4, row m0 + 32j + r.
     // A lane holds 4 consecutive columns of one row: stored straight from the registers, an
     // instruction would touch 32 rows with 16 bytes each. Instead every wave passes its block
@@ -339,7 +391,6 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     // contiguous bytes of a row: full cache lines. The stages are free once every wave has left the
     // loop and its loads have landed; a wave's staging area is private (waves 0,1 in stage 0, waves
     // 2,3 in stage 1), row pitch 144 bytes.
-    __syncthreads();
     constexpr int EP = 144;
     unsigned char *ep = ((wave & 2) ? lds_a1 : lds_a0) + (wave & 1) * (32 * EP);
     const int ep_row = lane >> 3, ep_chunk = lane & 7;
@@ -380,6 +431,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
             if (mm < p.M && c_lane < p.N) *reinterpret_cast<u32x4_t *>(p.y + (long long)mm * p.N + c_lane) = o;
         }
     }
+    }
     if (p.clk && threadIdx.x == 0) {
         unsigned long long *c = p.clk + 4ll * blockIdx.x;
         c[0] = clk_t0; c[1] = __builtin_amdgcn_s_memtime(); c[2] = clk_r0; c[3] = __builtin_amdgcn_s_memrealtime();
@@ -392,14 +444,16 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
 // can fill the device two per CU.
 long long lq_gemm_fwd_direct_workgroups(int M, int N) { return (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN); }
 
+template <bool GU>
 static int launch_direct(FwdParams p, hipStream_t st, const char *who) {
+    constexpr int BNO = GU ? BN / 2 : BN;
     p.tiles_m = (p.M + BM - 1) / BM;
-    p.tiles_n = (p.N + BN - 1) / BN;
+    p.tiles_n = (p.N + BNO - 1) / BNO;
     const long long nwg = (long long)p.tiles_m * p.tiles_n;
     if (nwg > 0x7FFFFFFFll) return lq_fail(LQ_ERR_BAD_ARG, "%s: problem too large", who);
     // the 32-bit lane offsets of the activation and weight loads span 128 / 256 rows
     if ((long long)BN * p.K * 2 >= (1ll << 32)) return lq_fail(LQ_ERR_BAD_ARG, "%s: K too large", who);
-    hipLaunchKernelGGL(gemm_fwd_direct_kernel, dim3((unsigned)nwg), dim3(256), 0, st, p);
+    hipLaunchKernelGGL(gemm_fwd_direct_kernel<GU>, dim3((unsigned)nwg), dim3(256), 0, st, p);
     return lq_check_launch(who);
 }
 
@@ -412,5 +466,18 @@ int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scal
     p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.bias = (const unsigned short *)bias; p.y = (unsigned short *)y;
     p.M = M; p.N = N; p.K = K;
-    return launch_direct(p, st, "lq_a16w4_fwd");
+    return launch_direct<false>(p, st, "lq_a16w4_fwd");
+}
+
+// Called by lq_a16w4_gate_up_silu (lq_gemm.hip) after argument validation: K % 256 == 0, N % 16 == 0, M > 16.
+int lq_gemm_fwd_gate_up_launch(const void *x, const void *codes_g, const void *scales_g, const void *zeros_g,
+                               const void *codes_u, const void *scales_u, const void *zeros_u, void *h, int M, int N, int K,
+                               hipStream_t st) {
+    FwdParams p = {};
+    p.x = (const unsigned char *)x;
+    p.w = (const unsigned char *)codes_g; p.scales = (const unsigned short *)scales_g; p.zeros = (const unsigned short *)zeros_g;
+    p.w2 = (const unsigned char *)codes_u; p.scales2 = (const unsigned short *)scales_u; p.zeros2 = (const unsigned short *)zeros_u;
+    p.y = (unsigned short *)h;
+    p.M = M; p.N = N; p.K = K;
+    return launch_direct<true>(p, st, "lq_a16w4_gate_up_silu");
 }

@@ -1,0 +1,70 @@
+"""Gated MLP with the gate / up products and the SiLU product in one launch.
+
+Mirrors the reference's GPTQ-side ``QuantLlamaMLP`` / ``make_fused_mlp`` (PTQ/quant/fused_mlp.py:177-254)
+for this package's ``QLinearA16W4`` layers (native code layout): ``forward`` is
+``down_proj(silu(gate_proj(x)) * up_proj(x))`` with the first three operations done by
+``lq_a16w4_gate_up_silu`` on fp32 accumulators, as the reference's Triton kernel does (:160-166).
+Inference only, like the reference's: no backward is defined through the fused product.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from . import ops
+
+# Below this many tokens the two products go through the ordinary forward (GEMV, GEMV chunks or the split
+# reduction, whichever the library picks) and the SiLU product is formed on their bf16 results: the fused
+# kernel's 128-row tiles would be mostly empty (on the 7B matrices it takes 51 us from 17 to 192 tokens, the
+# composed path 44 us at 17 tokens, 54 at 64, 84 at 192).
+FUSED_MIN_TOKENS = 64
+
+
+def _w4(layer):
+    return (layer.weight.data, layer.scales, layer.zeros)
+
+
+class QuantLlamaMLP(nn.Module):
+    """PTQ/quant/fused_mlp.py:177-218 on QLinearA16W4 layers: keeps the three projections as submodules (their
+    buffers stay where checkpoints expect them) and fuses gate / up / SiLU in ``forward``."""
+
+    def __init__(self, gate_proj, down_proj, up_proj):
+        super().__init__()
+        if tuple(gate_proj.wshape) != tuple(up_proj.wshape):
+            raise ValueError("gate_proj and up_proj must have the same shape")
+        if gate_proj.bias is not None or up_proj.bias is not None:
+            raise ValueError("the fused gate / up product takes no bias")
+        self.gate_proj, self.down_proj, self.up_proj = gate_proj, down_proj, up_proj
+        self.intermediate_size, self.infeatures = int(gate_proj.wshape[0]), int(gate_proj.wshape[1])
+        self.outfeatures = int(down_proj.wshape[0])
+
+    def forward(self, x):
+        return self.down_proj(self.fused_gate_up(x))
+
+    def fused_gate_up(self, x):
+        """silu(gate_proj(x)) * up_proj(x), shape x.shape[:-1] + (intermediate_size,)."""
+        out_shape = x.shape[:-1] + (self.intermediate_size,)
+        x2 = x.reshape(-1, x.shape[-1])
+        M, K = x2.shape
+        if M >= FUSED_MIN_TOKENS and K % 256 == 0 and x2.dtype == torch.bfloat16:
+            if not x2.is_contiguous():
+                x2 = x2.contiguous()
+            h = ops.a16w4_gate_up_silu(x2, _w4(self.gate_proj), _w4(self.up_proj), (self.intermediate_size, K))
+        else:
+            h = torch.nn.functional.silu(self.gate_proj.forward_eval(x2)) * self.up_proj.forward_eval(x2)
+        return h.reshape(out_shape)
+
+
+def make_fused_mlp(m, parent_name=""):
+    """Replace every gated MLP (a module with QLinearA16W4 children named gate_proj, up_proj and down_proj, e.g.
+    transformers' LlamaMLP after the layer swap of main0.py:300-343) by a QuantLlamaMLP
+    (PTQ/quant/fused_mlp.py:241-254)."""
+    from .quant import QLinearA16W4
+    kids = dict(m.named_children())
+    if all(isinstance(kids.get(k), QLinearA16W4) for k in ("gate_proj", "up_proj", "down_proj")) and not isinstance(m, QuantLlamaMLP):
+        return QuantLlamaMLP(m.gate_proj, m.down_proj, m.up_proj)
+    for name, child in m.named_children():
+        new = make_fused_mlp(child, parent_name=f"{parent_name}.{name}")
+        if new is not child:
+            setattr(m, name, new)
+    return m

@@ -160,6 +160,29 @@ def a16w4_forward_static(x, codes, scales, zeros, shape, out, bias=None):
     return out
 
 
+def a16w4_gate_up_silu(x, gate, up, shape, out=None):
+    """h[M,N] = silu(X . deq(Wgate)^T) * (X . deq(Wup)^T) in one launch (lq_a16w4_gate_up_silu); gate and up are
+    (codes, scales, zeros) triples of two [N, K] matrices. Needs M > 16 and K % 256 == 0."""
+    N, K = shape
+    _chk(x, torch.bfloat16, "x")
+    if x.dim() != 2 or x.shape[1] != K:
+        raise ValueError(f"x must be [M,{K}], got {tuple(x.shape)}")
+    for w in (gate, up):
+        _codes_ok(w[0], N, K)
+        _qparam_ok(w[1], w[2], N, K)
+    M = x.shape[0]
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    else:
+        _chk(out, torch.bfloat16, "out")
+        if tuple(out.shape) != (M, N):
+            raise ValueError(f"out must be [{M},{N}]")
+    with torch.cuda.device(x.device):
+        _C.call("lq_a16w4_gate_up_silu", x.data_ptr(), gate[0].data_ptr(), gate[1].data_ptr(), gate[2].data_ptr(),
+                up[0].data_ptr(), up[1].data_ptr(), up[2].data_ptr(), out.data_ptr(), M, N, K, GROUP, _stream(x))
+    return out
+
+
 def a16w4_dx(dy, codes, scales, zeros, shape, out=None):
     """dX[M,K] = dY[M,N] . deq(W)[N,K]."""
     N, K = shape

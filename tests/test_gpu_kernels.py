@@ -477,3 +477,106 @@ def test_workspace_smaller_than_wanted_is_used_as_far_as_it_goes(ops, slices):
     assert rel_l2(out.float().cpu(), ref.float().cpu()) < 4e-3
     if slices < 2:
         assert torch.equal(out, ref)  # no room for a split: the same kernel as the plain entry point
+
+
+# ------------------------------------------------------ fused gate / up / SiLU product --
+def _gate_up_case(ops, co, M, N, K, seed):
+    _, pg, sg, zg = make_w4(N, K, seed)
+    _, pu, su, zu = make_w4(N, K, seed + 1)
+    x = randn_bf16((M, K), seed + 2)
+    _, g64 = co.a16w4_fwd(bits(x), pg.numpy(), bits(sg), bits(zg), None, M, N, K, want_f64=True)
+    _, u64 = co.a16w4_fwd(bits(x), pu.numpy(), bits(su), bits(zu), None, M, N, K, want_f64=True)
+    g64, u64 = torch.from_numpy(g64), torch.from_numpy(u64)
+    want = g64 / (1 + torch.exp(-g64)) * u64
+    gate, up = (dev(pg), dev(sg), dev(zg)), (dev(pu), dev(su), dev(zu))
+    xd = dev(x)
+    got = ops.a16w4_gate_up_silu(xd, gate, up, (N, K))
+    torch.cuda.synchronize()
+    err = rel_l2(got.float().cpu(), want)
+    # the same product from two ordinary forwards and bf16 tensor operations (two more roundings)
+    unfused = torch.nn.functional.silu(ops.a16w4_forward(xd, *gate, (N, K))) * ops.a16w4_forward(xd, *up, (N, K))
+    err_unfused = rel_l2(unfused.float().cpu(), want)
+    print(f"gate/up M={M} N={N} K={K}: fused rel_l2={err:.3e}, two forwards + bf16 silu*mul rel_l2={err_unfused:.3e}")
+    assert err <= REL_L2_TOL and err <= err_unfused * 1.05
+    assert rel_l2(got.float(), unfused.float()) <= REL_L2_TOL
+    return got
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 16, 256), (128, 128, 256), (130, 272, 512), (300, 400, 768), (1000, 1040, 1280),
+                                   (2048, 11008, 4096)])
+def test_a16w4_gate_up_silu(ops, co, M, N, K):
+    """silu(X Wg^T) * (X Wu^T) in one launch against float64, ragged in M and N (N = 16: one partial tile; 272,
+    400, 1040: a partial last tile of 16 columns), 4..20 reduction steps, and the benchmark's shape."""
+    if N * K > 2 ** 24:
+        # the float64 oracle on the full matrix takes minutes: check a band of tokens against it instead
+        _, pg, sg, zg = make_w4(N, K, 5)
+        _, pu, su, zu = make_w4(N, K, 6)
+        x = randn_bf16((M, K), 7)
+        got = ops.a16w4_gate_up_silu(dev(x), (dev(pg), dev(sg), dev(zg)), (dev(pu), dev(su), dev(zu)), (N, K))
+        rows = [0, 127, 128, 1000, 2047]
+        xs = x[rows]
+        _, g64 = co.a16w4_fwd(bits(xs), pg.numpy(), bits(sg), bits(zg), None, len(rows), N, K, want_f64=True)
+        _, u64 = co.a16w4_fwd(bits(xs), pu.numpy(), bits(su), bits(zu), None, len(rows), N, K, want_f64=True)
+        g64, u64 = torch.from_numpy(g64), torch.from_numpy(u64)
+        want = g64 / (1 + torch.exp(-g64)) * u64
+        err = rel_l2(got[rows].float().cpu(), want)
+        print(f"gate/up full size: rel_l2={err:.3e} on {len(rows)} token rows")
+        assert err <= REL_L2_TOL
+        return
+    _gate_up_case(ops, co, M, N, K, seed=M + N + K)
+
+
+def test_a16w4_gate_up_silu_rejects_what_it_does_not_cover(ops):
+    from latentq_llm_amd._C import LatentQError
+    _, p, s, z = make_w4(64, 256, 1)
+    w = (dev(p), dev(s), dev(z))
+    with pytest.raises(LatentQError, match="more than 16 tokens"):
+        ops.a16w4_gate_up_silu(dev(randn_bf16((16, 256), 2)), w, w, (64, 256))
+    _, p, s, z = make_w4(64, 384, 1)
+    w = (dev(p), dev(s), dev(z))
+    with pytest.raises(LatentQError, match="multiple of 256"):
+        ops.a16w4_gate_up_silu(dev(randn_bf16((32, 384), 2)), w, w, (64, 384))
+
+
+def test_fused_mlp_module_matches_the_three_layers(hip_lib):
+    """QuantLlamaMLP / make_fused_mlp on QLinearA16W4 layers: the fused path (many tokens) and the composed path
+    (few tokens) both agree with down(silu(gate(x)) * up(x)) run layer by layer."""
+    import torch.nn as nn
+    from latentq_llm_amd import quant as Q
+    from latentq_llm_amd.fused_mlp import QuantLlamaMLP, make_fused_mlp
+
+    hid, ffn = 256, 512
+
+    def layer(n, k, seed):
+        _, packed, scales, zeros = make_w4(n, k, seed)
+        m = Q.QLinearA16W4(k, n, bias=False, lbit=0)
+        m.zeros.data, m.scales.data, m.wshape = zeros.clone(), scales.clone(), [n, k]
+        m.weight.set_value(packed, [m.scales, m.zeros, m.wshape])
+        m = m.bfloat16().cuda()
+        m.to("cuda")
+        return m
+
+    class MLP(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.gate_proj, self.up_proj, self.down_proj = layer(ffn, hid, 1), layer(ffn, hid, 2), layer(hid, ffn, 3)
+
+        def forward(self, x):
+            return self.down_proj(torch.nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.mlp = MLP()
+
+    blk = Block()
+    plain = blk.mlp
+    fused = make_fused_mlp(blk).mlp
+    assert isinstance(fused, QuantLlamaMLP) and fused.gate_proj is plain.gate_proj
+    for tokens in ((2, 3), (4, 128)):  # 6 tokens: composed path; 512 tokens: fused kernel
+        x = randn_bf16(tokens + (hid,), 9).cuda()
+        want, got = plain(x), fused(x)
+        assert got.shape == want.shape == tokens + (hid,)
+        err = rel_l2(got.float(), want.float())
+        print(f"{tokens}: fused MLP vs layer by layer rel_l2={err:.3e}")
+        assert err <= REL_L2_TOL
