@@ -159,6 +159,7 @@ int lq_a16w4_gate_up_silu(const void *x, const void *codes_gate, const void *sca
 #define LQ_PLAN_DIRECT 2       /* weights-direct forward kernel, 128 x 256 tiles */
 #define LQ_PLAN_STAGED_128 3   /* staged kernel, 128 x 128 tiles */
 #define LQ_PLAN_STAGED_256 4   /* staged kernel, 256 x 128 tiles */
+#define LQ_PLAN_DIRECT_128 5   /* weights-direct forward kernel, 128 x 128 tiles */
 int lq_a16w4_plan(int backward, int64_t M, int64_t N, int64_t K, int64_t workspace_bytes, int compute_units,
                   int *kernel, int *splits, int *steps_per_split);
 

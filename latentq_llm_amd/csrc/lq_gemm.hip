@@ -610,8 +610,9 @@ static bool small_tiles(const GemmParams &p) {
 
 // weights-direct forward GEMM (lq_gemm_fwd.hip)
 long long lq_gemm_fwd_direct_workgroups(int M, int N);
+long long lq_gemm_fwd_direct128_workgroups(int M, int N);
 int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
-                              void *y, int M, int N, int K, hipStream_t st, unsigned long long *clk);
+                              void *y, int M, int N, int K, hipStream_t st, unsigned long long *clk, bool narrow);
 int lq_gemm_fwd_gate_up_launch(const void *x, const void *codes_g, const void *scales_g, const void *zeros_g,
                                const void *codes_u, const void *scales_u, const void *zeros_u, void *h, int M, int N, int K,
                                hipStream_t st);
@@ -687,8 +688,9 @@ struct W4Plan {
 // (microseconds, measured): the weights-direct kernel (128 x 256 tiles) takes ~0.86 with one
 // workgroup on a compute unit and ~1.45 for two sharing it; the staged kernel ~0.56 per round of
 // 128 x 128 tiles and ~0.88 per round of 256 x 128 tiles (one workgroup per unit and round). The
-// weights-direct kernel loads scales and zeros four groups at a time: rows must be 4-byte aligned,
-// i.e. the number of groups per row even.
+// weights-direct kernel with 128 x 128 tiles fits three workgroups on a unit: ~0.74 alone, ~1.23 for
+// two, ~1.38 for three. The weights-direct kernels load scales and zeros four groups at a time: rows
+// must be 4-byte aligned, i.e. the number of groups per row even.
 static W4Plan plan_fwd(long long M, long long N, long long K, size_t ws_bytes, long long cus) {
     W4Plan out;
     const long long wg_direct = lq_gemm_fwd_direct_workgroups((int)M, (int)N);
@@ -698,8 +700,19 @@ static W4Plan plan_fwd(long long M, long long N, long long K, size_t ws_bytes, l
     const long long cols = (N + 127) / 128;
     const double est_small = 0.56 * (double)((((M + 127) / 128) * cols + cus - 1) / cus);
     const double est_big = 0.88 * (double)((((M + 255) / 256) * cols + cus - 1) / cus);
+    double est_direct128 = 1e30;
+    if ((K / LQ_GROUP) % 2 == 0) {
+        const long long wg = lq_gemm_fwd_direct128_workgroups((int)M, (int)N);
+        const long long rem128 = wg % (3 * cus);
+        const double tail = rem128 == 0 ? 0.0
+                            : rem128 <= cus ? 0.74
+                            : rem128 <= 2 * cus ? 0.74 + 0.49 * (double)(rem128 - cus) / (double)cus
+                                                : 1.38;
+        est_direct128 = 1.38 * (double)(wg / (3 * cus)) + tail;
+    }
     double step_us = est_direct;
     out.kernel = LQ_PLAN_DIRECT;
+    if (est_direct128 < step_us) { step_us = est_direct128; out.kernel = LQ_PLAN_DIRECT_128; }
     if (est_small < step_us) { step_us = est_small; out.kernel = LQ_PLAN_STAGED_128; }
     if (est_big < step_us) { step_us = est_big; out.kernel = LQ_PLAN_STAGED_256; }
     double est_gemm = step_us * (double)(K / 64 + 3) + 4.0;
@@ -775,8 +788,9 @@ static int a16w4_fwd_impl(const char *who, const void *x, const void *codes, con
         }
         return LQ_OK;
     }
-    if (plan.kernel == LQ_PLAN_DIRECT)
-        return lq_gemm_fwd_direct_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream, clk);
+    if (plan.kernel == LQ_PLAN_DIRECT || plan.kernel == LQ_PLAN_DIRECT_128)
+        return lq_gemm_fwd_direct_launch(x, codes, scales, zeros, bias_or_null, y, (int)M, (int)N, (int)K, (hipStream_t)stream, clk,
+                                         plan.kernel == LQ_PLAN_DIRECT_128);
     GemmParams p = {};
     p.clk = clk;
     p.a = x; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
@@ -900,6 +914,7 @@ extern "C" int lq_calib_gemm_clocks(int backward, const void *a, const void *cod
     LQ_REQUIRE(plan.kernel != LQ_PLAN_GEMV_CHUNKS, "lq_calib_gemm_clocks: this shape runs as GEMV chunks");
     const long long cols = backward ? K : N;
     const long long wg = plan.kernel == LQ_PLAN_DIRECT ? lq_gemm_fwd_direct_workgroups((int)M, (int)N)
+                         : plan.kernel == LQ_PLAN_DIRECT_128 ? lq_gemm_fwd_direct128_workgroups((int)M, (int)N)
                          : plan.kernel == LQ_PLAN_STAGED_256 ? ((M + 255) / 256) * ((cols + 127) / 128)
                                                              : ((M + 127) / 128) * ((cols + 127) / 128);
     LQ_REQUIRE(4 * wg <= clocks_capacity, "lq_calib_gemm_clocks: clocks must hold %lld values, holds %lld", 4 * wg,

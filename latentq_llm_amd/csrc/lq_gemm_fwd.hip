@@ -79,12 +79,16 @@ constexpr int BM = 128, BN = 256;
 constexpr int ROWB = 128;            // bytes of A per tile row and step: 64 bf16
 constexpr int STAGE = BM * ROWB;     // 16 KB per A stage
 
-// GU: gate / up mode. The workgroup then covers 128 output columns (both matrices' rows c0 .. c0 + 127)
-// instead of 256.
-template <bool GU>
+// NT: 32-column tiles per wave (2: the 128 x 256 workgroup tile described above; 1: 128 x 128, a wave owns
+// 128 x 32: twice as many workgroups for outputs whose 128 x 256 tiles leave compute units idle, at the price
+// of one fragment read per MFMA instead of half of one).
+// GU (with NT = 2): gate / up mode. The workgroup then covers 128 output columns (both matrices' rows
+// c0 .. c0 + 127) instead of 256.
+template <int NT, bool GU>
 __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
-    constexpr int BNO = GU ? BN / 2 : BN;  // output columns per workgroup
-    constexpr int WN = BNO / 4;            // output columns per wave
+    static_assert(NT == 2 || (NT == 1 && !GU), "gate / up mode uses both column tiles");
+    constexpr int BNO = (GU || NT == 1) ? BN / 2 : BN;  // output columns per workgroup
+    constexpr int WN = BNO / 4;                         // output columns per wave
     constexpr int ESZ = 2;    // bytes per A element
     constexpr int WROW = 32;  // bytes of one weight row consumed per step
     // 16-byte weight loads per lane and column tile in one batch: the pieces of two consecutive
@@ -172,17 +176,17 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     const u32x4_t w_rsrc1 = GU ? make_rsrc(p.w2 + (long long)c0 * wpitch, (unsigned)rows_here * wpitch) : w_rsrc0;
     const u32x4_t s_rsrc1 = GU ? make_rsrc(p.scales2 + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u) : s_rsrc0;
     const u32x4_t z_rsrc1 = GU ? make_rsrc(p.zeros2 + (long long)c0 * groups_per_row, (unsigned)rows_here * groups_per_row * 2u) : z_rsrc0;
-    unsigned w_off[2], q_off[2];
+    unsigned w_off[NT], q_off[NT];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const unsigned n = GU ? wave * 32 + r : wave * 64 + i * 32 + r;
+    for (int i = 0; i < NT; ++i) {
+        const unsigned n = GU ? wave * 32 + r : wave * WN + i * 32 + r;
         w_off[i] = n * wpitch + h * (WROW / 2);
         q_off[i] = n * (unsigned)groups_per_row * 2u;
     }
 
-    f32x16_t acc[2][4];
+    f32x16_t acc[NT][4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < NT; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -191,12 +195,12 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     // All global loads of the loop are inline assembly: the compiler then inserts no vmcnt waits of
     // its own (it could only wait for everything, LDS-direct loads included); the single
     // s_waitcnt of a step is tied to the loaded registers instead.
-    u32x4_t cw[2][NB], cn[2][NB];  // codes of the current and of the next batch
+    u32x4_t cw[NT][NB], cn[NT][NB];  // codes of the current and of the next batch
     // Raw bf16 scales / zeros of four consecutive groups of the lane's two rows (one 8-byte load per
     // row every 8 steps: a 2-byte load per group would pull a whole cache line through L1 each time).
     // The 8-byte loads need 4-byte aligned rows: the launcher requires an even number of groups per row.
-    u32x2_t qs[2], qz[2];
-    float s[2], nzs[2];
+    u32x2_t qs[NT], qz[NT];
+    float s[NT], nzs[NT];
     auto load_codes_one = [&](int kt, u32x4_t (*c)[NB], int i) {
         const u32x4_t w_rsrc = i == 0 ? w_rsrc0 : w_rsrc1;
         asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(c[i][0]) : "v"(w_off[i]), "s"(w_rsrc), "s"(kt * WROW));
@@ -204,7 +208,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     };
     auto load_codes = [&](int kt, u32x4_t (*c)[NB]) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) load_codes_one(kt, c, i);
+        for (int i = 0; i < NT; ++i) load_codes_one(kt, c, i);
     };
     // Called on the even step two steps before group g starts; loads when g opens a quad.
     auto load_qparams_one = [&](int g, int i) {
@@ -216,12 +220,12 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     };
     auto load_qparams = [&](int g) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) load_qparams_one(g, i);
+        for (int i = 0; i < NT; ++i) load_qparams_one(g, i);
     };
     auto use_qparams = [&](int g) {
         const int shift = (g & 3) * 16;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < NT; ++i) {
             const unsigned long long s4 = ((unsigned long long)qs[i][1] << 32) | qs[i][0];
             const unsigned long long z4 = ((unsigned long long)qz[i][1] << 32) | qz[i][0];
             const float sc = __uint_as_float((unsigned)(s4 >> shift) << 16);
@@ -253,19 +257,28 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     auto wait_and_meet = [&](auto newest, auto with_qparams) {
         constexpr int NEWEST = decltype(newest)::value;
         (void)cn; (void)qs; (void)qz;  // named outside the constexpr branches so that the lambda captures them
-        if constexpr (decltype(with_qparams)::value != 0) {
-            asm volatile("s_waitcnt vmcnt(%8) lgkmcnt(0)\n\ts_barrier"
-                         : "+v"(cn[0][0]), "+v"(cn[0][1]), "+v"(cn[1][0]), "+v"(cn[1][1]), "+v"(qs[0]), "+v"(qs[1]), "+v"(qz[0]),
-                           "+v"(qz[1]) : "n"(NEWEST) : "memory");
+        if constexpr (NT == 2) {
+            if constexpr (decltype(with_qparams)::value != 0) {
+                asm volatile("s_waitcnt vmcnt(%8) lgkmcnt(0)\n\ts_barrier"
+                             : "+v"(cn[0][0]), "+v"(cn[0][1]), "+v"(cn[NT - 1][0]), "+v"(cn[NT - 1][1]), "+v"(qs[0]), "+v"(qs[NT - 1]),
+                               "+v"(qz[0]), "+v"(qz[NT - 1]) : "n"(NEWEST) : "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(%4) lgkmcnt(0)\n\ts_barrier"
+                             : "+v"(cn[0][0]), "+v"(cn[0][1]), "+v"(cn[NT - 1][0]), "+v"(cn[NT - 1][1]) : "n"(NEWEST) : "memory");
+            }
         } else {
-            asm volatile("s_waitcnt vmcnt(%4) lgkmcnt(0)\n\ts_barrier"
-                         : "+v"(cn[0][0]), "+v"(cn[0][1]), "+v"(cn[1][0]), "+v"(cn[1][1]) : "n"(NEWEST) : "memory");
+            if constexpr (decltype(with_qparams)::value != 0) {
+                asm volatile("s_waitcnt vmcnt(%4) lgkmcnt(0)\n\ts_barrier"
+                             : "+v"(cn[0][0]), "+v"(cn[0][1]), "+v"(qs[0]), "+v"(qz[0]) : "n"(NEWEST) : "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(%2) lgkmcnt(0)\n\ts_barrier" : "+v"(cn[0][0]), "+v"(cn[0][1]) : "n"(NEWEST) : "memory");
+            }
         }
     };
 
     // Operands of the first reduction slice of the step about to run; slice 3 of every step
     // prepares them for the step after it, so the MFMA stream continues across the step boundary.
-    u32x4_t af[2][4], bf[2][2];
+    u32x4_t af[2][4], bf[2][NT];
 
     // One reduction step on stage AI with the codes in cw, cut into 8 half-slices of 4 MFMAs (one
     // column tile x four row tiles of one reduction slice). A half-slice also issues the fragment
@@ -290,7 +303,7 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
+            for (int i = 0; i < NT; ++i) {
                 if (t == 3 && i == 0) {
                     wait_and_meet(ic<2>(), ic<ODD ? 0 : 1>());
                     if (ODD) use_qparams((kt + 1) >> 1);
@@ -305,14 +318,21 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
                 else deq_one(cw, 1, 0, bf[0], i);
                 if (t == 0 && !ODD) load_codes_one(kt_codes, cn, i);
                 if (t == 1 && !ODD) load_qparams_one((kt + 2) >> 1 < groups_per_row ? (kt + 2) >> 1 : groups_per_row - 1, i);
-                if (t >= 2) issue_a_one(kt_a, la_load, 2 * (t - 2) + i);
+                if (t >= 2) {
+                    if constexpr (NT == 2) {
+                        issue_a_one(kt_a, la_load, 2 * (t - 2) + i);
+                    } else {
+                        issue_a_one(kt_a, la_load, 2 * (t - 2));
+                        issue_a_one(kt_a, la_load, 2 * (t - 2) + 1);
+                    }
+                }
                 mfma_half(af[t & 1], bf[t & 1], i);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
         if (ODD) {
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < NT; ++i)
 #pragma unroll
                 for (int b = 0; b < NB; ++b) cw[i][b] = cn[i][b];
         }
@@ -324,13 +344,13 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     issue_a(nk > 1 ? 1 : 0, lds_a1);
     wait_and_meet(ic<4>(), ic<1>());
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < NT; ++i)
 #pragma unroll
         for (int b = 0; b < NB; ++b) cw[i][b] = cn[i][b];
     use_qparams(0);
     read_a(lds_a0, 0, af[0]);
-    deq_one(cw, 0, 0, bf[0], 0);
-    deq_one(cw, 0, 0, bf[0], 1);
+#pragma unroll
+    for (int i = 0; i < NT; ++i) deq_one(cw, 0, 0, bf[0], i);
     __builtin_amdgcn_sched_barrier(0);
     int kt = 0;
     for (; kt + 6 <= nk; kt += 6) {
@@ -353,15 +373,24 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     __syncthreads();
-    if constexpr (GU) {
-        // ---- gate / up epilogue: acc[0] and acc[1] hold the same output element of the two products,
-        // column c0 + 32*wave + 8*(q/4) + 4h + q%4, row m0 + 32j + r. H = silu(gate) * up on the fp32
-        // accumulators, rounded once. A wave's 32 rows x 32 columns pass through LDS (row pitch 80
-        // bytes) and leave as 16 bytes per lane, 4 lanes on the 64 contiguous bytes of a row.
+    if constexpr (GU || NT == 1) {
+        // ---- 32 output columns per wave: column c0 + 32*wave + 8*(q/4) + 4h + q%4, row m0 + 32j + r.
+        // Gate / up mode: acc[0] and acc[1] hold the same output element of the two products and
+        // H = silu(gate) * up is formed on the fp32 accumulators, rounded once. A wave's 32 rows x 32
+        // columns pass through LDS (row pitch 80 bytes) and leave as 16 bytes per lane, 4 lanes on the 64
+        // contiguous bytes of a row.
         constexpr int EP = 80;
         unsigned char *ep = ((wave & 2) ? lds_a1 : lds_a0) + (wave & 1) * (32 * EP);
         const int ep_row = lane >> 2, ep_chunk = lane & 3;
         const int c_lane = c0 + wave * WN + ep_chunk * 8;
+        float bias_n[4][4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int c = c0 + wave * WN + 8 * q + 4 * h + e;
+                bias_n[q][e] = (!GU && p.bias && c < p.N) ? lq_bf16_bits_to_f32(p.bias[c]) : 0.0f;
+            }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -370,7 +399,12 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const float g = acc[0][j][4 * q + e];
-                    v[e] = g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * acc[1][j][4 * q + e];
+                    if constexpr (GU) {
+                        v[e] = g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * acc[NT - 1][j][4 * q + e];
+                    } else {
+                        v[e] = g;
+                        if (p.bias) v[e] += bias_n[q][e];
+                    }
                 }
                 u32x2_t o = {lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3])};
                 *reinterpret_cast<u32x2_t *>(ep + r * EP + (8 * q + 4 * h) * 2) = o;
@@ -443,30 +477,31 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
 // Number of workgroups this kernel would launch; the dispatcher in lq_gemm.hip prefers it when they
 // can fill the device two per CU.
 long long lq_gemm_fwd_direct_workgroups(int M, int N) { return (long long)((M + BM - 1) / BM) * ((N + BN - 1) / BN); }
+long long lq_gemm_fwd_direct128_workgroups(int M, int N) { return (long long)((M + BM - 1) / BM) * ((N + BN / 2 - 1) / (BN / 2)); }
 
-template <bool GU>
+template <int NT, bool GU>
 static int launch_direct(FwdParams p, hipStream_t st, const char *who) {
-    constexpr int BNO = GU ? BN / 2 : BN;
+    constexpr int BNO = (GU || NT == 1) ? BN / 2 : BN;
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BNO - 1) / BNO;
     const long long nwg = (long long)p.tiles_m * p.tiles_n;
     if (nwg > 0x7FFFFFFFll) return lq_fail(LQ_ERR_BAD_ARG, "%s: problem too large", who);
     // the 32-bit lane offsets of the activation and weight loads span 128 / 256 rows
     if ((long long)BN * p.K * 2 >= (1ll << 32)) return lq_fail(LQ_ERR_BAD_ARG, "%s: K too large", who);
-    hipLaunchKernelGGL(gemm_fwd_direct_kernel<GU>, dim3((unsigned)nwg), dim3(256), 0, st, p);
+    hipLaunchKernelGGL((gemm_fwd_direct_kernel<NT, GU>), dim3((unsigned)nwg), dim3(256), 0, st, p);
     return lq_check_launch(who);
 }
 
 // Called by lq_a16w4_fwd (lq_gemm.hip) after argument validation: K % 256 == 0, N % 16 == 0, M > 16.
 int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
-                              void *y, int M, int N, int K, hipStream_t st, unsigned long long *clk) {
+                              void *y, int M, int N, int K, hipStream_t st, unsigned long long *clk, bool narrow) {
     FwdParams p = {};
     p.clk = clk;
     p.x = (const unsigned char *)x; p.w = (const unsigned char *)codes;
     p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.bias = (const unsigned short *)bias; p.y = (unsigned short *)y;
     p.M = M; p.N = N; p.K = K;
-    return launch_direct<false>(p, st, "lq_a16w4_fwd");
+    return narrow ? launch_direct<1, false>(p, st, "lq_a16w4_fwd") : launch_direct<2, false>(p, st, "lq_a16w4_fwd");
 }
 
 // Called by lq_a16w4_gate_up_silu (lq_gemm.hip) after argument validation: K % 256 == 0, N % 16 == 0, M > 16.
@@ -479,5 +514,5 @@ int lq_gemm_fwd_gate_up_launch(const void *x, const void *codes_g, const void *s
     p.w2 = (const unsigned char *)codes_u; p.scales2 = (const unsigned short *)scales_u; p.zeros2 = (const unsigned short *)zeros_u;
     p.y = (unsigned short *)h;
     p.M = M; p.N = N; p.K = K;
-    return launch_direct<true>(p, st, "lq_a16w4_gate_up_silu");
+    return launch_direct<2, true>(p, st, "lq_a16w4_gate_up_silu");
 }

@@ -209,7 +209,8 @@ def a16w4_dx(dy, codes, scales, zeros, shape, out=None):
     return dx
 
 
-PLAN_KERNELS = {0: "gemv", 1: "gemv_chunks", 2: "direct_128x256", 3: "staged_128x128", 4: "staged_256x128"}
+PLAN_KERNELS = {0: "gemv", 1: "gemv_chunks", 2: "direct_128x256", 3: "staged_128x128", 4: "staged_256x128",
+                5: "direct_128x128"}
 
 
 def a16w4_plan(M: int, shape, backward: bool = False, workspace_bytes: int = WORKSPACE_MAX_BYTES, compute_units: int = 0):

@@ -170,6 +170,12 @@ def test_dispatch_plan_host_logic(hip_lib):
     assert plan(2048, 11008, 4096 + 128)[0] != "direct_128x256"
     # one round of small tiles beats everything else when it fits
     assert plan(256, 11008, 4096) == ("staged_128x128", 1, 0)
+    # between one and two rounds of the 128 x 256 tiles the weights-direct kernel with 128 x 128 tiles (three
+    # workgroups per compute unit) fills the device better
+    for M in (384, 768, 1024, 1536):
+        assert plan(M, 11008, 4096) == ("direct_128x128", 1, 0), M
+    assert plan(3072, 4096, 11008) == ("direct_128x128", 1, 0)
+    assert plan(2048, 11008, 4096 + 128)[0] not in ("direct_128x256", "direct_128x128")
     # skinny grids: split reduction, slices of an even number of steps >= 8 that cover the reduction
     for M, N, K, back in [(128, 11008, 4096, True), (512, 11008, 4096, True), (1024, 11008, 4096, True),
                           (128, 4096, 11008, False), (512, 4096, 11008, False), (200, 2048, 1280, False)]:

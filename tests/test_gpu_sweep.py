@@ -69,3 +69,33 @@ def test_a8w8_random_shapes(ops, M, N, K):
     want = x8.double() @ w8.double().t()  # exact: |acc| < 2^31 << 2^53
     assert torch.equal(acc.double(), want)
     assert torch.equal(y, ((want.float() * sx[:, None]) * sw[None, :]).to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("M,N,K,bias", [(300, 11008, 256, False), (1000, 11024, 512, True), (768, 5504, 1024, False),
+                                        (3072, 4096, 2048, True), (1536, 11008, 4096, False), (384, 11024, 4096, True)])
+def test_forward_weights_direct_kernel_with_128x128_tiles(ops, M, N, K, bias):
+    """Shapes the planner gives to the weights-direct kernel with 128 x 128 tiles (between one and two rounds of
+    its 128 x 256 tiles): ragged token counts, a last tile of 16 columns (N = 11024), 4 to 64 reduction steps,
+    with and without bias, against the fp32 product of the dequantised matrix."""
+    assert ops.a16w4_plan(M, (N, K))[0] == "direct_128x128"
+    _, packed, scales, zeros = make_w4(N, K, M + N + K)
+    w = (packed.cuda(), scales.cuda(), zeros.cuda())
+    W = ops.a16w4_dequant(*w, (N, K)).float()
+    g = torch.Generator(device="cuda").manual_seed(M + 3)
+    x = torch.randn(M, K, device="cuda", generator=g).to(torch.bfloat16)
+    b = torch.randn(N, device="cuda", generator=g).to(torch.bfloat16) if bias else None
+    y = ops.a16w4_forward(x, *w, (N, K), bias=b).float()
+    ref = x.float() @ W.t() + (b.float() if bias else 0)
+    assert ((y - ref).norm() / ref.norm()).item() < TOL
+
+
+def test_forward_128x128_direct_kernel_identity_is_exact_dequant(ops):
+    """X = identity through the 128 x 128 weights-direct kernel: every output is one dequantised weight, bit for bit."""
+    N, K = 11008, 1024
+    M = K
+    assert ops.a16w4_plan(M, (N, K))[0] == "direct_128x128"
+    _, packed, scales, zeros = make_w4(N, K, 31)
+    w = (packed.cuda(), scales.cuda(), zeros.cuda())
+    x = torch.eye(K, device="cuda", dtype=torch.bfloat16)
+    y = ops.a16w4_forward(x, *w, (N, K))
+    assert torch.equal(y, ops.a16w4_dequant(*w, (N, K)).t().contiguous())
