@@ -438,6 +438,13 @@ def profile_target(device, which, launches=10):
             o.a16w4_dx(h, *blk.gate, (FFN, HID))
         for _ in range(launches):
             o.a16w4_dx(blk.dy, *blk.down, (HID, FFN))
+        # the inference-side fused product silu(gate(x)) * up(x), and the 128 x 128-tile instance of the forward kernel
+        hbuf = torch.empty((TOKENS, FFN), dtype=torch.bfloat16, device=device)
+        for _ in range(launches):
+            o.a16w4_gate_up_silu(blk.x, blk.gate, blk.up, (FFN, HID), out=hbuf)
+        x1536 = torch.randn(1536, HID, device=device).to(torch.bfloat16)
+        for _ in range(launches):
+            o.a16w4_forward(x1536, *blk.gate, (FFN, HID))
     elif which == "requant":
         # the benchmark size (8192 x 2048), then 4 and 16 times as many rows: steady state against launch cost
         for rows in (8192, 4 * 8192, 16 * 8192):
