@@ -401,6 +401,23 @@ def bench_gate_up(device, blk):
         flop = 4.0 * M * HID * FFN
         out.append({"M": M, "fused_us": t_fused * 1e6, "fused_TFLOP/s": flop / t_fused / 1e12,
                     "two_gemms_silu_mul_us": t_parts * 1e6, "two_gemms_silu_mul_TFLOP/s": flop / t_parts / 1e12})
+    # decode: one GEMV pass over both matrices against two GEMVs and the two tensor operations, as HIP graphs over
+    # rotating weight sets larger than the last-level cache
+    sets = [(synth_w4(FFN, HID, 70 + 2 * i, device), synth_w4(FFN, HID, 71 + 2 * i, device)) for i in range(7)]
+    for M in (1, 4, 16):
+        x = torch.randn(M, HID, device=device).to(torch.bfloat16)
+        h = torch.empty((M, FFN), dtype=torch.bfloat16, device=device)
+        g_, u_ = torch.empty_like(h), torch.empty_like(h)
+        t_fused = graph_time([(lambda w=w: ops.a16w4_gate_up_silu(x, w[0], w[1], (FFN, HID), out=h)) for w in sets])
+
+        def parts(w):
+            ops.a16w4_forward(x, *w[0], (FFN, HID), out=g_)
+            ops.a16w4_forward(x, *w[1], (FFN, HID), out=u_)
+            torch.mul(torch.nn.functional.silu(g_), u_, out=h)
+        t_parts = graph_time([(lambda w=w: parts(w)) for w in sets])
+        nbytes = 2 * (FFN * HID // 2 + 4 * FFN * HID // GROUP) + 2 * M * HID + 2 * M * FFN
+        out.append({"M": M, "fused_us": t_fused * 1e6, "fused_GB/s": nbytes / t_fused / 1e9, "fused_frac_hbm": nbytes / t_fused / 8e12,
+                    "two_gemvs_silu_mul_us": t_parts * 1e6, "bytes": nbytes})
     return out
 
 

@@ -142,8 +142,10 @@ int lq_a16w4_fwd_static(const void *x, const void *codes, const void *scales, co
  * fusedmatmul_248_kernel: "C = silu(A * B1) * (A * B2)", called from QuantLlamaMLP.triton_llama_mlp
  * :206-218), on the native code layout. Neither product is rounded on its own, so h differs from
  * running lq_a16w4_fwd twice and multiplying in bf16 by the roundings that path adds.
- * Both matrices [N,K] with their own scales and zeros; no bias. K % 256 == 0; N % 16 == 0; M > 16
- * (LQ_ERR_BAD_ARG otherwise: a caller with fewer tokens runs the two products through lq_a16w4_fwd). */
+ * Both matrices [N,K] with their own scales and zeros; no bias. N % 16 == 0; K % 128 == 0, and
+ * K % 256 == 0 for M > 16. Up to 16 tokens run as one GEMV pass over both matrices (sums in fp32, the
+ * weights not rounded to bf16 first, as in lq_a16w4_fwd for such M), more tokens through the MFMA
+ * kernel of lq_a16w4_fwd. */
 int lq_a16w4_gate_up_silu(const void *x, const void *codes_gate, const void *scales_gate, const void *zeros_gate,
                           const void *codes_up, const void *scales_up, const void *zeros_up, void *h, int64_t M,
                           int64_t N, int64_t K, int group, void *stream);

@@ -625,6 +625,9 @@ int lq_gemm_i8_tile_launch(const void *x8, const void *w8, const float *sx, cons
 // GEMV path (lq_gemv.hip)
 int lq_gemv_a16w4_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
                          void *y, int M, int N, int K, hipStream_t st);
+int lq_gemv_a16w4_gate_up_launch(const void *x, const void *codes_g, const void *scales_g, const void *zeros_g,
+                                 const void *codes_u, const void *scales_u, const void *zeros_u, void *h, int M, int N, int K,
+                                 hipStream_t st);
 
 static int check_w4_common(const char *who, const void *a, const void *codes, const void *scales, const void *zeros,
                            const void *out, int64_t M, int64_t N, int64_t K, int group) {
@@ -815,9 +818,10 @@ extern "C" int lq_a16w4_gate_up_silu(const void *x, const void *codes_gate, cons
     rc = check_w4_common(who, x, codes_up, scales_up, zeros_up, h, M, N, K, group);
     if (rc) return rc;
     LQ_REQUIRE(N % 16 == 0, "%s: N=%lld must be a multiple of 16", who, (long long)N);
-    LQ_REQUIRE(K % 256 == 0, "%s: K=%lld must be a multiple of 256", who, (long long)K);
-    LQ_REQUIRE(M > 16, "%s: needs more than 16 tokens (M=%lld); below that run the two products through lq_a16w4_fwd", who,
-               (long long)M);
+    if (M <= 16)
+        return lq_gemv_a16w4_gate_up_launch(x, codes_gate, scales_gate, zeros_gate, codes_up, scales_up, zeros_up, h, (int)M, (int)N,
+                                            (int)K, (hipStream_t)stream);
+    LQ_REQUIRE(K % 256 == 0, "%s: K=%lld must be a multiple of 256 for more than 16 tokens", who, (long long)K);
     return lq_gemm_fwd_gate_up_launch(x, codes_gate, scales_gate, zeros_gate, codes_up, scales_up, zeros_up, h, (int)M, (int)N,
                                       (int)K, (hipStream_t)stream);
 }

@@ -51,24 +51,34 @@ constexpr int kXRow = 1024 + 16;  // LDS bytes per staged token row: 4 groups x 
 // MP = number of token rows staged per wave and batch (>= M). NT = 16-row weight tiles per
 // workgroup: every workgroup stages the activations of its K range again, so with many tokens two
 // tiles per workgroup halve that traffic (and share the activation-sum MFMAs).
-template <int WAVES, int MP, int NT, bool QS>
+// GU (with NT = 2, no QS): gate / up mode. Tile 1 is the same 16 rows of a second matrix (codes2, scales2,
+// zeros2) and the output is silu(tile 0) * tile 1 on the fp32 sums: the gate / up pair of a gated MLP in one
+// pass over both matrices.
+template <int WAVES, int MP, int NT, bool QS, bool GU = false>
 __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *__restrict__ x,
                                                           const unsigned char *__restrict__ codes,
                                                           const unsigned short *__restrict__ scales,
                                                           const unsigned short *__restrict__ zeros,
                                                           const unsigned short *__restrict__ bias,
-                                                          unsigned short *__restrict__ y, int M, int N, int K) {
+                                                          unsigned short *__restrict__ y, int M, int N, int K,
+                                                          const unsigned char *__restrict__ codes2 = nullptr,
+                                                          const unsigned short *__restrict__ scales2 = nullptr,
+                                                          const unsigned short *__restrict__ zeros2 = nullptr) {
+    static_assert(!GU || (NT == 2 && !QS), "gate / up mode: two tiles, scales and zeros straight from memory");
+    constexpr int RT = GU ? 1 : NT;  // 16-row tiles of output rows per workgroup
     __shared__ float red[WAVES][NT][4][64];
     __shared__ __attribute__((aligned(16))) unsigned char xs[WAVES][MP][kXRow];
     extern __shared__ __attribute__((aligned(16))) unsigned char sq[];  // QS: scales then zeros of the workgroup's rows
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // scalar: uniform control flow
     const int n = lane & 15, kq = lane >> 4;
-    const int row = blockIdx.x * (16 * NT) + n;  // weight row of this lane's B fragment in tile 0 (tile j: + 16 j)
+    const int row = blockIdx.x * (16 * RT) + n;  // weight row of this lane's B fragment in tile 0 (tile j: + 16 j)
     const int G = K / LQ_GROUP;
 
     // load layout of the codes: lane 4*r + c -> row r of this block, 16-byte chunk c of the group
-    const unsigned char *wrow = codes + (long long)(blockIdx.x * (16 * NT) + (lane >> 2)) * (K / 2) + (lane & 3) * 16;
+    const long long wrow_off = (long long)(blockIdx.x * (16 * RT) + (lane >> 2)) * (K / 2) + (lane & 3) * 16;
+    const unsigned char *wrow = codes + wrow_off;
+    const unsigned char *wrow2 = GU ? codes2 + wrow_off : nullptr;  // gate / up mode: tile 1 is the second matrix
     const long long tile_stride = 16ll * (K / 2);  // bytes between the same row of consecutive tiles
     const int bperm_src = (4 * n + kq) * 4;  // ds_bpermute: take from lane 4*n + kq
     const int bcast_src = n * 4;             // ds_bpermute: take from lane n (kq = 0)
@@ -142,7 +152,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) {
                 const int g = g0 + u < G ? g0 + u : G - 1;
-                wv[j][u] = *reinterpret_cast<const u32x4_t *>(wrow + j * tile_stride + g * 64);
+                const unsigned char *wt = (GU && j == 1) ? wrow2 : wrow + j * tile_stride;
+                wv[j][u] = *reinterpret_cast<const u32x4_t *>(wt + g * 64);
             }
         if constexpr (QS) {
             if (first) {
@@ -164,7 +175,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
         } else
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
-            const unsigned short *sr = srow + (long long)j * 16 * G, *zr = zrow + (long long)j * 16 * G;
+            const unsigned short *sr = GU ? (j == 0 ? srow : scales2 + (long long)row * G) : srow + (long long)j * 16 * G;
+            const unsigned short *zr = GU ? (j == 0 ? zrow : zeros2 + (long long)row * G) : zrow + (long long)j * 16 * G;
             if (full) {
                 u32x2_t sraw = {0u, 0u}, zraw = {0u, 0u};
                 if (kq == 0) {
@@ -241,7 +253,21 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(const unsigned short *
 #pragma unroll
         for (int r = 0; r < 4; ++r) red[wave][j][r][lane] = acc[j][r];
     __syncthreads();
-    if (wave < NT) {
+    if constexpr (GU) {
+        if (wave == 0) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float g = 0.f, u = 0.f;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) {
+                    g += red[w][0][r][lane];
+                    u += red[w][1][r][lane];
+                }
+                const int m = 4 * kq + r;
+                if (m < M) y[(long long)m * N + row] = lq_f32_to_bf16_bits(g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u);
+            }
+        }
+    } else if (wave < NT) {
         // wave j finishes tile j; lane holds D[m = 4*kq + r][n]
         const int orow = row + 16 * wave;
         const float b = bias ? lq_bf16_bits_to_f32(bias[orow]) : 0.0f;
@@ -266,6 +292,21 @@ struct GemvArgs {
     int M, N, K;
     hipStream_t st;
 };
+
+struct GemvGuArgs {
+    const void *x, *codes, *scales, *zeros, *codes2, *scales2, *zeros2;
+    void *y;
+    int M, N, K;
+    hipStream_t st;
+};
+
+template <int W, int MP>
+void launch_gu(const GemvGuArgs &a) {
+    hipLaunchKernelGGL((gemv_kernel<W, MP, 2, false, true>), dim3(a.N / 16), dim3(64 * W), 0, a.st, (const unsigned short *)a.x,
+                       (const unsigned char *)a.codes, (const unsigned short *)a.scales, (const unsigned short *)a.zeros,
+                       (const unsigned short *)nullptr, (unsigned short *)a.y, a.M, a.N, a.K, (const unsigned char *)a.codes2,
+                       (const unsigned short *)a.scales2, (const unsigned short *)a.zeros2);
+}
 
 template <int W, int MP, int NT>
 void launch_one(const GemvArgs &a) {
@@ -325,4 +366,29 @@ int lq_gemv_a16w4_launch(const void *x, const void *codes, const void *scales, c
         launch_waves<16, 1, 8>(pick_waves(batches, 8), a);
     }
     return lq_check_launch("lq_a16w4_fwd(gemv)");
+}
+
+// silu(x Wgate^T) * (x Wup^T) for 1 <= M <= 16: both matrices in one pass. N % 16 == 0 and K % 128 == 0 are
+// guaranteed by the caller.
+int lq_gemv_a16w4_gate_up_launch(const void *x, const void *codes_g, const void *scales_g, const void *zeros_g,
+                                 const void *codes_u, const void *scales_u, const void *zeros_u, void *h, int M, int N, int K,
+                                 hipStream_t st) {
+    const GemvGuArgs a = {x, codes_g, scales_g, zeros_g, codes_u, scales_u, zeros_u, h, M, N, K, st};
+    const int batches = (K / LQ_GROUP + 3) / 4;
+    if (M <= 4) {
+        switch (pick_waves(batches, 16)) {
+            case 2: launch_gu<2, 4>(a); break;
+            case 4: launch_gu<4, 4>(a); break;
+            case 8: launch_gu<8, 4>(a); break;
+            default: launch_gu<16, 4>(a); break;
+        }
+    } else {
+        // 16 staged token rows cost a wave 16.25 KB of LDS: at most 8 waves
+        switch (pick_waves(batches, 8)) {
+            case 2: launch_gu<2, 16>(a); break;
+            case 4: launch_gu<4, 16>(a); break;
+            default: launch_gu<8, 16>(a); break;
+        }
+    }
+    return lq_check_launch("lq_a16w4_gate_up_silu(gemv)");
 }

@@ -13,10 +13,11 @@ import torch.nn as nn
 
 from . import ops
 
-# Below this many tokens the two products go through the ordinary forward (GEMV, GEMV chunks or the split
-# reduction, whichever the library picks) and the SiLU product is formed on their bf16 results: the fused
-# kernel's 128-row tiles would be mostly empty (on the 7B matrices it takes 51 us from 17 to 192 tokens, the
-# composed path 44 us at 17 tokens, 54 at 64, 84 at 192).
+# Up to 16 tokens the fused product is one GEMV pass over both matrices, from FUSED_MIN_TOKENS on the MFMA kernel.
+# In between the two products go through the ordinary forward (GEMV chunks or the split reduction, whichever the
+# library picks) and the SiLU product is formed on their bf16 results: the fused kernel's 128-row tiles would be
+# mostly empty (on the 7B matrices it takes 51 us from 17 to 192 tokens, the composed path 44 us at 17 tokens, 54
+# at 64, 84 at 192).
 FUSED_MIN_TOKENS = 64
 
 
@@ -46,7 +47,7 @@ class QuantLlamaMLP(nn.Module):
         out_shape = x.shape[:-1] + (self.intermediate_size,)
         x2 = x.reshape(-1, x.shape[-1])
         M, K = x2.shape
-        if M >= FUSED_MIN_TOKENS and K % 256 == 0 and x2.dtype == torch.bfloat16:
+        if x2.dtype == torch.bfloat16 and (0 < M <= 16 or (M >= FUSED_MIN_TOKENS and K % 256 == 0)):
             if not x2.is_contiguous():
                 x2 = x2.contiguous()
             h = ops.a16w4_gate_up_silu(x2, _w4(self.gate_proj), _w4(self.up_proj), (self.intermediate_size, K))

@@ -162,7 +162,7 @@ def a16w4_forward_static(x, codes, scales, zeros, shape, out, bias=None):
 
 def a16w4_gate_up_silu(x, gate, up, shape, out=None):
     """h[M,N] = silu(X . deq(Wgate)^T) * (X . deq(Wup)^T) in one launch (lq_a16w4_gate_up_silu); gate and up are
-    (codes, scales, zeros) triples of two [N, K] matrices. Needs M > 16 and K % 256 == 0."""
+    (codes, scales, zeros) triples of two [N, K] matrices. Needs K % 256 == 0 above 16 tokens."""
     N, K = shape
     _chk(x, torch.bfloat16, "x")
     if x.dim() != 2 or x.shape[1] != K:
@@ -177,6 +177,8 @@ def a16w4_gate_up_silu(x, gate, up, shape, out=None):
         _chk(out, torch.bfloat16, "out")
         if tuple(out.shape) != (M, N):
             raise ValueError(f"out must be [{M},{N}]")
+    if M == 0:
+        return out
     with torch.cuda.device(x.device):
         _C.call("lq_a16w4_gate_up_silu", x.data_ptr(), gate[0].data_ptr(), gate[1].data_ptr(), gate[2].data_ptr(),
                 up[0].data_ptr(), up[1].data_ptr(), up[2].data_ptr(), out.data_ptr(), M, N, K, GROUP, _stream(x))
