@@ -676,7 +676,7 @@ def main():
     tot = 2 * kern["fwd_gate_up"]["us"] + kern["fwd_down"]["us"] + 2 * kern["dx_gate_up"]["us"] + kern["dx_down"]["us"]
     avg_us = tot / 6
     achieved = 2 * TOKENS * HID * FFN / (avg_us * 1e-6) / 1e12
-    roofline = {"bound": "mfma", "kernel": "A16W4 dequant-GEMM: gemm_fwd_direct_kernel<false> (forward), gemm_kernel<1> (dX)",
+    roofline = {"bound": "mfma", "kernel": "A16W4 dequant-GEMM: gemm_fwd_direct_kernel<2, false> (forward), gemm_kernel<1> (dX)",
                 "achieved": achieved, "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": achieved * 1e12 / PEAK_BF16,
                 "avg_launch_us": avg_us, "flop_per_launch": 2 * TOKENS * HID * FFN, "traffic": gemm_traffic_bytes(),
                 "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated on a copy)"}
@@ -697,11 +697,11 @@ def main():
         roofline["ceiling"] = {"what": "MFMA-only loop (lq_calib_mfma_loop), random bf16 operands, the forward kernel's 2 x 4 waves per compute unit",
                                "TFLOP/s": loop, "achieved_over_ceiling": achieved / loop}
         line["ceiling"] = ceil
+        line["gate_up_silu"] = bench_gate_up(dev, blk)
         del blk
         torch.cuda.empty_cache()
         line["requant"] = bench_requant(dev)
         line["gradq8"] = bench_gradq8(dev)
-        line["gate_up_silu"] = bench_gate_up(dev, blk)
         line["latent_lbit4"] = bench_latent(dev)
         line["gemv"] = bench_gemv(dev)
         line["a8w8"] = bench_a8w8(dev)
