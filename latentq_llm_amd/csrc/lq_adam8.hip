@@ -69,6 +69,22 @@ __device__ __forceinline__ void block_minmax(float &lo, float &hi, float (*red)[
     }
 }
 
+// byte SEL of `old` replaced by sat_u8(rne(v)) (v_cvt_pk_u8_f32)
+template <int SEL>
+__device__ __forceinline__ unsigned cvt_pk_u8(float v, unsigned old) {
+    unsigned r;
+    asm("v_cvt_pk_u8_f32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "n"(SEL), "v"(old));
+    return r;
+}
+
+// m / d, correctly rounded, for two bf16 numbers. The quotient of two 8-bit significands keeps a relative
+// distance of at least 2^-33 from every midpoint of two fp32 numbers (m = d * mid has no solution: mid has 25
+// significant bits), and q0 = m r with the hardware reciprocal r (one ulp), corrected once by the exact residual
+// (q0 + (m - q0 d) r, one rounding), is within 2^-45 of the quotient: it rounds to the same fp32 number as the
+// IEEE division (every significand pair and every one-ulp variant of r is checked on the CPU). Quotients or
+// divisors outside [2^-40, 2^40] (residual underflow, overflow, zero, NaN) take the division (div_bf16_operands
+// names this sequence in the comments below; it is written out in the kernel).
+
 // x[8] -> uint8 codes with the block's (scale, max); returns them packed, 8 bytes.
 // The quotient (hi - x) / scale must be the correctly rounded one (a quotient one ulp off can fall
 // on the other side of a rounding tie). The divisor is shared by the whole block, so the division
@@ -93,9 +109,14 @@ __device__ __forceinline__ u32x2_t quantize8(const float x[8], float scale, floa
         } else {
             q = t / scale;
         }
-        q = rintf(q);
-        q = fminf(fmaxf(q, 0.0f), 255.0f);
-        w[k >> 2] |= ((unsigned)q & 0xFFu) << (8 * (k & 3));
+        // clamp(rint(q), 0, 255) and the byte insertion in one instruction (round to nearest even, saturating,
+        // NaN -> 0 like fmaxf(NaN, 0))
+        switch (k & 3) {
+            case 0: w[k >> 2] = cvt_pk_u8<0>(q, w[k >> 2]); break;
+            case 1: w[k >> 2] = cvt_pk_u8<1>(q, w[k >> 2]); break;
+            case 2: w[k >> 2] = cvt_pk_u8<2>(q, w[k >> 2]); break;
+            default: w[k >> 2] = cvt_pk_u8<3>(q, w[k >> 2]); break;
+        }
     }
     return u32x2_t{w[0], w[1]};
 }
@@ -109,6 +130,19 @@ __device__ __forceinline__ u32x2_t quantize8(const float x[8], float scale, floa
 __device__ __forceinline__ float sqrt_bf16_to_bf16(float v) {
     if (v >= 0x1p-100f) return bf16r(__builtin_amdgcn_sqrtf(v));
     return bf16r(__builtin_sqrtf(v));
+}
+
+// A thread's 8 updated latent values back to one code word and one residual word (codec parameters by value)
+template <bool kFast>
+__device__ __forceinline__ void requant8(const float (&out)[8], float ws, float wz, float wr, const CodecParams pq,
+                                         unsigned &cnew, unsigned &rnew) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        unsigned nib, code;
+        lq_latent_requant_elem<kFast>(out[k], ws, wz, wr, pq, nib, code);
+        rnew = (rnew << 4) | nib;
+        cnew |= code << (4 * (k ^ 1));
+    }
 }
 
 template <int BS, bool LATENT>
@@ -139,7 +173,11 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
         p4 = a.param[Tc];
     }
 
-    float m[8], d[8], out[8];
+    // Phase 1: the moments. The square root and the quotient use short sequences that are exact on all but
+    // extreme operands; whether any of a thread's 8 elements is such an operand is collected in one flag per
+    // sequence, and the (cold) exact sequences then redo all 8: one branch per thread instead of one per element.
+    float m[8], d[8], v[8], out[8];
+    bool odd_sqrt = false;
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
         const float g = (k & 1) ? lq_bf16_hi(g4[k >> 1]) : lq_bf16_lo(g4[k >> 1]);
@@ -152,11 +190,25 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
         mk = bf16r(fmaf(a.one_minus_beta1, g, mk));
         vk = bf16r(vk * a.beta2);
         vk = bf16r(fmaf(a.one_minus_beta2 * g, g, vk));
-        float dk = sqrt_bf16_to_bf16(vk);
-        dk = bf16r(dk + a.eps);
         m[k] = mk;
-        d[k] = dk;
-        float ratio;
+        v[k] = vk;
+        // bf16(sqrt(v)) from the hardware's one-ulp square root (see sqrt_bf16_to_bf16); it does not take
+        // denormals, so nonzero inputs below 2^-100 go through the exact one (zero, negative and NaN inputs give
+        // the same result either way)
+        d[k] = bf16r(__builtin_amdgcn_sqrtf(vk));
+        odd_sqrt |= vk < 0x1p-100f && vk > 0.0f;
+    }
+    if (odd_sqrt) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) d[k] = sqrt_bf16_to_bf16(v[k]);
+    }
+    float ratio[8];
+    bool odd_div = false;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        d[k] = bf16r(d[k] + a.eps);
+        const float r = __builtin_amdgcn_rcpf(d[k]);
+        const float q0 = m[k] * r;
         if (!LATENT && !a.param) {
             // Only bf16(m / d) is stored here, and the quotient of two bf16 numbers never comes closer
             // than 2^-17 (relative) to the midpoint of two bf16 values (256 m_a = (2j+1) m_b has no
@@ -164,33 +216,39 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
             // same bf16 value as the correctly rounded one (every significand pair is checked by the
             // CPU tests): reciprocal and product instead of the division sequence. Results outside
             // [2^-100, 2^100] (bf16 subnormals, overflow, NaN; zero numerators excepted) take the division.
-            ratio = mk * __builtin_amdgcn_rcpf(dk);
-            const float ar = fabsf(ratio);
-            if (!(ar <= 0x1p100f && (ar >= 0x1p-100f || mk == 0.0f))) ratio = mk / dk;
+            ratio[k] = q0;
+            const float ar = fabsf(q0);
+            odd_div |= !(ar <= 0x1p100f && (ar >= 0x1p-100f || m[k] == 0.0f));
         } else {
-            ratio = mk / dk;
+            // The fp32 quotient itself enters the update: one residual correction of q0 gives the IEEE
+            // quotient of two bf16 numbers (div_bf16_operands) unless quotient or divisor leave [2^-40, 2^40].
+            ratio[k] = fmaf(fmaf(-q0, d[k], m[k]), r, q0);
+            const float aq = fabsf(ratio[k]), ad = fabsf(d[k]);
+            odd_div |= !(aq >= 0x1p-40f && aq <= 0x1p40f && ad >= 0x1p-40f && ad <= 0x1p40f);
         }
+    }
+    if (odd_div) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) ratio[k] = m[k] / d[k];
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
         if constexpr (LATENT) {
             const float p = bf16r(lq_latent_value(lq_code(cword, k), vtab[(rword >> (28 - 4 * k)) & 0xFu], ws, wz));
-            out[k] = bf16r(fmaf(a.neg_step, ratio, p));
+            out[k] = bf16r(fmaf(a.neg_step, ratio[k], p));
         } else if (a.param) {
             const float p = (k & 1) ? lq_bf16_hi(p4[k >> 1]) : lq_bf16_lo(p4[k >> 1]);
-            out[k] = fmaf(a.neg_step, ratio, p);
+            out[k] = fmaf(a.neg_step, ratio[k], p);
         } else {
-            out[k] = ratio;
+            out[k] = ratio[k];
         }
     }
     if constexpr (LATENT) {
         const bool fast = (ws >= 0x1p-40f) && (ws <= 0x1p40f);
         const float wr = 1.0f / ws;
         unsigned cnew = 0, rnew = 0;
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            unsigned nib, code;
-            lq_latent_requant_elem(out[k], ws, wz, wr, fast, a.quant_curve, nib, code);
-            rnew = (rnew << 4) | nib;
-            cnew |= code << (4 * (k ^ 1));
-        }
+        if (fast) requant8<true>(out, ws, wz, wr, a.quant_curve, cnew, rnew);
+        else requant8<false>(out, ws, wz, wr, a.quant_curve, cnew, rnew);
         if (live) {
             a.codes[T] = cnew;
             a.residual[T] = rnew;

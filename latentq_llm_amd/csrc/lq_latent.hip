@@ -45,6 +45,26 @@ __global__ __launch_bounds__(256) void latent_reconstruct_kernel(const u32x4_t *
     }
 }
 
+// The 32 elements of one thread through the re-quantiser (codec parameters by value: scalars)
+template <bool kFast>
+__device__ __forceinline__ void requant_thread(const u32x4_t (&in)[4], float s, float z, float r, const CodecParams p,
+                                               u32x4_t &cout, u32x4_t &rout) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        unsigned cword = 0, rword = 0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float t = (k & 1) ? lq_bf16_hi(in[i][k >> 1]) : lq_bf16_lo(in[i][k >> 1]);
+            unsigned nib, code;
+            lq_latent_requant_elem<kFast>(t, s, z, r, p, nib, code);
+            rword = (rword << 4) | nib;
+            cword |= code << (4 * (k ^ 1));
+        }
+        cout[i] = cword;
+        rout[i] = rword;
+    }
+}
+
 __global__ __launch_bounds__(256) void latent_requant_kernel(const u32x4_t *__restrict__ latent,
                                                              const unsigned short *__restrict__ scales,
                                                              const unsigned short *__restrict__ zeros,
@@ -60,20 +80,9 @@ __global__ __launch_bounds__(256) void latent_requant_kernel(const u32x4_t *__re
     const bool fast = (s >= 0x1p-40f) && (s <= 0x1p40f);
     const float r = 1.0f / s;
     u32x4_t cout, rout;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        unsigned cword = 0, rword = 0;
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const float t = (k & 1) ? lq_bf16_hi(in[i][k >> 1]) : lq_bf16_lo(in[i][k >> 1]);
-            unsigned nib, code;
-            lq_latent_requant_elem(t, s, z, r, fast, p, nib, code);
-            rword = (rword << 4) | nib;
-            cword |= code << (4 * (k ^ 1));
-        }
-        cout[i] = cword;
-        rout[i] = rword;
-    }
+    // one branch per thread (a thread's 32 elements share their group's scale)
+    if (fast) requant_thread<true>(in, s, z, r, p, cout, rout);
+    else requant_thread<false>(in, s, z, r, p, cout, rout);
     codes[L] = cout;
     residual[L] = rout;
 }

@@ -24,20 +24,16 @@ __device__ __forceinline__ float lq_latent_value(unsigned code, float value_bf16
 
 // One element of the re-quantiser: Z = bf16(bf16(t / s) + z), q = rint(Z), residual nibble and
 // carry from bf16(Z - q), code = clamp(bf16(q + carry), 0, 15).
-// t / s is correctly rounded: for 2^-40 <= s <= 2^40 (fast) the quotient comes from the correctly
-// rounded reciprocal r (q0 = t*r, e = t - q0*s exactly, q = q0 + e*r: three operations instead of a
-// division sequence); |t| is clamped to 2^60 first, which keeps t*r finite and changes nothing
-// downstream (any |Z| >= 2^20 is an integer in bf16: zero residual, saturated code).
-__device__ __forceinline__ void lq_latent_requant_elem(float t, float s, float z, float r, bool fast, const CodecParams &pq,
+// Only bf16(t / s) is needed, and t and s are bf16 numbers: their quotient keeps a relative distance of at
+// least 2^-17 from every bf16 rounding tie (a tie has a 9-bit odd significand, and s * tie = t has no solution
+// with t below 2^8), so for 2^-40 <= s <= 2^40 (kFast; the caller branches once per group) the product
+// t * RN(1/s), which is within 2^-23 of the quotient, rounds to the same bf16 number. Where the quotient is a
+// bf16 subnormal that argument fails, and there q = rint(Z) and the residual level (0) are the same either way;
+// infinities and NaN go the same way through the product as through the quotient.
+template <bool kFast>
+__device__ __forceinline__ void lq_latent_requant_elem(float t, float s, float z, float r, const CodecParams &pq,
                                                        unsigned &nib, unsigned &code) {
-    float quo;
-    if (fast && t == t) {
-        const float tc = __builtin_amdgcn_fmed3f(t, -0x1p60f, 0x1p60f);
-        const float q0 = tc * r;
-        quo = fmaf(fmaf(-q0, s, tc), r, q0);
-    } else {
-        quo = t / s;
-    }
+    const float quo = kFast ? t * r : t / s;
     const float Z = lq_bf16r(lq_bf16r(quo) + z);
     const float q = rintf(Z);  // round half to even, as torch.round
     const float f = lq_bf16r(Z - q);

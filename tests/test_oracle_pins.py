@@ -536,3 +536,50 @@ def test_deterministic_uniform_quantiser_known_answers():
         lv = int(math.floor(abs(t) + Fraction(1, 2))) * (1 if t >= 0 else -1)
         want = (1, 1) if lv > 7 else (lv + 8, 0)
         assert (nib[i], int(carry[i])) == want, (float(v), lv)
+
+
+def test_fp32_quotient_of_bf16_numbers_from_one_residual_correction():
+    """The fused Adam kernels form m / d for bf16 m and d as q0 = m r, q = q0 + (m - q0 d) r with the hardware's
+    reciprocal r (within one ulp of 1/d) and need the IEEE quotient. Every pair of 8-bit significands, r taken
+    as RN(1/d) and as its two neighbours, in exact rational arithmetic: q equals RN(m/d); and the quotient's
+    distance from the nearest midpoint of two fp32 numbers is at least 2^-33 (relative)."""
+    from fractions import Fraction
+
+    def rn32(fr):  # exact rational -> nearest fp32 (ties to even), as a Fraction; normal range only
+        if fr == 0:
+            return Fraction(0)
+        sgn, a = (1 if fr > 0 else -1), abs(fr)
+        e = a.numerator.bit_length() - a.denominator.bit_length()
+        if Fraction(2) ** e > a:
+            e -= 1
+        scale = Fraction(2) ** (e - 23)
+        n = a / scale  # in [2^23, 2^24)
+        lo = n.numerator // n.denominator
+        rem = n - lo
+        if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and lo % 2 == 1):
+            lo += 1
+        return sgn * lo * scale
+
+    worst = Fraction(1)
+    for mi in range(128, 256):
+        for di in range(128, 256, 1):
+            m, d = Fraction(mi, 128), Fraction(di, 128) * 4  # the exponents only scale the result
+            exact = m / d
+            want = rn32(exact)
+            r0 = rn32(1 / d)
+            ulp_r = Fraction(2) ** (-23 - 3)  # ulp of a number in [1/8, 1/4)... r in (1/8, 1/4]
+            for r in (r0 - ulp_r, r0, r0 + ulp_r):
+                q0 = rn32(m * r)
+                q = rn32(q0 + (m - q0 * d) * r)
+                assert q == want, (mi, di, float(r - r0))
+            # distance of the exact quotient from the nearest fp32 midpoint, relative
+            e = exact.numerator.bit_length() - exact.denominator.bit_length()
+            if Fraction(2) ** e > exact:
+                e -= 1
+            half = Fraction(2) ** (e - 24)
+            n = exact / half  # midpoints are the odd integers here
+            lo = n.numerator // n.denominator
+            for t in (lo, lo + 1):
+                if t % 2 == 1:
+                    worst = min(worst, abs(n - t) * half / exact)
+    assert worst >= Fraction(1, 2 ** 33), float(worst)
