@@ -125,3 +125,23 @@ def test_deterministic_uniform_quantiser_bit_exact(dtype):
     deq = Q.cuda_dequant_linear(q).reshape(-1).float().cpu()
     keep = (want_c == 0) & (x.abs().to(torch.float32).numpy() <= 1.0)
     assert float((deq.numpy()[keep] - x.to(torch.float32).numpy()[keep]).__abs__().max()) <= 0.0625 + 1e-6
+
+
+@pytest.mark.parametrize("mode,mu", [(0, 0), (0, 1), (0, 2), (0, 3), (1, 0)])
+def test_residual_codec_every_bf16_input(ops, mode, mu):
+    """All 65 536 bf16 bit patterns (in range, out of range, infinities, NaN) through the codec kernel: packed words
+    and carry flags equal the C restatement's, for the four three-segment curves and the uniform mode."""
+    from oracle import c_oracle as co
+    p1, y1, p2, y2 = CURVES[mu]
+    args = (0, p1, y1, p2 - p1, y2, 8 - p2) if mode == 0 else (1,)
+    xb = np.arange(65536, dtype=np.uint16)
+    want_q, want_c = co.residual_quant(xb.copy(), *args)
+    x = torch.from_numpy(xb.view(np.int16).copy()).view(torch.bfloat16).cuda()
+    q = torch.empty(65536 // 8, dtype=torch.int32, device="cuda")
+    ops.residual_quant(x, q, *args)
+    torch.cuda.synchronize()
+    got_q = q.cpu().numpy().view(np.uint32)
+    got_c = x.cpu().view(torch.int16).numpy().view(np.uint16)
+    bad = np.nonzero(got_q != want_q)[0]
+    assert bad.size == 0, [(hex(int(w) * 8), hex(int(got_q[w])), hex(int(want_q[w]))) for w in bad[:5]]
+    assert np.array_equal(got_c, want_c)

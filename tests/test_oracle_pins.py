@@ -583,3 +583,33 @@ def test_fp32_quotient_of_bf16_numbers_from_one_residual_correction():
                 if t % 2 == 1:
                     worst = min(worst, abs(n - t) * half / exact)
     assert worst >= Fraction(1, 2 ** 33), float(worst)
+
+
+def test_round_half_away_as_trunc_of_a_sum():
+    """The codec kernels take roundf(x) (halves away from zero) as trunc(x + copysign(pred(0.5), x)) in fp32.
+    The same expression in numpy against the definition on 2^26 floats: every float in [0, 4), the neighbourhoods of
+    all half-integers up to 2^12, of 2^22, 2^23 and 2^24, both signs, zeros, infinities."""
+    half = np.float32(0.49999997)
+    assert half == np.nextafter(np.float32(0.5), np.float32(0))
+
+    def trick(x):
+        return np.trunc((x + np.copysign(half, x)).astype(np.float32))
+
+    def want(x):  # floor(|x| + 1/2) with the sign of x, exact in float64
+        a = np.abs(x.astype(np.float64))
+        return np.copysign(np.floor(a + 0.5), x).astype(np.float32)
+
+    dense = np.arange(0, np.float32(4.0).view(np.uint32) + 1, dtype=np.uint32).view(np.float32)  # all floats in [0, 4]
+    parts = [dense[::1] if len(dense) < (1 << 26) else dense[:: len(dense) >> 25]]
+    for k in range(0, 4097):
+        c = np.float32(k + 0.5).view(np.uint32)
+        parts.append(np.arange(int(c) - 40, int(c) + 41, dtype=np.int64).astype(np.uint32).view(np.float32))
+    for big in (2.0 ** 22, 2.0 ** 23, 2.0 ** 24, 3.0e38):
+        c = np.float32(big).view(np.uint32)
+        parts.append(np.arange(int(c) - 2000, int(c) + 2001, dtype=np.int64).astype(np.uint32).view(np.float32))
+    parts.append(np.array([0.0, -0.0, np.inf, -np.inf, 0.5, 1.5, 2.5, 0.49999997, 0.50000006], np.float32))
+    x = np.concatenate(parts)
+    x = np.concatenate([x, -x])
+    x = x[np.isfinite(x) | np.isinf(x)]
+    got, ref = trick(x), want(x)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), x[got.view(np.uint32) != ref.view(np.uint32)][:10]
