@@ -155,3 +155,44 @@ def test_requant_and_a8w8_replay(ops):
             assert torch.equal(out, wc) and torch.equal(y8[0], wy), f"pass {rep}"
             ops.requant_sr(p, sc, z, grads[0], 1e-2, (N, K), seed=1, offset=0)  # eager work in between
             torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("M", [3, 16, 300])
+def test_fused_gate_up_replays_match_eager(ops, M):
+    """lq_a16w4_gate_up_silu (the GEMV pass over both matrices for up to 16 tokens, the MFMA kernel above) followed
+    by the down projection, captured once and replayed on fresh inputs."""
+    hid, ffn = 512, 1408
+    gate = [dev(t) for t in make_w4(ffn, hid, 1)[1:]]
+    up = [dev(t) for t in make_w4(ffn, hid, 2)[1:]]
+    down = [dev(t) for t in make_w4(hid, ffn, 3)[1:]]
+    x = torch.zeros(M, hid, dtype=torch.bfloat16, device="cuda")
+    h = torch.empty(M, ffn, dtype=torch.bfloat16, device="cuda")
+    y = torch.empty(M, hid, dtype=torch.bfloat16, device="cuda")
+
+    def step():
+        ops.a16w4_gate_up_silu(x, gate, up, (ffn, hid), out=h)
+        ops.a16w4_forward(h, *down, (hid, ffn), out=y)
+
+    inputs = [dev(randn_bf16((M, hid), 30 + i)) for i in range(3)]
+    want = []
+    for xi in inputs:
+        x.copy_(xi)
+        step()
+        want.append(y.clone())
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(s):
+        step()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(g, stream=s):
+            step()
+    torch.cuda.synchronize()
+    for i in (2, 0, 1, 2):
+        x.copy_(inputs[i])
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want[i]), f"replay with input {i} differs from the eager result"
+        _ = (x.float() @ x.float().t()).sum().item()  # eager work between replays
