@@ -39,7 +39,8 @@ __device__ __forceinline__ void lq_latent_requant_elem(float t, float s, float z
     const float f = lq_bf16r(Z - q);
     bool carry;
     nib = nibble_of(level_3fold(f, pq), carry);
-    float c = lq_bf16r(q + (carry ? 1.0f : 0.0f));
-    c = fminf(fmaxf(c, 0.0f), 15.0f);
-    code = (unsigned)c & 0xFu;
+    // clamp(bf16(q + carry), 0, 15): q + carry is an integer, bf16 keeps every integer up to 256 and is
+    // monotonic, so the rounding cannot change what the clamp returns; a NaN ends as code 0
+    const float c = __builtin_amdgcn_fmed3f(fmaxf(q + (carry ? 1.0f : 0.0f), 0.0f), 0.0f, 15.0f);
+    code = (unsigned)c;
 }

@@ -42,13 +42,14 @@ __device__ __forceinline__ float level_uniform(float x) {
     return lq_round_half_away(fmaf(x, 8.0f, v));
 }
 
-// float level -> (nibble, carry). Negative values below -8 saturate to nibble 0 like the
-// float->unsigned conversion of the reference's target.
+// float level -> (nibble, carry). Levels below -8 (and NaN) give nibble 0: v_cvt_u32_f32 saturates negative
+// inputs to 0 and converts NaN to 0, which is what the float->unsigned conversion of the reference's target does
+// as well. Without a carry the level is at most 7, so level + 8 fits the nibble; the mask keeps wild inputs in it.
 __device__ __forceinline__ unsigned nibble_of(float lv, bool &carry) {
     carry = lv > 7.5f;
-    if (carry) return 1u;
-    const float t = lv + 8.0f;
-    return t > 0.0f ? ((unsigned)t & 0xFu) : 0u;
+    unsigned t;
+    asm("v_cvt_u32_f32 %0, %1" : "=v"(t) : "v"(lv + 8.0f));
+    return carry ? 1u : (t & 0xFu);
 }
 
 // nibble - 8 -> value of the three-segment curve (inverse slopes in p), branch-free
