@@ -42,10 +42,11 @@
 // barriers and the compiler's wait insertion never sees them; they are spread over the step, one
 // kind per half-slice.
 //
-// The chip is power-limited on this kernel (the shader clock sits near 1.35 GHz while it runs,
-// against 2.1 GHz for a loop of MFMAs on constant operands), so what the loop does besides MFMAs
-// costs throughput even where it overlaps them in time: the forms of the loads above are chosen to
-// keep the bytes moved between L2 and the CU near the bytes used.
+// The chip is power-limited on this kernel (under sustained load the shader clock sits at 1.64 GHz with two
+// workgroups per compute unit and at 2.0 GHz with one, against 1.81 GHz for a loop of nothing but MFMAs on
+// random operands and 2.38 GHz on all-zero ones; lq_calib_gemm_clocks and lq_calib_mfma_loop measure this), so
+// what the loop does besides MFMAs costs throughput even where it overlaps them in time: the forms of the loads
+// above are chosen to keep the bytes moved between L2 and the CU near the bytes used.
 #include "lq_common.h"
 
 #include <type_traits>
