@@ -421,6 +421,20 @@ def bench_gate_up(device, blk):
     return out
 
 
+def bench_c0(device):
+    """configs[0] (the reference's own CPU-runnable case: 3072 x 768 at 1024 tokens) on the GPU: forward and dX."""
+    from latentq_llm_amd import ops
+    N0, K0, M0 = 3072, 768, 1024
+    w = synth_w4(N0, K0, 5, device)
+    x = torch.randn(M0, K0, device=device).to(torch.bfloat16)
+    dy = torch.randn(M0, N0, device=device).to(torch.bfloat16)
+    tf = graph_time([lambda: ops.a16w4_forward(x, *w, (N0, K0))] * 8)
+    td = graph_time([lambda: ops.a16w4_dx(dy, *w, (N0, K0))] * 8)
+    flop = 2.0 * M0 * N0 * K0
+    return {"workload": "configs[0]: 3072x768 at 1024 tokens", "fwd_us": tf * 1e6, "dx_us": td * 1e6,
+            "TFLOP/s": 2 * flop / (tf + td) / 1e12, "plans": [ops.a16w4_plan(M0, (N0, K0))[0], ops.a16w4_plan(M0, (N0, K0), backward=True)[0]]}
+
+
 def bench_copy(device):
     """Plain streaming copy (lq_calib_copy) over buffers larger than the last-level cache: the
     HBM rate this device sustains for read + write traffic, for comparison with the 8 TB/s peak."""
@@ -700,6 +714,7 @@ def main():
         line["gate_up_silu"] = bench_gate_up(dev, blk)
         del blk
         torch.cuda.empty_cache()
+        line["c0"] = bench_c0(dev)
         line["requant"] = bench_requant(dev)
         line["gradq8"] = bench_gradq8(dev)
         line["latent_lbit4"] = bench_latent(dev)
