@@ -26,7 +26,47 @@ __global__ __launch_bounds__(256) void dequant_kernel(const unsigned *__restrict
     out[w] = o;
 }
 
+// byte SEL of `old` replaced by sat_u8(rne(v)) (v_cvt_pk_u8_f32: saturates to 0..255, NaN -> 0)
+template <int SEL>
+__device__ __forceinline__ unsigned act_cvt_pk_u8(float v, unsigned old) {
+    unsigned r;
+    asm("v_cvt_pk_u8_f32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "n"(SEL), "v"(old));
+    return r;
+}
+
 // x8 = clamp(rne(bf16(bf16(x * 127) / clampv)), -128, 127); 8 elements per thread.
+// The clamp value is the maximum of a bf16 tensor in every use the reference makes of it, i.e. a bf16 number;
+// the quotient of two bf16 numbers keeps 2^-17 (relative) from every bf16 rounding tie, so bf16(a / c) is
+// bf16(a * RN(1/c)) (kFast: c has no bits below bf16's and 2^-40 <= |c| <= 2^40; decided once per launch's
+// uniform value, any other clamp value takes the division). clamp(rint(q), -128, 127) is sat_u8(rne(q + 128)) - 128:
+// q is a bf16 number, so the sum is exact wherever it matters. A NaN becomes 0 (what the tensor library's
+// float -> int8 conversion makes of it); the byte conversion would make it -128, so 8 inputs with a NaN among
+// them take the slow form.
+template <bool kFast>
+__device__ __forceinline__ u32x2_t act_quant8(const u32x4_t v, float c, float r) {
+    unsigned w[2] = {0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float f = (j & 1) ? lq_bf16_hi(v[j >> 1]) : lq_bf16_lo(v[j >> 1]);
+        const float a = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(f * 127.0f));
+        if (kFast) {
+            const float q = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(a * r)) + 128.0f;
+            switch (j & 3) {
+                case 0: w[j >> 2] = act_cvt_pk_u8<0>(q, w[j >> 2]); break;
+                case 1: w[j >> 2] = act_cvt_pk_u8<1>(q, w[j >> 2]); break;
+                case 2: w[j >> 2] = act_cvt_pk_u8<2>(q, w[j >> 2]); break;
+                default: w[j >> 2] = act_cvt_pk_u8<3>(q, w[j >> 2]); break;
+            }
+        } else {
+            const float q = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(a / c));
+            const float rr = q == q ? __builtin_amdgcn_fmed3f(rintf(q), -128.0f, 127.0f) : 0.0f;
+            w[j >> 2] |= ((unsigned)(int)rr & 0xFFu) << (8 * (j & 3));
+        }
+    }
+    if (kFast) return u32x2_t{w[0] ^ 0x80808080u, w[1] ^ 0x80808080u};
+    return u32x2_t{w[0], w[1]};
+}
+
 __global__ __launch_bounds__(256) void act_quant_kernel(const unsigned short *__restrict__ x,
                                                         const float *__restrict__ clampv, signed char *__restrict__ x8,
                                                         long long n) {
@@ -34,25 +74,22 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const unsigned short *__
     const long long base = ((long long)blockIdx.x * 256 + threadIdx.x) * 8;
     if (base >= n) return;
     if (base + 8 <= n && (((uintptr_t)(x + base)) & 15) == 0 && (((uintptr_t)(x8 + base)) & 7) == 0) {
-        u32x4_t v = *reinterpret_cast<const u32x4_t *>(x + base);
-        unsigned r[2] = {0u, 0u};
+        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(x + base);
+        const bool c_is_bf16 = (__float_as_uint(c) & 0xFFFFu) == 0u && fabsf(c) >= 0x1p-40f && fabsf(c) <= 0x1p40f;
+        // a NaN among the 8 inputs: the two forms differ on it (see above)
+        bool any_nan = false;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            float f = (j & 1) ? lq_bf16_hi(v[j >> 1]) : lq_bf16_lo(v[j >> 1]);
-            float a = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(f * 127.0f));
-            float q = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(a / c));
-            float rr = __builtin_amdgcn_fmed3f(rintf(q), -128.0f, 127.0f);
-            int iv = (int)rr;
-            r[j >> 2] |= ((unsigned)iv & 0xFFu) << (8 * (j & 3));
-        }
-        u32x2_t o = {r[0], r[1]};
+        for (int j = 0; j < 4; ++j) any_nan |= (v[j] & 0x7FFFu) > 0x7F80u || (v[j] & 0x7FFF0000u) > 0x7F800000u;
+        u32x2_t o;
+        if (c_is_bf16 && !any_nan) o = act_quant8<true>(v, c, 1.0f / c);
+        else o = act_quant8<false>(v, c, 0.0f);
         *reinterpret_cast<u32x2_t *>(x8 + base) = o;
     } else {
         for (long long i = base; i < n && i < base + 8; ++i) {
             float f = lq_bf16_bits_to_f32(x[i]);
             float a = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(f * 127.0f));
             float q = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(a / c));
-            float rr = __builtin_amdgcn_fmed3f(rintf(q), -128.0f, 127.0f);
+            float rr = q == q ? __builtin_amdgcn_fmed3f(rintf(q), -128.0f, 127.0f) : 0.0f;
             x8[i] = (signed char)(int)rr;
         }
     }

@@ -364,12 +364,20 @@ def test_a8w8_extreme_accumulators(ops, co):
     assert int(acc[0, 0]) == 127 * 127 * 8192 and int(acc[0, 1]) == -127 * 127 * 8192
 
 
-def test_act_quant_bit_exact(ops, co):
-    x = randn_bf16((333, 77), 1, 2.0)
-    clampv = float(x.max())
+@pytest.mark.parametrize("shape,clamp", [((333, 77), None), ((2048, 1024), None), ((64, 128), 3.14159), ((64, 128), 1e-30),
+                                         ((64, 128), -2.0), ((40, 8), 0.0)])
+def test_act_quant_bit_exact(ops, co, shape, clamp):
+    """The tensor's own maximum as clamp value (a bf16 number: the reciprocal-product form), clamp values that are not
+    bf16 numbers, tiny, negative or zero (the division form), with NaN and infinities among the inputs."""
+    x = randn_bf16(shape, 1, 2.0)
+    clampv = float(x.max()) if clamp is None else clamp
+    x.view(-1)[5] = float("nan")
+    x.view(-1)[17] = float("inf")
+    x.view(-1)[18] = float("-inf")
+    x.view(-1)[19] = 3e38
     got = ops.act_quant_i8(dev(x), torch.tensor([clampv], device="cuda")).cpu().numpy()
     want = co.act_quant_i8(bits(x), clampv).reshape(got.shape)
-    assert np.array_equal(got, want)
+    assert np.array_equal(got, want), np.nonzero(got != want)[0][:10]
 
 
 # ------------------------------------------------------------------ repack --
