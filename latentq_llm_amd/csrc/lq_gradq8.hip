@@ -10,8 +10,9 @@
 // draw b of the element: byte i & 3 of word (i >> 2) & 3 of Philox4x32-10(counter = offset + i / 16,
 // key = seed), i the flat element index. The 256 values are bf16 numbers, symmetric about zero.
 //
-// One workgroup per row: the row's absolute maximum needs the whole row before its first element can
-// be quantised, and a second read of an 8-22 KB row by the workgroup that just read it stays in L2.
+// A row belongs to one workgroup (to 64, 128 or 256 of its threads): the row's absolute maximum needs the whole
+// row before its first element can be quantised; rows of up to 12 288 elements stay in registers in between,
+// longer ones are read a second time (from L2).
 #include "lq_common.h"
 
 namespace {
@@ -77,24 +78,30 @@ __device__ __forceinline__ float absmax8(const u32x4_t v, float m) {
     return m;
 }
 
-// One workgroup per row, a thread takes 16 consecutive elements per step of 4096. kPieces > 0: the row has at
-// most kPieces * 4096 elements and a thread keeps its pieces in registers between the maximum and the
-// quantisation; 0: any K, the row is read a second time (from L2).
-template <bool kPhilox, bool kAcc, int kPieces>
+// T threads per row (64, 128 or 256: short rows get a wave or two instead of a mostly idle workgroup, 256 / T rows
+// per workgroup); a thread takes 16 consecutive elements per step of 16 T. kPieces > 0: the row has at most
+// kPieces * 16 T elements and a thread keeps its pieces in registers between the maximum and the quantisation;
+// 0: any K, the row is read a second time (from L2).
+template <bool kPhilox, bool kAcc, int kPieces, int T>
 __global__ __launch_bounds__(256) void gradq8_kernel(const unsigned short *__restrict__ dw, signed char *__restrict__ q,
                                                      unsigned short *__restrict__ scale, const unsigned short *__restrict__ noise,
-                                                     long long K, unsigned long long seed, unsigned long long offset) {
+                                                     long long N, long long K, unsigned long long seed,
+                                                     unsigned long long offset) {
+    constexpr int R = 256 / T;      // rows per workgroup
+    constexpr int STEP = 16 * T;    // elements of a row the row's threads take per piece
     __shared__ float red[4];
-    const long long n = blockIdx.x;
+    const int tid = threadIdx.x % T;
+    const long long n_raw = (long long)blockIdx.x * R + threadIdx.x / T;
+    const bool live = n_raw < N;    // rows past the end still take part in the barrier
+    const long long n = live ? n_raw : N - 1;
     const unsigned short *row = dw + n * K;
-    const int tid = threadIdx.x;
     const u32x4_t zero4 = {0u, 0u, 0u, 0u};
     constexpr int kHeld = kPieces > 0 ? kPieces : 1;
     u32x4_t h0[kHeld], h1[kHeld], old[kHeld], z0[kHeld], z1[kHeld];
     if (kPieces > 0) {
 #pragma unroll
         for (int i = 0; i < kPieces; ++i) {
-            const long long k = (long long)tid * 16 + (long long)i * 4096;
+            const long long k = (long long)tid * 16 + (long long)i * STEP;
             h0[i] = h1[i] = old[i] = z0[i] = z1[i] = zero4;
             if (k < K) {
                 h0[i] = *reinterpret_cast<const u32x4_t *>(row + k);
@@ -114,28 +121,34 @@ __global__ __launch_bounds__(256) void gradq8_kernel(const unsigned short *__res
 #pragma unroll
             for (int i = 0; i < kPieces; ++i) m = absmax8(h1[i], absmax8(h0[i], m));
         } else {
-            for (long long k = (long long)tid * 16; k < K; k += 4096)
+            for (long long k = (long long)tid * 16; k < K; k += STEP)
                 m = absmax8(*reinterpret_cast<const u32x4_t *>(row + k + 8), absmax8(*reinterpret_cast<const u32x4_t *>(row + k), m));
         }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-        if ((tid & 63) == 0) red[tid >> 6] = m;
-        __syncthreads();
-        m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        if constexpr (T > 64) {
+            // waves of one row are neighbours: wave w belongs to row group w / (T / 64)
+            const int wave = threadIdx.x >> 6;
+            if ((threadIdx.x & 63) == 0) red[wave] = m;
+            __syncthreads();
+            if constexpr (T == 256) m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+            else m = fmaxf(red[wave & ~1], red[wave | 1]);
+        }
         const float vmax = bf16r(m * 4.0f);
         const float lo = bf16r(1e-5f);
         s = bf16r(fmaxf(vmax, lo) * (1.0f / 127.0f));
-        if (tid == 0) scale[n] = lq_f32_to_bf16_bits(s);
+        if (tid == 0 && live) scale[n] = lq_f32_to_bf16_bits(s);
     } else {
         s = lq_bf16_bits_to_f32(scale[n]);
     }
-    // the scale is the same for the whole workgroup, so this branch does not diverge
+    if (!live) return;
+    // the scale is the same for a whole wave (a wave never spans two rows), so this branch does not diverge
     const bool fast = __builtin_amdgcn_readfirstlane((int)(s >= 0x1p-40f && s <= 0x1p40f)) != 0;
     const float r = 1.0f / s;
     if (kPieces > 0) {
 #pragma unroll
         for (int i = 0; i < kPieces; ++i) {
-            const long long k = (long long)tid * 16 + (long long)i * 4096;
+            const long long k = (long long)tid * 16 + (long long)i * STEP;
             if (k < K) {
                 const long long e0 = n * K + k;
                 const unsigned long long c = offset + (unsigned long long)(e0 >> 4);
@@ -145,7 +158,7 @@ __global__ __launch_bounds__(256) void gradq8_kernel(const unsigned short *__res
             }
         }
     } else {
-        for (long long k = (long long)tid * 16; k < K; k += 4096) {
+        for (long long k = (long long)tid * 16; k < K; k += STEP) {
             const long long e0 = n * K + k;
             const u32x4_t v0 = *reinterpret_cast<const u32x4_t *>(row + k);
             const u32x4_t v1 = *reinterpret_cast<const u32x4_t *>(row + k + 8);
@@ -166,14 +179,16 @@ __global__ __launch_bounds__(256) void gradq8_kernel(const unsigned short *__res
 template <bool kPhilox, bool kAcc>
 void launch_gradq8(const void *dw, int8_t *q, void *scale, const void *noise, int64_t N, int64_t K, uint64_t seed,
                    uint64_t offset, hipStream_t st) {
-    const dim3 grid((unsigned)N), block(256);
-#define LQ_GRADQ8_LAUNCH(P)                                                                                         \
-    hipLaunchKernelGGL((gradq8_kernel<kPhilox, kAcc, P>), grid, block, 0, st, (const unsigned short *)dw,           \
-                       (signed char *)q, (unsigned short *)scale, (const unsigned short *)noise, (long long)K,      \
-                       (unsigned long long)seed, (unsigned long long)offset)
-    if (K <= 4096) LQ_GRADQ8_LAUNCH(1);
-    else if (K <= 3 * 4096) LQ_GRADQ8_LAUNCH(3);
-    else LQ_GRADQ8_LAUNCH(0);
+#define LQ_GRADQ8_LAUNCH(P, T)                                                                                        \
+    hipLaunchKernelGGL((gradq8_kernel<kPhilox, kAcc, P, T>), dim3((unsigned)((N + 256 / T - 1) / (256 / T))), dim3(256), 0, \
+                       st, (const unsigned short *)dw, (signed char *)q, (unsigned short *)scale,                     \
+                       (const unsigned short *)noise, (long long)N, (long long)K, (unsigned long long)seed,           \
+                       (unsigned long long)offset)
+    if (K <= 1024) LQ_GRADQ8_LAUNCH(1, 64);
+    else if (K <= 2048) LQ_GRADQ8_LAUNCH(1, 128);
+    else if (K <= 4096) LQ_GRADQ8_LAUNCH(1, 256);
+    else if (K <= 3 * 4096) LQ_GRADQ8_LAUNCH(3, 256);
+    else LQ_GRADQ8_LAUNCH(0, 256);
 #undef LQ_GRADQ8_LAUNCH
 }
 

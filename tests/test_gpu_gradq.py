@@ -34,7 +34,7 @@ def _noise(shape, seed):
 
 
 @pytest.mark.parametrize("N,K,std", [(1, 16, 1.0), (7, 144, 1e-3), (33, 2048, 0.02), (16, 4112, 5.0), (4, 11008, 1e-6),
-                                     (3, 12304, 0.3)])
+                                     (3, 12304, 0.3), (5, 4096, 0.1), (9, 1040, 2.0), (6, 1024, 1e-2)])
 @pytest.mark.parametrize("mode", ["inject", "philox"])
 def test_gradq8_set_and_add_bit_exact(ops, N, K, std, mode):
     dws = [randn_bf16((N, K), 50 + i, std) for i in range(3)]
