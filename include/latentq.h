@@ -193,6 +193,14 @@ int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const float *sw,
  * x8: int8[n]. */
 int lq_act_quant_i8(const void *x, const float *clampv_dev, int8_t *x8, int64_t n, void *stream);
 
+/* Per-channel int8 re-quantiser of the latent weight of an 8-bit-weight layer: the reference's
+ * Qfunc_8bit_res (utils/quant.py:88-103) for a latent kept as a plain tensor (lbit 0, 16, 32), called
+ * from MyAdam.update_step (:1141):
+ *   codes[n,k] = clamp(round_half_even(bf16(latent[n,k] / qscales[n])), -128, 127)      NaN -> 0
+ * latent: bf16[N,K], 16-byte aligned; qscales: bf16[N]; codes: int8[N,K], 8-byte aligned; K % 8 == 0.
+ * (With a 4-bit residual codec, lbit = 4, the layer keeps the reference's chain of tensor operations.) */
+int lq_w8_requant(const void *latent, const void *qscales, int8_t *codes, int64_t N, int64_t K, void *stream);
+
 /* ---------------------------------------------------------------------------
  * 4-bit residual codec of the latent weight (exact lbit = 4 mode).
  *

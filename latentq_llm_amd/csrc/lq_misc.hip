@@ -95,6 +95,50 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const unsigned short *__
     }
 }
 
+// Per-channel int8 re-quantiser of an 8-bit-weight layer's latent (the reference's Qfunc_8bit_res without a
+// residual codec, utils/quant.py:88-103): code = clamp(rint(bf16(t / qs[n])), -128, 127) for the bf16 latent t
+// and the bf16 scale of its row. Same arithmetic as act_quant8: for 2^-40 <= |qs| <= 2^40 the quotient of the two
+// bf16 numbers is their reciprocal product, and rounding, clamp and byte insertion are one instruction; rows
+// with another scale, and pieces with a NaN (which becomes 0), take the written-out form.
+__global__ __launch_bounds__(256) void w8_requant_kernel(const u32x4_t *__restrict__ latent,
+                                                         const unsigned short *__restrict__ qscales,
+                                                         u32x2_t *__restrict__ codes, long long n_pieces, long long K8) {
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;  // 8 consecutive elements of one row
+    if (i >= n_pieces) return;
+    const float c = lq_bf16_bits_to_f32(qscales[i / K8]);
+    const u32x4_t v = latent[i];
+    bool any_nan = false;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) any_nan |= (v[j] & 0x7FFFu) > 0x7F80u || (v[j] & 0x7FFF0000u) > 0x7F800000u;
+    const bool fast = fabsf(c) >= 0x1p-40f && fabsf(c) <= 0x1p40f && !any_nan;
+    unsigned w[2] = {0u, 0u};
+    if (fast) {
+        const float r = 1.0f / c;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float t = (j & 1) ? lq_bf16_hi(v[j >> 1]) : lq_bf16_lo(v[j >> 1]);
+            const float q = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(t * r)) + 128.0f;
+            switch (j & 3) {
+                case 0: w[j >> 2] = act_cvt_pk_u8<0>(q, w[j >> 2]); break;
+                case 1: w[j >> 2] = act_cvt_pk_u8<1>(q, w[j >> 2]); break;
+                case 2: w[j >> 2] = act_cvt_pk_u8<2>(q, w[j >> 2]); break;
+                default: w[j >> 2] = act_cvt_pk_u8<3>(q, w[j >> 2]); break;
+            }
+        }
+        w[0] ^= 0x80808080u;
+        w[1] ^= 0x80808080u;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float t = (j & 1) ? lq_bf16_hi(v[j >> 1]) : lq_bf16_lo(v[j >> 1]);
+            const float q = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(t / c));
+            const float rr = q == q ? __builtin_amdgcn_fmed3f(rintf(q), -128.0f, 127.0f) : 0.0f;
+            w[j >> 2] |= ((unsigned)(int)rr & 0xFFu) << (8 * (j & 3));
+        }
+    }
+    codes[i] = u32x2_t{w[0], w[1]};
+}
+
 __device__ __forceinline__ unsigned swap_nibbles(unsigned g) {
     return ((g & 0x0F0F0F0Fu) << 4) | ((g >> 4) & 0x0F0F0F0Fu);
 }
@@ -146,6 +190,18 @@ extern "C" int lq_act_quant_i8(const void *x, const float *clampv_dev, int8_t *x
     hipLaunchKernelGGL(act_quant_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                        (const unsigned short *)x, clampv_dev, (signed char *)x8, (long long)n);
     return lq_check_launch("lq_act_quant_i8");
+}
+
+extern "C" int lq_w8_requant(const void *latent, const void *qscales, int8_t *codes, int64_t N, int64_t K, void *stream) {
+    LQ_REQUIRE(latent && qscales && codes, "lq_w8_requant: null pointer argument");
+    LQ_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && N * K / 8 / 256 < 0x7FFFFFFFll,
+               "lq_w8_requant: need N > 0 and K a positive multiple of 8 (N=%lld K=%lld)", (long long)N, (long long)K);
+    LQ_REQUIRE(lq_aligned(latent, 16) && lq_aligned(codes, 8) && lq_aligned(qscales, 2),
+               "lq_w8_requant: latent must be 16-byte, codes 8-byte aligned");
+    const long long pieces = N * K / 8;
+    hipLaunchKernelGGL(w8_requant_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const u32x4_t *)latent, (const unsigned short *)qscales, (u32x2_t *)codes, pieces, (long long)(K / 8));
+    return lq_check_launch("lq_w8_requant");
 }
 
 static int repack_common(const void *src, void *dst, int64_t N, int64_t K, void *stream, bool to_native, const char *who) {

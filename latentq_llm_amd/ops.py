@@ -238,6 +238,19 @@ def a16w4_dequant(codes, scales, zeros, shape):
     return w
 
 
+def w8_requant(latent, qscales):
+    """int8 codes of a bf16 latent weight [N, K] with one bf16 scale per row (lq_w8_requant)."""
+    _chk(latent, torch.bfloat16, "latent")
+    _chk(qscales, torch.bfloat16, "qscales")
+    if latent.dim() != 2 or qscales.numel() != latent.shape[0]:
+        raise ValueError("latent must be [N, K] and qscales hold N entries")
+    N, K = latent.shape
+    out = torch.empty((N, K), dtype=torch.int8, device=latent.device)
+    with torch.cuda.device(latent.device):
+        _C.call("lq_w8_requant", latent.data_ptr(), qscales.data_ptr(), out.data_ptr(), N, K, _stream(latent))
+    return out
+
+
 def a8w8_forward(x8, w8, sx, sw, bias=None, want_acc: bool = False):
     """bf16 Y = ((int32 X8.W8^T) * sx[m]) * sw[n] (+ bias); optionally also the int32 accumulators."""
     _chk(x8, torch.int8, "x8")

@@ -140,6 +140,14 @@ def Qfunc_4bit_g_res(tensor, residual_handle, qparam, groupsize=GROUPSIZE):
 def Qfunc_8bit_res(tensor, residual_handle, qscales):
     """Per-channel int8 re-quantizer with residual memory (utils/quant.py:88-103)."""
     shape = tensor.shape
+    if (FUSED_LATENT and not isinstance(residual_handle, ResidualTensor) and tensor.is_cuda and tensor.dim() == 2
+            and tensor.dtype == torch.bfloat16 and tensor.is_contiguous() and tensor.shape[1] % 8 == 0
+            and tensor.data_ptr() % 16 == 0 and torch.is_tensor(qscales) and qscales.dtype == torch.bfloat16
+            and qscales.is_contiguous() and qscales.numel() == tensor.shape[0]):
+        # the chain below as one pass (same roundings)
+        if residual_handle is not None:
+            residual_handle.data = tensor.to(residual_handle.dtype)
+        return ops.w8_requant(tensor, qscales)
     q = tensor / qscales
     q.round_()
     if isinstance(residual_handle, ResidualTensor):

@@ -129,6 +129,14 @@ def requant(packed, scales, zeros, grad, lr, N, K, group=128, u=None, seed=0, of
     return out
 
 
+def w8_requant(latent_bits, qscale_bits, N, K):
+    lat = _c(latent_bits.reshape(-1), np.uint16)
+    qs = _c(qscale_bits.reshape(-1), np.uint16)
+    out = np.empty(N * K, np.int8)
+    lib().lqo_w8_requant(_p(lat), _p(qs), _p(out), C.c_int64(N), C.c_int64(K))
+    return out
+
+
 def gradq8_noise(n, seed, offset=0):
     """The noise lqo_gradq8 draws for flat elements 0..n-1 when none is injected (float32)."""
     out = np.empty(n, np.float32)

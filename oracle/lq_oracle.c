@@ -290,6 +290,23 @@ void lqo_act_quant_i8(const uint16_t *x, float clampv, int8_t *x8, int64_t n) {
     }
 }
 
+/* Qfunc_8bit_res without a residual codec, utils/quant.py:88-103: q = tensor / qscales (a bf16 tensor
+ * operation), q.round_() (half to even), clamp_(-128, 127), .to(int8); a NaN converts to 0. */
+void lqo_w8_requant(const uint16_t *latent, const uint16_t *qscales, int8_t *codes, int64_t N, int64_t K) {
+    for (int64_t n = 0; n < N; ++n) {
+        float c = bf16_to_f32(qscales[n]);
+        for (int64_t k = 0; k < K; ++k) {
+            volatile float quo = bf16_to_f32(latent[n * K + k]) / c;
+            float q = bf16_round(quo);
+            float r = nearbyintf(q);
+            if (r != r) r = 0.0f;
+            if (r < -128.0f) r = -128.0f;
+            if (r > 127.0f) r = 127.0f;
+            codes[n * K + k] = (int8_t)r;
+        }
+    }
+}
+
 /* ------------------------------------------------------- GPTQ layout ---- */
 /* QuantLinearGPTQ.pack, PTQ/quant/quant_linear.py:360-372: qweight[k/8, n]
  * holds code(k, n) at bits 4*(k%8). */

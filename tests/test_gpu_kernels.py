@@ -595,3 +595,21 @@ def test_fused_mlp_module_matches_the_three_layers(hip_lib):
         err = rel_l2(got.float(), want.float())
         print(f"{tokens}: fused MLP vs layer by layer rel_l2={err:.3e}")
         assert err <= REL_L2_TOL
+
+
+@pytest.mark.parametrize("N,K", [(1, 8), (12, 64), (100, 1032), (2048, 8192)])
+def test_w8_requant_bit_exact(ops, co, N, K):
+    """lq_w8_requant against the C restatement of Qfunc_8bit_res: random latents, ties, saturation, infinities, NaN
+    (-> 0), scales of both signs and outside the range in which the kernel multiplies by the reciprocal."""
+    lat = randn_bf16((N, K), N + K, 0.05)
+    qs = (torch.rand(N, 1, generator=torch.Generator().manual_seed(N)) * 1e-3 + 1e-4).to(torch.bfloat16)
+    if N >= 12:
+        qs[3] = -qs[3]
+        qs[4] = 2.0 ** -50
+        qs[5] = 2.0 ** 50
+        lat[5] *= 2.0 ** 55
+        lat[1, 0], lat[1, 1], lat[2, 3] = float("inf"), float("-inf"), float("nan")
+        lat[0, :8] = (torch.tensor([0.5, 1.5, 2.5, -0.5, -1.5, 127.5, -128.5, 300.0]) * qs[0].float()).to(torch.bfloat16)
+    want = co.w8_requant(bits(lat), bits(qs), N, K)
+    got = ops.w8_requant(dev(lat), dev(qs)).cpu().numpy().reshape(-1)
+    assert np.array_equal(got, want), np.nonzero(got != want)[0][:10]

@@ -613,3 +613,19 @@ def test_round_half_away_as_trunc_of_a_sum():
     x = x[np.isfinite(x) | np.isinf(x)]
     got, ref = trick(x), want(x)
     assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), x[got.view(np.uint32) != ref.view(np.uint32)][:10]
+
+
+def test_w8_requant_oracle_matches_torch_bf16_tensor_ops():
+    """Qfunc_8bit_res without a residual codec (utils/quant.py:88-103) as torch runs it on bf16 tensors on the CPU:
+    q = t / qs; q.round_(); q.clamp_(-128, 127).to(int8), against the C restatement, with ties, saturating values
+    and scales of both signs."""
+    N, K = 12, 64
+    lat = randn_bf16((N, K), 3, 0.05)
+    qs = (torch.rand(N, 1, generator=torch.Generator().manual_seed(4)) * 1e-3 + 1e-4).to(torch.bfloat16)
+    qs[3] = -qs[3]
+    lat[0, :8] = (torch.tensor([0.5, 1.5, 2.5, -0.5, -1.5, 127.5, -128.5, 300.0]) * qs[0].float()).to(torch.bfloat16)
+    lat[1, 0] = float("inf")
+    lat[1, 1] = float("-inf")
+    want = (lat / qs).round_().clamp_(-128, 127).to(torch.int8).numpy().reshape(-1)
+    got = co.w8_requant(bits(lat), bits(qs), N, K)
+    assert np.array_equal(got, want)
