@@ -528,6 +528,12 @@ def profile_target(device, which, launches=10):
                 for i in range(launches):
                     w = synth_w4(N, K, 20 + i, device)
                     o.a16w4_forward(x, *w, (N, K))
+        # the fused gate / up product as one GEMV pass over both matrices
+        for M in (1, 16):
+            x = torch.randn(M, HID, device=device).to(torch.bfloat16)
+            for i in range(launches):
+                wg, wu = synth_w4(FFN, HID, 50 + i, device), synth_w4(FFN, HID, 70 + i, device)
+                o.a16w4_gate_up_silu(x, wg, wu, (FFN, HID))
     elif which == "a8w8":
         for (N, K) in [(2048, 2048), (8192, 2048), (2048, 8192)]:
             x8 = torch.randint(-127, 128, (TOKENS, K), device=device, dtype=torch.int8)
