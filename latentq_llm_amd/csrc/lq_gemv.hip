@@ -357,6 +357,11 @@ int lq_gemv_a16w4_launch(const void *x, const void *codes, const void *scales, c
                                                  // wave's loads are then in flight at once
     if (M <= 4) {
         launch_waves<4, 1, 16>(pick_waves(batches, 16), a);
+    } else if (M <= 8) {
+        // 8 staged token rows (8.1 KB of LDS per wave): 8 waves with one 16-row tile, 16 when K has more than 16
+        // batches (measured on 11008 x 4096 / 4096 x 11008 / 8192^2 at 8 tokens: 11.1 / 10.9 / 14.9 us against
+        // 12.1 / 11.8 / 18.5 with 16 staged rows and the two-tile workgroups below)
+        launch_waves<8, 1, 16>(pick_waves(batches, batches > 16 ? 16 : 8), a);
     } else if (N % 32 == 0 && N >= 32 * 256) {
         // many tokens and enough rows for one 32-row workgroup per CU: half the activation traffic;
         // 4 waves = 65 KB of staged activations: two workgroups per CU, all of them resident at once
