@@ -672,7 +672,9 @@ static SplitPlan plan_split(long long M, long long C, int total_steps, size_t ws
         if (per < 8) per = 8;
         S = (total_steps + per - 1) / per;
         if (S < 2) continue;
-        const double est = (big ? pace_big : 0.56) * (per + 3) * (double)((tiles * S + cus - 1) / cus) + 4.0 + 3.0 +
+        // with more than three quarters of the units busy the clock gives ~9 % (as for the unsplit kernels)
+        const double busy = 4 * tiles * S > 3 * cus ? 1.09 : 1.0;
+        const double est = busy * (big ? pace_big : 0.56) * (per + 3) * (double)((tiles * S + cus - 1) / cus) + 4.0 + 3.0 +
                            2.0 * S * M * C * 4 / 5.0e6;
         if (est < best.est_us) {
             best.splits = (int)S; best.steps_per_split = per; best.big = big != 0; best.est_us = est;
@@ -691,8 +693,10 @@ struct W4Plan {
 // (microseconds, measured): the weights-direct kernel (128 x 256 tiles) takes ~0.86 with one
 // workgroup on a compute unit and ~1.45 for two sharing it; the staged kernel ~0.56 per round of
 // 128 x 128 tiles and ~0.88 per round of 256 x 128 tiles (one workgroup per unit and round). The
-// weights-direct kernel with 128 x 128 tiles fits three workgroups on a unit: ~0.74 alone, ~1.23 for
-// two, ~1.38 for three. The weights-direct kernels load scales and zeros four groups at a time: rows
+// weights-direct kernel with 128 x 128 tiles fits three workgroups on a unit: ~0.55-0.61 alone (the
+// more units are busy, the lower the clock: 0.55 up to three quarters of them, 0.61 with all), ~0.74
+// as soon as a few units hold two, ~1.23 for two everywhere, ~1.38 for three; a full round of the
+// staged 128 x 128 tiles likewise takes ~0.66 instead of ~0.56. The weights-direct kernels load scales and zeros four groups at a time: rows
 // must be 4-byte aligned, i.e. the number of groups per row even.
 static W4Plan plan_fwd(long long M, long long N, long long K, size_t ws_bytes, long long cus) {
     W4Plan out;
@@ -701,14 +705,16 @@ static W4Plan plan_fwd(long long M, long long N, long long K, size_t ws_bytes, l
     const double est_direct = (K / LQ_GROUP) % 2 != 0 ? 1e30
                               : 1.45 * (double)(wg_direct / (2 * cus)) + (rem == 0 ? 0.0 : rem <= cus ? 0.86 : 1.45);
     const long long cols = (N + 127) / 128;
-    const double est_small = 0.56 * (double)((((M + 127) / 128) * cols + cus - 1) / cus);
+    const long long tiles_small = ((M + 127) / 128) * cols;
+    const double est_small = tiles_small <= cus && 4 * tiles_small > 3 * cus ? 0.66 : 0.56 * (double)((tiles_small + cus - 1) / cus);
     const double est_big = 0.88 * (double)((((M + 255) / 256) * cols + cus - 1) / cus);
     double est_direct128 = 1e30;
     if ((K / LQ_GROUP) % 2 == 0) {
         const long long wg = lq_gemm_fwd_direct128_workgroups((int)M, (int)N);
         const long long rem128 = wg % (3 * cus);
         const double tail = rem128 == 0 ? 0.0
-                            : rem128 <= cus ? 0.74
+                            : 4 * rem128 <= 3 * cus ? 0.55
+                            : rem128 <= cus ? 0.61
                             : rem128 <= 2 * cus ? 0.74 + 0.49 * (double)(rem128 - cus) / (double)cus
                                                 : 1.38;
         est_direct128 = 1.38 * (double)(wg / (3 * cus)) + tail;

@@ -168,8 +168,11 @@ def test_dispatch_plan_host_logic(hip_lib):
     assert plan(2048, 4096, 11008, backward=True) == ("staged_256x128", 1, 0)
     # an odd number of groups per row rules the weights-direct kernel out
     assert plan(2048, 11008, 4096 + 128)[0] != "direct_128x256"
-    # one round of small tiles beats everything else when it fits
-    assert plan(256, 11008, 4096) == ("staged_128x128", 1, 0)
+    # one workgroup per compute unit: the staged 128 x 128 tiles when K rules the weights-direct kernels out, else
+    # the weights-direct kernel with 128 x 128 tiles (a little faster alone on a unit)
+    assert plan(256, 11008, 4096 + 128) == ("staged_128x128", 1, 0)
+    assert plan(256, 11008, 4096) == ("direct_128x128", 1, 0)
+    assert plan(1024, 4096, 4096) == ("direct_128x128", 1, 0)
     # between one and two rounds of the 128 x 256 tiles the weights-direct kernel with 128 x 128 tiles (three
     # workgroups per compute unit) fills the device better
     for M in (384, 768, 1024, 1536):
