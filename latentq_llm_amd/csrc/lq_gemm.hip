@@ -981,17 +981,22 @@ extern "C" int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const 
     if (lq_gemm_i8_256_workgroups((int)M, (int)N) * 2 > (long long)lq_device_cu_count())
         return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 256, 2, (hipStream_t)stream);
     // the same kernel with 128 x 128 tiles (two workgroups per CU) when there are more of them than
-    // compute units, or when the reduction is short (<= 16 steps: less to set up than the staged
-    // kernel's producer waves); measured 16.0 -> 13.1 us on 2048^3, 40.6 -> 37.0 on 2048 x 4096 x 4096.
-    // A lone workgroup per CU on a long reduction is faster in the staged kernel (41 against 44 us on
-    // 2048 x 2048 x 8192).
-    if (((M + 127) / 128) * ((N + 127) / 128) > (long long)lq_device_cu_count() || K <= 2048)
+    // compute units; measured 40.6 -> 37.0 us on 2048 x 4096 x 4096
+    const long long tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+    const long long cus = lq_device_cu_count();
+    if (tiles128 > cus)
         return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 2, (hipStream_t)stream);
-    // a workgroup with a CU to itself and a long reduction: four 32 KB stages (loads three steps
-    // ahead) instead of two; measured 41 -> 37 us on 2048 x 2048 x 8192, 146 -> 127 on K = 32768, but
-    // slower than the staged kernel below 48 steps (27.5 against 24.2 us at K = 4096)
-    if (K >= 6144)
+    // a workgroup with a CU to itself: four 32 KB stages (loads three steps ahead) instead of two whenever a
+    // quarter of the CUs stay idle (15-17 against 20-22 us for the staged kernel on 128-512 tokens x 4096 x 4096,
+    // 13.9 against 15.8 for two stages on 512 x 6144 x 2048), and on long reductions with every CU busy
+    // (41 -> 37 us on 2048 x 2048 x 8192, 146 -> 127 on K = 32768)
+    if (4 * tiles128 <= 3 * cus || K >= 6144)
         return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 4, (hipStream_t)stream);
+    // every CU busy with one workgroup: two stages for short reductions (<= 16 steps: less to set up than the
+    // staged kernel's producer waves; 16.0 -> 13.1 us on 2048^3), the staged kernel in between (25.3 against
+    // 27.7 us on 1024 x 4096 x 4096)
+    if (K <= 2048)
+        return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 2, (hipStream_t)stream);
     GemmParams p = {};
     p.a = x; p.b = w; p.sx = sx; p.sw = sw; p.bias = (const unsigned short *)bias_or_null; p.c = y;
     p.acc_out = acc_or_null;
