@@ -187,11 +187,41 @@ int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const float *sw,
                 const void *bias_or_null, void *y, int32_t *acc_or_null, int64_t M, int64_t N,
                 int64_t K, void *stream);
 
+/* lq_a8w8_fwd with the per-channel scales as the reference's modules store them: qscales is the bf16[N]
+ * buffer `qscales` of QLinearA8W8 / QLinearQAT (utils/quant.py:496-498), read and widened in the epilogue
+ * (sw[n] = float(qscales[n]), exact), so that a layer's forward needs no conversion pass. */
+int lq_a8w8_fwd_qs(const void *x, const void *w, const float *sx, const void *qscales_bf16,
+                   const void *bias_or_null, void *y, int32_t *acc_or_null, int64_t M, int64_t N,
+                   int64_t K, void *stream);
+
 /* Per-tensor symmetric activation quantizer used in front of lq_a8w8_fwd:
  *   x8 = clamp(round_half_even(x * (127/clampv)), -128, 127)
  * (reference utils/quant.py:264-266). x: bf16[n]; clampv: DEVICE fp32 scalar;
  * x8: int8[n]. */
 int lq_act_quant_i8(const void *x, const float *clampv_dev, int8_t *x8, int64_t n, void *stream);
+
+/* The same quantiser with the clamp value the dynamic layers of the reference use, the maximum of the
+ * activation tensor itself (`clampv = input.max()`, utils/quant.py:259-266, 319-322), found on the device:
+ * two launches, no host synchronisation and no other kernel. A NaN anywhere in x makes the clamp value NaN
+ * (as the tensor library's max does) and every x8 zero.
+ *   clampv = max_i x[i];  x8 as lq_act_quant_i8 with that value;
+ *   sx[m]  = alpha for every m < M, alpha = clampv * fl32(1/127) (how the tensor library divides a tensor by
+ *            the host scalar 127.), rounded to bf16 when alpha_bf16 != 0 (the training Function divides a bf16
+ *            0-dim tensor, :271; the eval Function a host float, :326): the per-row scales lq_a8w8_fwd reads.
+ * x: bf16[M,K], 16-byte aligned; x8: int8[M,K], 8-byte aligned; sx: fp32[M];
+ * work: fp32[LQ_ACT_WORK_FLOATS] device scratch; on return work[0] = clampv and work[1] = alpha (device values). */
+#define LQ_ACT_WORK_FLOATS 1032
+int lq_act_quant_i8_dynamic(const void *x, int8_t *x8, float *sx, float *work, int64_t M, int64_t K, int alpha_bf16,
+                            void *stream);
+
+/* Per-token activation quantiser, one pass: for every token row m
+ *   amax  = max_k |x[m,k]|                         (NaN if the row holds one)
+ *   sx[m] = amax / 127                             (fp32, IEEE division)
+ *   x8[m,k] = clamp(round_half_even(x[m,k] * (127 / amax)), -128, 127)   (fp32; NaN -> 0; an all-zero row: 0)
+ * so that lq_a8w8_fwd's epilogue (acc * sx[m]) * sw[n] is the per-token x per-channel scaling. The reference
+ * quantises per tensor only (utils/quant.py:259-266); this is the per-token form of the same step.
+ * x: bf16[M,K], 16-byte aligned, K % 8 == 0; x8: int8[M,K]; sx: fp32[M]. */
+int lq_act_quant_i8_per_token(const void *x, int8_t *x8, float *sx, int64_t M, int64_t K, void *stream);
 
 /* Per-channel int8 re-quantiser of the latent weight of an 8-bit-weight layer: the reference's
  * Qfunc_8bit_res (utils/quant.py:88-103) for a latent kept as a plain tensor (lbit 0, 16, 32), called
@@ -327,6 +357,14 @@ int lq_transpose_bf16(const void *src, void *dst, int64_t R, int64_t C, void *st
  * counters of a profiler run and gives the copy bandwidth this device sustains.
  * ------------------------------------------------------------------------- */
 int lq_calib_copy(const void *src, void *dst, int64_t nbytes, void *stream);
+
+/* Measurement aid, no counterpart in the reference: a plain streaming READ of nbytes (a multiple of 16, src
+ * 16-byte aligned) with 16-byte loads and nothing written (sink: 64 words of device memory that receive at most
+ * a checksum word). workgroups <= 0: one thread per 16 bytes (every load of the grid in flight at once, the
+ * shape of the GEMV's weight loads); otherwise that many workgroups of 256 threads, grid-stride. The time of
+ * this launch is what reading that many bytes costs on this device, the floor under a bandwidth-bound kernel
+ * that reads them. */
+int lq_calib_read(const void *src, int64_t nbytes, int workgroups, void *sink, void *stream);
 
 /* Measurement aids for the GEMM's ceiling, no counterpart in the reference.
  * lq_calib_mfma_loop: nothing but matrix instructions in the forward GEMM's shape: workgroups of 4

@@ -29,6 +29,9 @@ SIGNATURES = {
     "lq_a16w4_dequant": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp],
     "lq_a8w8_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "lq_act_quant_i8": [_vp, _vp, _vp, _i64, _vp],
+    "lq_act_quant_i8_dynamic": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp],
+    "lq_act_quant_i8_per_token": [_vp, _vp, _vp, _i64, _i64, _vp],
+    "lq_a8w8_fwd_qs": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "lq_residual_quant": [_vp, _vp, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],
     "lq_residual_dequant": [_vp, _vp, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],
     "lq_a16w4_gate_up_silu": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
@@ -38,6 +41,7 @@ SIGNATURES = {
     "lq_repack_gptq_to_native": [_vp, _vp, _i64, _i64, _vp],
     "lq_repack_native_to_gptq": [_vp, _vp, _i64, _i64, _vp],
     "lq_calib_copy": [_vp, _vp, _i64, _vp],
+    "lq_calib_read": [_vp, _i64, _i32, _vp, _vp],
     "lq_calib_mfma_loop": [_vp, _vp, _i64, _i64, _i32, _vp, _i64, _vp, _vp, _vp],
     "lq_calib_gemm_clocks": [_i32, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp, _vp],
     "lq_transpose_bf16": [_vp, _vp, _i64, _i64, _vp],

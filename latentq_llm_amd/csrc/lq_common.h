@@ -43,6 +43,14 @@ __device__ __forceinline__ unsigned short lq_f32_to_bf16_bits(float a) {
     return __builtin_bit_cast(unsigned short, r);
 }
 
+// byte SEL of `old` replaced by sat_u8(rne(v)) (v_cvt_pk_u8_f32: saturates to 0..255, NaN -> 0)
+template <int SEL>
+__device__ __forceinline__ unsigned act_cvt_pk_u8(float v, unsigned old) {
+    unsigned r;
+    asm("v_cvt_pk_u8_f32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "n"(SEL), "v"(old));
+    return r;
+}
+
 // ---- native int4 layout ----------------------------------------------------
 // A little-endian 32-bit word of the native layout holds the codes of 8
 // consecutive k: code j sits at bit 4*(j^1)  (even index = high nibble of its byte).

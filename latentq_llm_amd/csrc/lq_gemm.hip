@@ -55,7 +55,8 @@ struct GemmParams {
     const unsigned short *zeros;
     const unsigned short *bias;  // bf16 [out cols] or null
     const float *sx;             // MODE_I8: per-row scale
-    const float *sw;             // MODE_I8: per-column scale
+    const float *sw;             // MODE_I8: per-column scale (fp32, or bf16 when sw_bf16 is set)
+    int sw_bf16;
     void *c;                     // bf16 [M, C]
     int *acc_out;                // MODE_I8: optional int32 [M, C]
     int M;                       // rows of A / C
@@ -515,7 +516,8 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             for (int r = 0; r < 4; ++r) {
                 const bool in = c + r < p.C;
                 bias_v[i][q][r] = (p.bias && in) ? lq_bf16_bits_to_f32(p.bias[c + r]) : 0.0f;
-                if (MODE == MODE_I8) sw_v[i][q][r] = in ? p.sw[c + r] : 0.0f;
+                if (MODE == MODE_I8)
+                    sw_v[i][q][r] = !in ? 0.0f : p.sw_bf16 ? lq_bf16_bits_to_f32(reinterpret_cast<const unsigned short *>(p.sw)[c + r]) : p.sw[c + r];
             }
         }
 #pragma unroll
@@ -619,7 +621,7 @@ int lq_gemm_fwd_gate_up_launch(const void *x, const void *codes_g, const void *s
 
 // int8 GEMM with 256 x 256 tiles (lq_gemm_i8.hip)
 long long lq_gemm_i8_256_workgroups(int M, int N);
-int lq_gemm_i8_tile_launch(const void *x8, const void *w8, const float *sx, const float *sw, const void *bias, void *y,
+int lq_gemm_i8_tile_launch(const void *x8, const void *w8, const float *sx, const void *sw, bool sw_bf16, const void *bias, void *y,
                            int *acc_or_null, int M, int N, int K, int tile, int stages, hipStream_t st);
 
 // GEMV path (lq_gemv.hip)
@@ -966,41 +968,51 @@ extern "C" int lq_a16w4_dx_ws(const void *dy, const void *codes, const void *sca
                          workspace && workspace_bytes > 0 ? (size_t)workspace_bytes : 0, stream);
 }
 
-extern "C" int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const float *sw, const void *bias_or_null,
-                           void *y, int32_t *acc_or_null, int64_t M, int64_t N, int64_t K, void *stream) {
+static int a8w8_fwd_impl(const void *x, const void *w, const float *sx, const void *sw, bool sw_bf16, const void *bias_or_null,
+                         void *y, int32_t *acc_or_null, int64_t M, int64_t N, int64_t K, void *stream) {
     LQ_REQUIRE(x && w && sx && sw && y, "lq_a8w8_fwd: null pointer argument");
     LQ_REQUIRE(M > 0 && N > 0 && K > 0, "lq_a8w8_fwd: M, N, K must be positive");
     LQ_REQUIRE(K % 128 == 0, "lq_a8w8_fwd: K=%lld must be a multiple of 128", (long long)K);
     LQ_REQUIRE(N % 16 == 0, "lq_a8w8_fwd: N=%lld must be a multiple of 16", (long long)N);
     LQ_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "lq_a8w8_fwd: dimension too large");
-    LQ_REQUIRE(lq_aligned(x, 16) && lq_aligned(w, 16) && lq_aligned(y, 16) && lq_aligned(sx, 4) && lq_aligned(sw, 4) &&
+    LQ_REQUIRE(lq_aligned(x, 16) && lq_aligned(w, 16) && lq_aligned(y, 16) && lq_aligned(sx, 4) && lq_aligned(sw, sw_bf16 ? 2 : 4) &&
                    (!acc_or_null || lq_aligned(acc_or_null, 16)),
                "lq_a8w8_fwd: x, w, y, acc must be 16-byte aligned");
     // 256 x 256 tiles, both operands through LDS, when they occupy more than half of the compute
     // units; below that the staged kernel's smaller tiles fill the device better
     if (lq_gemm_i8_256_workgroups((int)M, (int)N) * 2 > (long long)lq_device_cu_count())
-        return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 256, 2, (hipStream_t)stream);
+        return lq_gemm_i8_tile_launch(x, w, sx, sw, sw_bf16, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 256, 2, (hipStream_t)stream);
     // the same kernel with 128 x 128 tiles (two workgroups per CU) when there are more of them than
     // compute units; measured 40.6 -> 37.0 us on 2048 x 4096 x 4096
     const long long tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
     const long long cus = lq_device_cu_count();
     if (tiles128 > cus)
-        return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 2, (hipStream_t)stream);
+        return lq_gemm_i8_tile_launch(x, w, sx, sw, sw_bf16, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 2, (hipStream_t)stream);
     // a workgroup with a CU to itself: four 32 KB stages (loads three steps ahead) instead of two whenever a
     // quarter of the CUs stay idle (15-17 against 20-22 us for the staged kernel on 128-512 tokens x 4096 x 4096,
     // 13.9 against 15.8 for two stages on 512 x 6144 x 2048), and on long reductions with every CU busy
     // (41 -> 37 us on 2048 x 2048 x 8192, 146 -> 127 on K = 32768)
     if (4 * tiles128 <= 3 * cus || K >= 6144)
-        return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 4, (hipStream_t)stream);
+        return lq_gemm_i8_tile_launch(x, w, sx, sw, sw_bf16, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 4, (hipStream_t)stream);
     // every CU busy with one workgroup: two stages for short reductions (<= 16 steps: less to set up than the
     // staged kernel's producer waves; 16.0 -> 13.1 us on 2048^3), the staged kernel in between (25.3 against
     // 27.7 us on 1024 x 4096 x 4096)
     if (K <= 2048)
-        return lq_gemm_i8_tile_launch(x, w, sx, sw, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 2, (hipStream_t)stream);
+        return lq_gemm_i8_tile_launch(x, w, sx, sw, sw_bf16, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 2, (hipStream_t)stream);
     GemmParams p = {};
-    p.a = x; p.b = w; p.sx = sx; p.sw = sw; p.bias = (const unsigned short *)bias_or_null; p.c = y;
+    p.a = x; p.b = w; p.sx = sx; p.sw = (const float *)sw; p.sw_bf16 = sw_bf16; p.bias = (const unsigned short *)bias_or_null; p.c = y;
     p.acc_out = acc_or_null;
     p.M = (int)M; p.C = (int)N; p.R = (int)K; p.Kw = (int)K;
     if (small_tiles(p)) return launch_gemm<MODE_I8, 128, 128, 2, 2>(p, (hipStream_t)stream, "lq_a8w8_fwd");
     return launch_gemm<MODE_I8, 256, 128, 2, 2>(p, (hipStream_t)stream, "lq_a8w8_fwd");
+}
+
+extern "C" int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const float *sw, const void *bias_or_null,
+                           void *y, int32_t *acc_or_null, int64_t M, int64_t N, int64_t K, void *stream) {
+    return a8w8_fwd_impl(x, w, sx, sw, false, bias_or_null, y, acc_or_null, M, N, K, stream);
+}
+
+extern "C" int lq_a8w8_fwd_qs(const void *x, const void *w, const float *sx, const void *qscales_bf16, const void *bias_or_null,
+                              void *y, int32_t *acc_or_null, int64_t M, int64_t N, int64_t K, void *stream) {
+    return a8w8_fwd_impl(x, w, sx, qscales_bf16, true, bias_or_null, y, acc_or_null, M, N, K, stream);
 }

@@ -38,7 +38,8 @@ struct I8Params {
     const unsigned char *x;  // int8 [M, K]
     const unsigned char *w;  // int8 [N, K]
     const float *sx;         // [M]
-    const float *sw;         // [N]
+    const float *sw;         // [N]: fp32, or bf16 when sw_bf16 is set
+    int sw_bf16;
     const unsigned short *bias;  // bf16 [N] or null
     int *acc_out;                // optional int32 [M, N]
     unsigned short *y;           // bf16 [M, N]
@@ -236,7 +237,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_i8_tile_kernel(I8Params p) 
             for (int e = 0; e < 4; ++e) {
                 const bool in = c + e < p.N;
                 bias_v[i][q][e] = (p.bias && in) ? lq_bf16_bits_to_f32(p.bias[c + e]) : 0.0f;
-                sw_v[i][q][e] = in ? p.sw[c + e] : 0.0f;
+                sw_v[i][q][e] = !in ? 0.0f : p.sw_bf16 ? lq_bf16_bits_to_f32(reinterpret_cast<const unsigned short *>(p.sw)[c + e]) : p.sw[c + e];
             }
         }
 #pragma unroll
@@ -280,10 +281,10 @@ long long lq_gemm_i8_256_workgroups(int M, int N) { return (long long)((M + 255)
 
 // Called by lq_a8w8_fwd (lq_gemm.hip) after argument validation: K % 128 == 0, N % 16 == 0.
 // tile = 256 or 128 (square tiles, 8 waves each); stages = 2, or 4 with the 128 tile.
-int lq_gemm_i8_tile_launch(const void *x8, const void *w8, const float *sx, const float *sw, const void *bias, void *y,
+int lq_gemm_i8_tile_launch(const void *x8, const void *w8, const float *sx, const void *sw, bool sw_bf16, const void *bias, void *y,
                            int *acc_or_null, int M, int N, int K, int tile, int stages, hipStream_t st) {
     I8Params p = {};
-    p.x = (const unsigned char *)x8; p.w = (const unsigned char *)w8; p.sx = sx; p.sw = sw;
+    p.x = (const unsigned char *)x8; p.w = (const unsigned char *)w8; p.sx = sx; p.sw = (const float *)sw; p.sw_bf16 = sw_bf16;
     p.bias = (const unsigned short *)bias; p.y = (unsigned short *)y; p.acc_out = acc_or_null;
     p.M = M; p.N = N; p.K = K;
     p.tiles_m = (M + tile - 1) / tile;

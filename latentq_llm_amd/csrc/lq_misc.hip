@@ -1,5 +1,5 @@
-// Elementwise companions of the GEMM kernels: whole-matrix dequantise, activation
-// quantizer for the int8 path, and GPTQ <-> native layout converters.
+// Elementwise companions of the GEMM kernels: whole-matrix dequantise, the int8 weight
+// re-quantiser, GPTQ <-> native layout converters, calibration kernels and the bf16 transpose.
 #include "lq_common.h"
 
 namespace {
@@ -24,75 +24,6 @@ __global__ __launch_bounds__(256) void dequant_kernel(const unsigned *__restrict
         o[i] = lq_pack_bf16(lq_bf16_lo(dp) * s, lq_bf16_hi(dp) * s);
     }
     out[w] = o;
-}
-
-// byte SEL of `old` replaced by sat_u8(rne(v)) (v_cvt_pk_u8_f32: saturates to 0..255, NaN -> 0)
-template <int SEL>
-__device__ __forceinline__ unsigned act_cvt_pk_u8(float v, unsigned old) {
-    unsigned r;
-    asm("v_cvt_pk_u8_f32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "n"(SEL), "v"(old));
-    return r;
-}
-
-// x8 = clamp(rne(bf16(bf16(x * 127) / clampv)), -128, 127); 8 elements per thread.
-// The clamp value is the maximum of a bf16 tensor in every use the reference makes of it, i.e. a bf16 number;
-// the quotient of two bf16 numbers keeps 2^-17 (relative) from every bf16 rounding tie, so bf16(a / c) is
-// bf16(a * RN(1/c)) (kFast: c has no bits below bf16's and 2^-40 <= |c| <= 2^40; decided once per launch's
-// uniform value, any other clamp value takes the division). clamp(rint(q), -128, 127) is sat_u8(rne(q + 128)) - 128:
-// q is a bf16 number, so the sum is exact wherever it matters. A NaN becomes 0 (what the tensor library's
-// float -> int8 conversion makes of it); the byte conversion would make it -128, so 8 inputs with a NaN among
-// them take the slow form.
-template <bool kFast>
-__device__ __forceinline__ u32x2_t act_quant8(const u32x4_t v, float c, float r) {
-    unsigned w[2] = {0u, 0u};
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const float f = (j & 1) ? lq_bf16_hi(v[j >> 1]) : lq_bf16_lo(v[j >> 1]);
-        const float a = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(f * 127.0f));
-        if (kFast) {
-            const float q = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(a * r)) + 128.0f;
-            switch (j & 3) {
-                case 0: w[j >> 2] = act_cvt_pk_u8<0>(q, w[j >> 2]); break;
-                case 1: w[j >> 2] = act_cvt_pk_u8<1>(q, w[j >> 2]); break;
-                case 2: w[j >> 2] = act_cvt_pk_u8<2>(q, w[j >> 2]); break;
-                default: w[j >> 2] = act_cvt_pk_u8<3>(q, w[j >> 2]); break;
-            }
-        } else {
-            const float q = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(a / c));
-            const float rr = q == q ? __builtin_amdgcn_fmed3f(rintf(q), -128.0f, 127.0f) : 0.0f;
-            w[j >> 2] |= ((unsigned)(int)rr & 0xFFu) << (8 * (j & 3));
-        }
-    }
-    if (kFast) return u32x2_t{w[0] ^ 0x80808080u, w[1] ^ 0x80808080u};
-    return u32x2_t{w[0], w[1]};
-}
-
-__global__ __launch_bounds__(256) void act_quant_kernel(const unsigned short *__restrict__ x,
-                                                        const float *__restrict__ clampv, signed char *__restrict__ x8,
-                                                        long long n) {
-    const float c = clampv[0];
-    const long long base = ((long long)blockIdx.x * 256 + threadIdx.x) * 8;
-    if (base >= n) return;
-    if (base + 8 <= n && (((uintptr_t)(x + base)) & 15) == 0 && (((uintptr_t)(x8 + base)) & 7) == 0) {
-        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(x + base);
-        const bool c_is_bf16 = (__float_as_uint(c) & 0xFFFFu) == 0u && fabsf(c) >= 0x1p-40f && fabsf(c) <= 0x1p40f;
-        // a NaN among the 8 inputs: the two forms differ on it (see above)
-        bool any_nan = false;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) any_nan |= (v[j] & 0x7FFFu) > 0x7F80u || (v[j] & 0x7FFF0000u) > 0x7F800000u;
-        u32x2_t o;
-        if (c_is_bf16 && !any_nan) o = act_quant8<true>(v, c, 1.0f / c);
-        else o = act_quant8<false>(v, c, 0.0f);
-        *reinterpret_cast<u32x2_t *>(x8 + base) = o;
-    } else {
-        for (long long i = base; i < n && i < base + 8; ++i) {
-            float f = lq_bf16_bits_to_f32(x[i]);
-            float a = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(f * 127.0f));
-            float q = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(a / c));
-            float rr = q == q ? __builtin_amdgcn_fmed3f(rintf(q), -128.0f, 127.0f) : 0.0f;
-            x8[i] = (signed char)(int)rr;
-        }
-    }
 }
 
 // Per-channel int8 re-quantiser of an 8-bit-weight layer's latent (the reference's Qfunc_8bit_res without a
@@ -182,16 +113,6 @@ extern "C" int lq_a16w4_dequant(const void *codes, const void *scales, const voi
     return lq_check_launch("lq_a16w4_dequant");
 }
 
-extern "C" int lq_act_quant_i8(const void *x, const float *clampv_dev, int8_t *x8, int64_t n, void *stream) {
-    LQ_REQUIRE(x && clampv_dev && x8 && n >= 0, "lq_act_quant_i8: bad argument");
-    if (n == 0) return LQ_OK;
-    const long long blocks = ((n + 7) / 8 + 255) / 256;
-    LQ_REQUIRE(blocks <= 0x7FFFFFFFll, "lq_act_quant_i8: n too large");
-    hipLaunchKernelGGL(act_quant_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                       (const unsigned short *)x, clampv_dev, (signed char *)x8, (long long)n);
-    return lq_check_launch("lq_act_quant_i8");
-}
-
 extern "C" int lq_w8_requant(const void *latent, const void *qscales, int8_t *codes, int64_t N, int64_t K, void *stream) {
     LQ_REQUIRE(latent && qscales && codes, "lq_w8_requant: null pointer argument");
     LQ_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && N * K / 8 / 256 < 0x7FFFFFFFll,
@@ -239,6 +160,20 @@ __global__ __launch_bounds__(256) void calib_copy_kernel(const u32x4_t *__restri
     const long long stride = (long long)gridDim.x * 256;
     for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride)
         __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+// Read-only counterpart of the copy: every thread XORs the 16-byte pieces of its grid-stride share and the
+// workgroup's last wave writes one word, so that the loads cannot be dropped and nothing else is written.
+__global__ __launch_bounds__(256) void calib_read_kernel(const u32x4_t *__restrict__ src, long long n16,
+                                                        unsigned *__restrict__ sink) {
+    const long long stride = (long long)gridDim.x * 256;
+    u32x4_t a = {0u, 0u, 0u, 0u};
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) {
+        const u32x4_t v = __builtin_nontemporal_load(src + i);
+        a[0] ^= v[0]; a[1] ^= v[1]; a[2] ^= v[2]; a[3] ^= v[3];
+    }
+    const unsigned x = a[0] ^ a[1] ^ a[2] ^ a[3];
+    if (x == 0x9E3779B9u && threadIdx.x == 255) sink[blockIdx.x & 63] = x;  // practically never taken
 }
 
 // Measurement aid: nothing but matrix instructions, in the forward GEMM's shape. A workgroup is 4 waves
@@ -311,6 +246,20 @@ extern "C" int lq_calib_copy(const void *src, void *dst, int64_t nbytes, void *s
     hipLaunchKernelGGL(calib_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                        (const u32x4_t *)src, (u32x4_t *)dst, n16);
     return lq_check_launch("lq_calib_copy");
+}
+
+extern "C" int lq_calib_read(const void *src, int64_t nbytes, int workgroups, void *sink, void *stream) {
+    LQ_REQUIRE(src && sink, "lq_calib_read: null pointer argument");
+    LQ_REQUIRE(nbytes >= 0 && nbytes % 16 == 0 && lq_aligned(src, 16) && lq_aligned(sink, 4),
+               "lq_calib_read: nbytes must be a non-negative multiple of 16, src 16-byte aligned");
+    if (nbytes == 0) return LQ_OK;
+    const long long n16 = nbytes / 16;
+    long long blocks = workgroups > 0 ? workgroups : (n16 + 255) / 256;
+    if (blocks > (n16 + 255) / 256) blocks = (n16 + 255) / 256;
+    if (blocks > 0x7FFFFFFFll) blocks = 0x7FFFFFFFll;
+    hipLaunchKernelGGL(calib_read_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const u32x4_t *)src, n16,
+                       (unsigned *)sink);
+    return lq_check_launch("lq_calib_read");
 }
 
 // ---- bf16 matrix transpose --------------------------------------------------

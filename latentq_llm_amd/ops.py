@@ -252,11 +252,14 @@ def w8_requant(latent, qscales):
 
 
 def a8w8_forward(x8, w8, sx, sw, bias=None, want_acc: bool = False):
-    """bf16 Y = ((int32 X8.W8^T) * sx[m]) * sw[n] (+ bias); optionally also the int32 accumulators."""
+    """bf16 Y = ((int32 X8.W8^T) * sx[m]) * sw[n] (+ bias); optionally also the int32 accumulators.
+    sw is fp32 [N], or the bf16 per-channel scales as the modules store them (lq_a8w8_fwd_qs)."""
     _chk(x8, torch.int8, "x8")
     _chk(w8, torch.int8, "w8")
     _chk(sx, torch.float32, "sx")
-    _chk(sw, torch.float32, "sw")
+    if sw.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError(f"sw: expected float32 or bfloat16, got {sw.dtype}")
+    _chk(sw, sw.dtype, "sw")
     M, K = x8.shape
     N, K2 = w8.shape
     if K != K2:
@@ -265,13 +268,15 @@ def a8w8_forward(x8, w8, sx, sw, bias=None, want_acc: bool = False):
         raise ValueError("sx must have M entries and sw N entries")
     if bias is not None:
         _chk(bias, torch.bfloat16, "bias")
+        if bias.numel() != N:
+            raise ValueError("bias must have N elements")
     y = torch.empty((M, N), dtype=torch.bfloat16, device=x8.device)
     acc = torch.empty((M, N), dtype=torch.int32, device=x8.device) if want_acc else None
     if M > 0:
         with torch.cuda.device(x8.device):
-            _C.call("lq_a8w8_fwd", x8.data_ptr(), w8.data_ptr(), sx.data_ptr(), sw.data_ptr(),
-                    None if bias is None else bias.data_ptr(), y.data_ptr(), None if acc is None else acc.data_ptr(),
-                    M, N, K, _stream(x8))
+            _C.call("lq_a8w8_fwd" if sw.dtype == torch.float32 else "lq_a8w8_fwd_qs", x8.data_ptr(), w8.data_ptr(),
+                    sx.data_ptr(), sw.data_ptr(), None if bias is None else bias.data_ptr(), y.data_ptr(),
+                    None if acc is None else acc.data_ptr(), M, N, K, _stream(x8))
     return (y, acc) if want_acc else y
 
 
@@ -284,6 +289,39 @@ def act_quant_i8(x, clampv):
         with torch.cuda.device(x.device):
             _C.call("lq_act_quant_i8", x.data_ptr(), clampv.data_ptr(), out.data_ptr(), x.numel(), _stream(x))
     return out
+
+
+ACT_WORK_FLOATS = 1032
+
+
+def act_quant_i8_dynamic(x, alpha_bf16: bool = False):
+    """The dynamic layers' activation quantiser with clampv = x.max() found on the device
+    (lq_act_quant_i8_dynamic): returns (x8 int8 [M,K], sx fp32 [M] filled with alpha = clampv/127, work) where
+    work[0:1] is the clamp value and work[1:2] alpha, both fp32 device tensors. x: bf16 [M, K], M*K > 0."""
+    _chk(x, torch.bfloat16, "x")
+    if x.dim() != 2 or x.numel() == 0:
+        raise ValueError("x must be a non-empty [M, K] matrix")
+    M, K = x.shape
+    x8 = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    sx = torch.empty(M, dtype=torch.float32, device=x.device)
+    work = torch.empty(ACT_WORK_FLOATS, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        _C.call("lq_act_quant_i8_dynamic", x.data_ptr(), x8.data_ptr(), sx.data_ptr(), work.data_ptr(), M, K,
+                int(bool(alpha_bf16)), _stream(x))
+    return x8, sx, work
+
+
+def act_quant_i8_per_token(x):
+    """Per-token activation quantiser (lq_act_quant_i8_per_token): (x8 int8 [M,K], sx fp32 [M] = rowmax|x| / 127)."""
+    _chk(x, torch.bfloat16, "x")
+    if x.dim() != 2 or x.numel() == 0 or x.shape[1] % 8:
+        raise ValueError("x must be a non-empty [M, K] matrix with K a multiple of 8")
+    M, K = x.shape
+    x8 = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    sx = torch.empty(M, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        _C.call("lq_act_quant_i8_per_token", x.data_ptr(), x8.data_ptr(), sx.data_ptr(), M, K, _stream(x))
+    return x8, sx
 
 
 def adam8_update(grad, state1, state2, scale1, max1, scale2, max2, beta1, beta2, eps, step_size, param=None,

@@ -229,10 +229,20 @@ def _clamp_tensor(clampv, device):
     return torch.tensor([float(clampv)], dtype=torch.float32, device=device)
 
 
+def _qs_bias(qscales, bias):
+    """The per-channel scales and the bias as the int8 GEMM reads them (bf16 [N]); no kernel runs when the module's
+    buffers already have that form."""
+    sw = qscales.detach().reshape(-1)
+    if sw.dtype not in (torch.bfloat16, torch.float32):
+        sw = sw.float()
+    b = None if bias is None else bias.detach().to(torch.bfloat16).contiguous()
+    return sw.contiguous(), b
+
+
 def _a8w8_linear(input, weight_i8, qscales, bias, clampv, alpha_in_bf16):
-    """x8 = clamp(round(x*127/clampv)); Y = ((x8 . W8^T) * alpha) * qscales + bias with
+    """Static clamp value: x8 = clamp(round(x*127/clampv)); Y = ((x8 . W8^T) * alpha) * qscales + bias with
     alpha = clampv/127: the cutlass call `linear_a8_w8_bbf16_obf16(x8, W8, bias/qs, alpha) * qs`
-    of utils/quant.py:268-271 as one int8-MFMA kernel with a fused epilogue. Returns (Y, x8)."""
+    of utils/quant.py:178-183 as one int8-MFMA kernel with a fused epilogue. Returns (Y, x8)."""
     x = _as_bf16_2d(input)
     cv = _clamp_tensor(clampv, x.device)
     x8 = ops.act_quant_i8(x, cv)
@@ -241,10 +251,34 @@ def _a8w8_linear(input, weight_i8, qscales, bias, clampv, alpha_in_bf16):
     else:
         alpha = cv / 127.
     sx = alpha.expand(x.shape[0]).contiguous()
-    sw = qscales.detach().reshape(-1).float().contiguous()
-    b = None if bias is None else bias.detach().to(torch.bfloat16).contiguous()
+    sw, b = _qs_bias(qscales, bias)
     y = ops.a8w8_forward(x8, weight_i8.contiguous(), sx, sw, b)
     return (y if input.dtype == torch.bfloat16 else y.to(input.dtype)), x8
+
+
+def _a8w8_linear_dynamic(input, weight_i8, qscales, bias, alpha_in_bf16, per_token=False):
+    """The dynamic layers' forward (utils/quant.py:259-271, 319-329), HIP kernels only: the activation quantiser
+    finds clampv = input.max() on the device and writes the int8 activations and the per-row scales, the int8 GEMM
+    reads the module's bf16 qscales directly. per_token: one scale per token row from the row's own |max| instead.
+    Returns (Y, x8, scale): scale is the quantiser's fp32 work buffer ([0] = clampv, [1] = alpha) or, per token,
+    the fp32 [M] row scales."""
+    x = _as_bf16_2d(input)
+    sw, b = _qs_bias(qscales, bias)
+    if x.shape[0] == 0:
+        y = torch.empty((0, weight_i8.shape[0]), dtype=input.dtype, device=x.device)
+        return y, torch.empty((0, x.shape[1]), dtype=torch.int8, device=x.device), torch.zeros(2, device=x.device)
+    if per_token:
+        x8, sx = ops.act_quant_i8_per_token(x)
+        scale = sx
+    else:
+        x8, sx, scale = ops.act_quant_i8_dynamic(x, alpha_in_bf16)
+    y = ops.a8w8_forward(x8, weight_i8.contiguous(), sx, sw, b)
+    return (y if input.dtype == torch.bfloat16 else y.to(input.dtype)), x8, scale
+
+
+def _per_token(qparamaw):
+    """qparamaw is (clampv, qscales) as in the reference, or (clampv, qscales, "per_token")."""
+    return len(qparamaw) > 2 and qparamaw[2] == "per_token"
 
 
 def _fake_quant_activation(input, clampv):
@@ -291,17 +325,17 @@ class QLinearFunctionA8W8_dynamic0(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight_d, qparamaw, bias):
-        _, qscales = qparamaw
-        clampv = input.max().detach()
+        qscales = qparamaw[1]
+        out, _, work = _a8w8_linear_dynamic(input, weight_d, qscales, bias, alpha_in_bf16=False)
         ctx.save_for_backward(input, weight_d.data, bias)
-        ctx.save_qparamaw = (clampv, qscales)
-        return _a8w8_linear(input, weight_d, qscales, bias, clampv, alpha_in_bf16=False)[0]
+        ctx.save_qparamaw = (work, qscales)
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):
         input, weight_d, bias = ctx.saved_tensors
-        clampv, qscales = ctx.save_qparamaw
-        input_f = _fake_quant_activation(input, clampv)
+        work, qscales = ctx.save_qparamaw
+        input_f = _fake_quant_activation(input, work[0].to(input.dtype))  # clampv = input.max(), a 0-dim tensor
         weight_f = weight_d.to(input.dtype) * qscales
         return _a8w8_backward_common(ctx, grad_output, input_f, weight_f, bias, detach_dw=True)
 
@@ -312,18 +346,20 @@ class QLinearFunctionA8W8_dynamic(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight_d, qparamaw, bias):
-        _, qscales = qparamaw
-        clampv = input.max().detach()
-        out, x8 = _a8w8_linear(input, weight_d, qscales, bias, clampv, alpha_in_bf16=True)
-        ctx.save_qparamaw = (clampv, qscales)
+        qscales = qparamaw[1]
+        per_token = _per_token(qparamaw)
+        out, x8, scale = _a8w8_linear_dynamic(input, weight_d, qscales, bias, alpha_in_bf16=True, per_token=per_token)
+        ctx.save_qparamaw = (scale, qscales, per_token)
         ctx.save_for_backward(x8, weight_d.data, bias)
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
         x8, weight_d, bias = ctx.saved_tensors
-        clampv, qscales = ctx.save_qparamaw
-        input_f = x8.to(grad_output.dtype) * (clampv / 127.)
+        scale, qscales, per_token = ctx.save_qparamaw
+        # x8 * (clampv / 127.): the quantiser left that bf16-valued alpha in scale[1]; per token: the row scales
+        s = scale.view(-1, 1) if per_token else scale[1]
+        input_f = x8.to(grad_output.dtype) * s.to(grad_output.dtype)
         weight_f = (weight_d.to(grad_output.dtype) * qscales).to(grad_output.dtype)
         return _a8w8_backward_common(ctx, grad_output, input_f, weight_f, bias, detach_dw=True)
 
@@ -346,8 +382,7 @@ class QLinearFunctionA8W8_dynamic_eval(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight_d, qparamaw, bias):
-        _, qscales = qparamaw
-        return _a8w8_linear(input, weight_d, qscales, bias, input.max().detach(), alpha_in_bf16=False)[0]
+        return _a8w8_linear_dynamic(input, weight_d, qparamaw[1], bias, alpha_in_bf16=False, per_token=_per_token(qparamaw))[0]
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -363,17 +398,17 @@ class QLinearFunctionQAT_dynamic(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight_f, qparamaw, bias):
-        _, qscales = qparamaw
-        clampv = input.max().detach()
+        qscales = qparamaw[1]
+        out, _, work = _a8w8_linear_dynamic(input, _qat_weight_i8(weight_f, qscales), qscales, bias, alpha_in_bf16=False)
         ctx.save_for_backward(input, weight_f.data, bias)
-        ctx.save_qparamaw = (clampv, qscales)
-        return _a8w8_linear(input, _qat_weight_i8(weight_f, qscales), qscales, bias, clampv, alpha_in_bf16=False)[0]
+        ctx.save_qparamaw = (work, qscales)
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):
         input, weight_f, bias = ctx.saved_tensors
-        clampv, qscales = ctx.save_qparamaw
-        input_f = _fake_quant_activation(input, clampv)
+        work, qscales = ctx.save_qparamaw
+        input_f = _fake_quant_activation(input, work[0].to(input.dtype))
         weight_q = (weight_f / qscales).round_().clamp_(-128, 127).mul_(qscales).to(input.dtype)
         return _a8w8_backward_common(ctx, grad_output, input_f, weight_q, bias, detach_dw=False)
 
@@ -383,9 +418,8 @@ class QLinearFunctionQAT_dynamic_eval(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight_f, qparamaw, bias):
-        _, qscales = qparamaw
-        return _a8w8_linear(input, _qat_weight_i8(weight_f, qscales), qscales, bias, input.max().detach(),
-                            alpha_in_bf16=False)[0]
+        qscales = qparamaw[1]
+        return _a8w8_linear_dynamic(input, _qat_weight_i8(weight_f, qscales), qscales, bias, alpha_in_bf16=False)[0]
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -484,9 +518,14 @@ class QLinearA8W8(_QLinearBase):
         self.register_buffer('clampv', torch.ones(1))
         self.register_buffer('qscales', torch.zeros(output_features, 1, dtype=torch.bfloat16))
         self.weight = QuantTensor([output_features, input_features], lbit=lbit, wbit=8, gbit=gbit)
+        # "per_tensor": the reference's activation quantiser (one clamp value = input.max()); "per_token": one
+        # scale per token row (an addition; set the attribute after construction)
+        self.act_quant = "per_tensor"
 
     def _qparam(self):
         # the dynamic Functions ignore the stored clamp (utils/quant.py:259-260): no .item() sync here
+        if self.act_quant == "per_token":
+            return (self.clampv, self.qscales.data, "per_token")
         return (self.clampv, self.qscales.data)
 
     def to(self, device: Optional[Union[int, torch.device]]):

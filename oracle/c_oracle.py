@@ -175,6 +175,25 @@ def act_quant_i8(x, clampv: float) -> np.ndarray:
     return out
 
 
+def act_quant_i8_dynamic(x, M, K, alpha_bf16: bool):
+    """-> (x8 int8[M*K], sx float32[M], clampv, alpha)"""
+    x = _c(x.reshape(-1), np.uint16)
+    x8 = np.empty(M * K, np.int8)
+    sx = np.empty(M, np.float32)
+    out2 = np.empty(2, np.float32)
+    lib().lqo_act_quant_i8_dynamic(_p(x), _p(x8), _p(sx), _p(out2), C.c_int64(M), C.c_int64(K), C.c_int(1 if alpha_bf16 else 0))
+    return x8, sx, out2[0], out2[1]
+
+
+def act_quant_i8_per_token(x, M, K):
+    """-> (x8 int8[M*K], sx float32[M])"""
+    x = _c(x.reshape(-1), np.uint16)
+    x8 = np.empty(M * K, np.int8)
+    sx = np.empty(M, np.float32)
+    lib().lqo_act_quant_i8_per_token(_p(x), _p(x8), _p(sx), C.c_int64(M), C.c_int64(K))
+    return x8, sx
+
+
 def gptq_to_native(qweight, N, K) -> np.ndarray:
     qweight = _c(qweight.reshape(-1), np.int32)
     out = np.empty(N * K // 2, np.uint8)

@@ -290,6 +290,53 @@ void lqo_act_quant_i8(const uint16_t *x, float clampv, int8_t *x8, int64_t n) {
     }
 }
 
+/* The dynamic layers' quantiser, utils/quant.py:259-266 and 319-322: clampv = input.max() (the tensor
+ * library's max: NaN as soon as one element is NaN; of -0 and +0 this restatement takes +0), then
+ * lqo_act_quant_i8 with it. out2[0] = clampv, out2[1] = alpha = clampv / 127. as the tensor library's GPU
+ * kernels form it (a product with the fp32 reciprocal of the host scalar), rounded to bf16 when alpha_bf16
+ * (the training Function divides a bf16 0-dim tensor, :271); sx[m] = alpha for every row. */
+void lqo_act_quant_i8_dynamic(const uint16_t *x, int8_t *x8, float *sx, float *out2, int64_t M, int64_t K, int alpha_bf16) {
+    const int64_t n = M * K;
+    float best = bf16_to_f32(x[0]);
+    for (int64_t i = 1; i < n && best == best; ++i) {
+        float v = bf16_to_f32(x[i]);
+        if (v != v || v > best || (v == best && !signbit(v))) best = v;
+    }
+    if (best != best) best = bf16_to_f32(0x7FC0);
+    volatile float rcp = 1.0f / 127.0f;
+    volatile float alpha = best * rcp;
+    if (alpha_bf16) alpha = bf16_round(alpha);
+    out2[0] = best;
+    out2[1] = alpha;
+    for (int64_t m = 0; m < M; ++m) sx[m] = alpha;
+    lqo_act_quant_i8(x, best, x8, n);
+}
+
+/* Per-token form of the same step (this build's addition; the reference quantises per tensor): for every row
+ * amax = max |x| (NaN if the row holds one), sx = amax / 127, x8 = clamp(rint(x * (127 / amax)), -128, 127), all
+ * in fp32 with IEEE division; NaN -> 0; an all-zero row quantises to zeros with scale 0. */
+void lqo_act_quant_i8_per_token(const uint16_t *x, int8_t *x8, float *sx, int64_t M, int64_t K) {
+    for (int64_t m = 0; m < M; ++m) {
+        const uint16_t *row = x + m * K;
+        float amax = 0.0f;
+        for (int64_t k = 0; k < K && amax == amax; ++k) {
+            float a = fabsf(bf16_to_f32(row[k]));
+            if (a != a || a > amax) amax = a;
+        }
+        volatile float inv = amax == 0.0f ? 0.0f : 127.0f / amax;
+        volatile float sc = amax / 127.0f;
+        sx[m] = sc;
+        for (int64_t k = 0; k < K; ++k) {
+            volatile float p = bf16_to_f32(row[k]) * inv;
+            float r = nearbyintf(p);
+            if (r != r) r = 0.0f;
+            if (r < -128.0f) r = -128.0f;
+            if (r > 127.0f) r = 127.0f;
+            x8[m * K + k] = (int8_t)r;
+        }
+    }
+}
+
 /* Qfunc_8bit_res without a residual codec, utils/quant.py:88-103: q = tensor / qscales (a bf16 tensor
  * operation), q.round_() (half to even), clamp_(-128, 127), .to(int8); a NaN converts to 0. */
 void lqo_w8_requant(const uint16_t *latent, const uint16_t *qscales, int8_t *codes, int64_t N, int64_t K) {

@@ -380,6 +380,82 @@ def test_act_quant_bit_exact(ops, co, shape, clamp):
     assert np.array_equal(got, want), np.nonzero(got != want)[0][:10]
 
 
+@pytest.mark.parametrize("shape", [(333, 77), (2048, 1024), (1, 8), (7, 3), (2048, 8192)])
+@pytest.mark.parametrize("alpha_bf16", [False, True])
+def test_act_quant_dynamic_bit_exact(ops, co, shape, alpha_bf16):
+    """clampv = the tensor's own maximum found on the device: int8 values, clamp value, alpha and the per-row
+    scale vector against the oracle, bit for bit."""
+    M, K = shape
+    x = randn_bf16(shape, 21 + M, 2.0)
+    got8, gsx, work = ops.act_quant_i8_dynamic(dev(x), alpha_bf16)
+    want8, wsx, cv, alpha = co.act_quant_i8_dynamic(bits(x), M, K, alpha_bf16)
+    assert np.array_equal(got8.cpu().numpy().reshape(-1), want8)
+    w = work.cpu().numpy()
+    assert w[0] == cv == float(x.max()) and w[1] == alpha
+    assert np.array_equal(gsx.cpu().numpy().view(np.uint32), wsx.view(np.uint32))
+
+
+def test_act_quant_dynamic_edge_values(ops, co):
+    """All-negative tensors (max is the element nearest zero), infinities, and a NaN (NaN clamp, all zeros)."""
+    M, K = 64, 136
+    x = -randn_bf16((M, K), 5).abs() - 0.5
+    for tweak in (None, ("inf", float("inf")), ("ninf", float("-inf")), ("nan", float("nan"))):
+        xx = x.clone()
+        if tweak:
+            xx.view(-1)[1234] = tweak[1]
+        got8, gsx, work = ops.act_quant_i8_dynamic(dev(xx), True)
+        want8, wsx, cv, alpha = co.act_quant_i8_dynamic(bits(xx), M, K, True)
+        assert np.array_equal(got8.cpu().numpy().reshape(-1), want8), tweak
+        w = work.cpu().numpy()[:2]
+        assert np.array_equal(w.view(np.uint32) & 0x7FFFFFFF, np.array([cv, alpha], np.float32).view(np.uint32) & 0x7FFFFFFF) \
+            or (np.isnan(w).all() and np.isnan(cv) and np.isnan(alpha)), tweak
+        assert np.array_equal(np.isnan(gsx.cpu().numpy()), np.isnan(wsx))
+
+
+@pytest.mark.parametrize("shape", [(5, 8), (333, 72), (2048, 2048), (2048, 8192), (64, 8200), (3, 16392)])
+def test_act_quant_per_token_bit_exact(ops, co, shape):
+    """One scale per token row: int8 values and scales against the oracle bit for bit, with an all-zero row, a NaN,
+    an infinity, a tiny row and rows of rounding ties among the inputs; row lengths on both sides of what a wave
+    keeps in registers."""
+    M, K = shape
+    x = randn_bf16(shape, 31 + M, 3.0)
+    x[0] = 0
+    if M > 4:
+        x[1, 5] = float("nan")
+        x[2, 1] = float("inf")
+        x[3] *= 1e-30
+        x[4, :] = 127.0
+        x[4, 3] = -63.5
+        x[4, K - 1] = 0.5
+    got8, gsx = ops.act_quant_i8_per_token(dev(x))
+    want8, wsx = co.act_quant_i8_per_token(bits(x), M, K)
+    assert np.array_equal(gsx.cpu().numpy().view(np.uint32) , wsx.view(np.uint32))
+    g = got8.cpu().numpy().reshape(-1)
+    assert np.array_equal(g, want8), np.nonzero(g != want8)[0][:10]
+
+
+def test_a8w8_per_token_forward_matches_float64(ops):
+    """Per-token x per-channel scaled output of the int8 GEMM (bf16 scales read in the epilogue) against the float64
+    product of the dequantised operands."""
+    M, N, K = 300, 256, 1024
+    x = randn_bf16((M, K), 3, 1.0)
+    x[7] *= 40.0  # an outlier token: per-token scales keep the others' resolution
+    g = torch.Generator().manual_seed(5)
+    w8 = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    qs = (torch.rand(N, generator=g) * 0.01 + 1e-3).to(torch.bfloat16)
+    x8, sx = ops.act_quant_i8_per_token(dev(x))
+    y = ops.a8w8_forward(x8, dev(w8), sx, dev(qs)).cpu()
+    want = (x8.cpu().double() * sx.cpu().double()[:, None]) @ (w8.double() * qs.double()[:, None]).t()
+    err = rel_l2(y, want)
+    print(f"a8w8 per-token rel_l2={err:.3e}")
+    assert err < 4e-3
+    # and against the unquantised product: the quantisation error of per-token int8 activations
+    full = x.double() @ (w8.double() * qs.double()[:, None]).t()
+    assert rel_l2(y, full) < 2e-2
+    y32 = ops.a8w8_forward(x8, dev(w8), sx, dev(qs.float())).cpu()
+    assert torch.equal(y, y32)  # bf16 scales widened in the epilogue = the fp32 copy of them
+
+
 # ------------------------------------------------------------------ repack --
 @pytest.mark.parametrize("N,K", [(16, 128), (100, 384), (4096, 1024)])
 def test_repack_round_trip(ops, co, N, K):

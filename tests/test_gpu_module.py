@@ -111,6 +111,75 @@ def test_qlinear_a8w8(Q, train):
         assert rel_l2(m.weight.grad.float().cpu(), want_dw.float()) < 1e-2
 
 
+def _a8w8_layer(Q, N, K, seed, bias=True):
+    g = torch.Generator().manual_seed(seed)
+    w8 = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    qs = ((torch.randn(N, 1, generator=g) * 0.01).abs() + 1e-3).to(torch.bfloat16)
+    m = Q.QLinearA8W8(K, N, bias=bias, lbit=16, gbit=16)
+    m.qscales.data = qs.clone()
+    if bias:
+        m.bias.data = randn_bf16((N,), seed + 1).float()
+    m.weight.set_value(w8, m.qscales)
+    m = m.bfloat16().cuda()
+    m.to("cuda")
+    return m, w8, qs
+
+
+def test_qlinear_a8w8_forward_runs_library_kernels_only(Q):
+    """The forward of an A8W8 layer (eval and training Function) dispatches no tensor-library operator that launches
+    a kernel: the activation maximum, the quantiser, the per-row scales and the scaled int8 GEMM are the library's."""
+    from torch.utils._python_dispatch import TorchDispatchMode
+
+    class Record(TorchDispatchMode):
+        def __init__(self):
+            super().__init__()
+            self.names = []
+
+        def __torch_dispatch__(self, func, types, args=(), kwargs=None):
+            self.names.append(str(func))
+            return func(*args, **(kwargs or {}))
+
+    free = ("aten.empty", "aten.view", "aten.reshape", "aten._unsafe_view", "aten.detach", "aten.alias", "aten.t.",
+            "aten._reshape_alias", "aten.select", "aten.slice", "aten.unsqueeze", "aten.expand", "aten.as_strided",
+            "aten.is_pinned", "aten.lift_fresh", "aten.new_empty")
+    for train in (False, True):
+        m, _, _ = _a8w8_layer(Q, 128, 256, 11)
+        if train:
+            m.weight.requires_grad = True
+            m.add_hook()
+        x = randn_bf16((70, 256), 3).cuda().requires_grad_(train)
+        with Record() as rec:
+            y = m(x)
+        launching = [n for n in rec.names if not n.startswith(free)]
+        assert launching == [], launching
+        assert y.shape == (70, 128)
+
+
+def test_qlinear_a8w8_per_token(Q):
+    """act_quant = "per_token": forward against the float64 product of the per-token-quantised activations and the
+    dequantised weights, backward against the dense products on the same operands."""
+    N, K, M = 128, 256, 70
+    m, w8, qs = _a8w8_layer(Q, N, K, 21)
+    m.act_quant = "per_token"
+    m.weight.requires_grad = True
+    m.add_hook()
+    x_cpu = randn_bf16((M, K), 3)
+    x_cpu[5] *= 30.0
+    x = x_cpu.cuda().requires_grad_(True)
+    y = m(x)
+    x8, sx = co.act_quant_i8_per_token(bits(x_cpu), M, K)
+    xq = torch.from_numpy(x8.reshape(M, K).astype(np.float64)) * torch.from_numpy(sx.astype(np.float64))[:, None]
+    wf = w8.double() * qs.double()
+    want = xq @ wf.t() + m.bias.detach().double().cpu()
+    assert rel_l2(y.detach().float().cpu(), want) < 5e-3
+    with torch.no_grad():
+        assert torch.equal(m.forward_eval(x), y.detach())
+    dy = randn_bf16((M, N), 4)
+    y.backward(dy.cuda())
+    assert rel_l2(x.grad.float().cpu(), dy.double() @ wf) < 1e-2
+    assert rel_l2(m.weight.grad.float().cpu(), dy.double().t() @ xq) < 1e-2
+
+
 def test_qlinear_qat_forward(Q):
     N, K, M = 64, 128, 33
     m = Q.QLinearQAT(K, N, bias=False, lbit=16, gbit=16)

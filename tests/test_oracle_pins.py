@@ -19,7 +19,9 @@ function is pinned by what the mathematics fixes:
   A8W8 bf16 epilogue     "parity unpinned": the reference's epilogue lives in the external,
                          un-vendored torch_int (FWkey/torch-int-bf16, no pinned version); only the
                          closed form bf16((acc*sx)*sw + bias) of this build is checked
-  act quant              torch's bf16 tensor arithmetic
+  act quant              torch's bf16 tensor arithmetic (given clamp value, and clampv = input.max());
+                         alpha and the per-token form against numpy float32 (IEEE) arithmetic, written
+                         with numpy's own vector operations
   GPTQ <-> native        defining bit formula, brute force
 """
 from fractions import Fraction
@@ -313,6 +315,55 @@ def test_act_quant_matches_torch_bf16_arithmetic():
     assert np.array_equal(got, want)
     want2 = tr.act_quant_i8(x, float(clampv)).numpy()  # python-float clamp (the eval path)
     assert np.array_equal(got, want2)
+
+
+def test_act_quant_dynamic_matches_torch_chain():
+    """clampv = input.max() and the int8 values against torch's bf16 tensor operations (utils/quant.py:259-266);
+    alpha against numpy float32: clampv times the fp32 reciprocal of 127, rounded to bf16 on request."""
+    for seed, shape in [(3, (5, 77)), (4, (64, 128)), (5, (1, 9))]:
+        x = randn_bf16(shape, seed, 2.5)
+        M, K = shape
+        clampv = x.max()
+        want8 = tr.act_quant_i8(x, clampv).numpy().reshape(-1)
+        for alpha_bf16 in (False, True):
+            x8, sx, cv, alpha = co.act_quant_i8_dynamic(bits(x), M, K, alpha_bf16)
+            assert cv == float(clampv) and np.array_equal(x8, want8)
+            a = np.float32(float(clampv)) * (np.float32(1.0) / np.float32(127.0))
+            if alpha_bf16:
+                a = np.float32(torch.tensor(float(a)).to(torch.bfloat16).float().item())
+            assert alpha == a and np.all(sx == a) and sx.shape == (M,)
+    # all-negative tensor: the maximum is the element closest to zero; a NaN anywhere: NaN clamp, all codes zero
+    x = -randn_bf16((4, 16), 6).abs() - 1
+    x8, sx, cv, _ = co.act_quant_i8_dynamic(bits(x), 4, 16, False)
+    assert cv == float(x.max()) and np.array_equal(x8, tr.act_quant_i8(x, x.max()).numpy().reshape(-1))
+    x.view(-1)[7] = float("nan")
+    x8, sx, cv, alpha = co.act_quant_i8_dynamic(bits(x), 4, 16, True)
+    assert np.isnan(cv) and np.isnan(alpha) and np.isnan(sx).all() and not x8.any()
+    assert torch.isnan(x.max())
+
+
+def test_act_quant_per_token_matches_numpy_float32():
+    M, K = 9, 72
+    x = randn_bf16((M, K), 11, 3.0)
+    x[2] = 0                                  # all-zero row
+    x[3, 5] = float("nan")                    # NaN in a row
+    x[4, 1] = float("inf")
+    x[5] *= 1e-30
+    x[6, :] = torch.tensor([0.5, -0.5, 1.5, -1.5, 2.5, -2.5] * 12)  # ties (amax = 2.5: x * 50.8)
+    x[7, :] = 127.0
+    x[7, 3] = -63.5                            # -63.5 * (127 / 127) = -63.5: a tie, to even -64
+    x8, sx = co.act_quant_i8_per_token(bits(x), M, K)
+    xf = x.float().numpy()
+    with np.errstate(all="ignore"):
+        amax = np.abs(xf).max(axis=1)          # numpy's max propagates NaN
+        want_sx = (amax / np.float32(127.0)).astype(np.float32)
+        inv = np.where(amax == 0, np.float32(0), np.float32(127.0) / amax).astype(np.float32)
+        r = np.rint(xf * inv[:, None])         # float32 product, half to even
+        r = np.where(np.isnan(r), 0, np.clip(r, -128, 127)).astype(np.int8)
+    assert np.array_equal(sx.view(np.uint32), want_sx.view(np.uint32))
+    assert np.array_equal(x8.reshape(M, K), r)
+    assert not x8.reshape(M, K)[2].any() and sx[2] == 0 and np.isnan(sx[3]) and not x8.reshape(M, K)[3].any()
+    assert x8.reshape(M, K)[7, 3] == -64 and x8.reshape(M, K)[7, 0] == 127
 
 
 # ---------------------------------------------------------------------- layout --
