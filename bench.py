@@ -62,10 +62,13 @@ def event_time(fn, iters, warm=30, warm_seconds=0.08):
     return e0.elapsed_time(e1) * 1e-3 / iters
 
 
-def graph_time(calls, replays=20):
+def graph_time(calls, replays=20, warm_seconds=0.08):
     """Average seconds per kernel for launch-latency-scale kernels: the calls (one per rotating
     buffer set) are captured into one HIP graph so that launches are back to back, and the
-    graph is replayed between two HIP events on the replay stream."""
+    graph is replayed between two HIP events on the replay stream. The graph is first replayed for
+    at least `warm_seconds` (the same settling time event_time gives its kernels: the inputs of these
+    blocks are built on the host for seconds, with the device idle and its clock down), and the
+    timed replays follow without a pause."""
     for c in calls:
         c()
     torch.cuda.synchronize()
@@ -73,9 +76,14 @@ def graph_time(calls, replays=20):
     with torch.cuda.graph(g):
         for c in calls:
             c()
-    g.replay()
-    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < warm_seconds:
+        for _ in range(10):
+            g.replay()
+        torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(3):
+        g.replay()
     e0.record()
     for _ in range(replays):
         g.replay()
@@ -209,8 +217,13 @@ def bench_latent(device):
 
 
 def bench_gemv(device):
-    from latentq_llm_amd import ops
+    """configs[4]: the decode GEMV over the three 7B matrix shapes at 1, 4 and 16 tokens, as HIP graphs over
+    rotating weight sets larger than the last-level cache. Beside every point: a read-only launch over buffers
+    of the same rotation holding the same number of bytes (lq_calib_read, one 16-byte load per thread: the
+    GEMV's own access shape), i.e. what it costs on this device just to read what the kernel must read."""
+    from latentq_llm_amd import _C, ops
     out = []
+    sink = torch.zeros(64, dtype=torch.int32, device=device)
     for (N, K) in [(4096, 4096), (11008, 4096), (4096, 11008)]:
         nb = int(300e6 // (N * K // 2)) + 1
         ws = [synth_w4(N, K, 20 + i, device) for i in range(nb)]
@@ -220,8 +233,15 @@ def bench_gemv(device):
             calls = [(lambda w=w, y=y: ops.a16w4_forward(x, *w, (N, K), out=y)) for w, y in zip(ws, ys)]
             sec = graph_time(calls)
             nbytes = N * K // 2 + 4 * N * K // GROUP + 2 * M * K + 2 * M * N
+            rbytes = nbytes // 16 * 16
+            bufs = [torch.empty(rbytes, dtype=torch.uint8, device=device).random_(0, 256) for _ in range(nb)]
+            reads = [(lambda b=b: _C.call("lq_calib_read", b.data_ptr(), rbytes, 0, sink.data_ptr(),
+                                          torch.cuda.current_stream().cuda_stream)) for b in bufs]
+            sec_read = graph_time(reads)
+            del bufs
             out.append({"N": N, "K": K, "M": M, "us": sec * 1e6, "GB/s": nbytes / sec / 1e9,
-                        "frac_hbm": nbytes / sec / PEAK_HBM})
+                        "frac_hbm": nbytes / sec / PEAK_HBM, "read_same_bytes_us": sec_read * 1e6,
+                        "frac_of_read": sec_read / sec})
         del ws
     return out
 
@@ -622,6 +642,23 @@ def cpu_baseline():
             nb = N * K // 2 + 4 * N * K // GROUP + 2 * M * K + 2 * M * N
             c4.append({"N": N, "K": K, "M": M, "ms": sec * 1e3, "GB/s": nb / sec / 1e9})
     out["c4"] = c4
+    out["c4_note"] = "1 warm-up + 1-3 timed runs per point within 0.6 s each (a stated baseline, not a precise timing)"
+    # configs[3]: the int8 GEMM with its scale epilogue (C oracle, OpenMP over the same cores; the reference's own
+    # kernel for it is CUDA-only), once per shape on the first 256 of the 2048 tokens
+    c3 = []
+    rng = np.random.default_rng(3)
+    Ms = 256
+    for (N, K) in [(2048, 2048), (8192, 2048), (2048, 8192)]:
+        x8 = rng.integers(-127, 128, (Ms, K), dtype=np.int8)
+        w8 = rng.integers(-127, 128, (N, K), dtype=np.int8)
+        sxv = np.abs(rng.standard_normal(Ms).astype(np.float32)) * 0.05
+        swv = np.abs(rng.standard_normal(N).astype(np.float32)) * 0.01
+        t0 = time.time()
+        co.a8w8(x8, w8, sxv, swv, None, Ms, N, K)
+        sec = time.time() - t0
+        c3.append({"M_sample": Ms, "N": N, "K": K, "ms": sec * 1e3, "TOP/s": 2.0 * Ms * N * K / sec / 1e12})
+    out["c3"] = c3
+    out["c3_note"] = f"configs[3] shapes on a sample of {Ms} of the {TOKENS} tokens, one run each, int32 accumulate + fp32 scale epilogue"
     return out
 
 
