@@ -5,8 +5,9 @@
 
 One "step" is one pass of the A16W4 Llama-2-7B MLP block at 4 x 512 = 2048 bf16 tokens:
 forward  down(silu(gate(x)) * up(x))  and the dX backward through all three projections
-(six dequant-GEMMs, 1108.1 GFLOP), with synthetic seeded weights and activations already
-resident in HBM. The headline value is GEMM TFLOP/s of that step. The same JSON line also
+(six dequant-GEMM products, 1108.1 GFLOP, in the five launches the fused training block makes:
+the bf16 glue of autograd sits in the GEMM epilogues), with synthetic seeded weights and
+activations already resident in HBM. The headline value is GEMM TFLOP/s of that step. The same JSON line also
 carries the kernel roofline of the dominant kernel (measured with HIP events on the launch
 stream), HBM GB/s of the requantizer and of the decode GEMV sweep, the A8W8 GEMM rate, and
 the CPU baseline (the torch restatement of the reference's dequant path on the host cores).
@@ -106,8 +107,20 @@ class MLPBlock:
         self.dy = torch.randn(TOKENS, HID, generator=g).to(torch.bfloat16).to(device)
 
     def step(self):
+        """The block as latentq_llm_amd.fused_mlp.QuantLlamaMLP runs it in training: five launches, the bf16 glue
+        of autograd (silu, three products, silu backward, the sum of the two input gradients) in the GEMM epilogues."""
         o = self.ops
-        # bf16 glue exactly as autograd runs it for  down(silu(gate(x)) * up(x))
+        h, g, u = o.a16w4_gate_up_silu(self.x, self.gate, self.up, (FFN, HID), save=True)
+        y = o.a16w4_forward(h, *self.down, (HID, FFN))
+        dg, du = o.a16w4_dx_silu_bwd(self.dy, *self.down, (HID, FFN), g, u)
+        dx = o.a16w4_dx(dg, *self.gate, (FFN, HID))
+        o.a16w4_dx(du, *self.up, (FFN, HID), out=dx, accumulate=True)
+        return y, dx
+
+    def step_unfused(self):
+        """The same block layer by layer, with the bf16 glue exactly as autograd runs it (six GEMM launches and
+        six tensor-library kernels)."""
+        o = self.ops
         g = o.a16w4_forward(self.x, *self.gate, (FFN, HID))
         u = o.a16w4_forward(self.x, *self.up, (FFN, HID))
         act = torch.nn.functional.silu(g)
@@ -489,10 +502,19 @@ def profile_target(device, which, launches=10):
             o.a16w4_dx(h, *blk.gate, (FFN, HID))
         for _ in range(launches):
             o.a16w4_dx(blk.dy, *blk.down, (HID, FFN))
-        # the inference-side fused product silu(gate(x)) * up(x), and the 128 x 128-tile instance of the forward kernel
+        # the fused product silu(gate(x)) * up(x) (inference form, then the training form that also stores the two
+        # products), the down dX with the silu backward epilogue, the accumulating dX, and the 128 x 128-tile
+        # instance of the forward kernel
         hbuf = torch.empty((TOKENS, FFN), dtype=torch.bfloat16, device=device)
         for _ in range(launches):
             o.a16w4_gate_up_silu(blk.x, blk.gate, blk.up, (FFN, HID), out=hbuf)
+        for _ in range(launches):
+            _, g_, u_ = o.a16w4_gate_up_silu(blk.x, blk.gate, blk.up, (FFN, HID), out=hbuf, save=True)
+        for _ in range(launches):
+            dg_, du_ = o.a16w4_dx_silu_bwd(blk.dy, *blk.down, (HID, FFN), g_, u_)
+        dxb = torch.zeros((TOKENS, HID), dtype=torch.bfloat16, device=device)
+        for _ in range(launches):
+            o.a16w4_dx(du_, *blk.up, (FFN, HID), out=dxb, accumulate=True)
         x1536 = torch.randn(1536, HID, device=device).to(torch.bfloat16)
         for _ in range(launches):
             o.a16w4_forward(x1536, *blk.gate, (FFN, HID))
@@ -717,26 +739,47 @@ def main():
     dt = (time.perf_counter() - t0) / args.steps
     value = MLP_FLOP / dt / 1e12
 
-    # Dominant kernel: the dequant-GEMM. Per-launch duration from HIP events on the launch stream.
+    # Dominant kernel: the dequant-GEMM. Per-launch duration of the step's five launches from HIP events on the
+    # launch stream (the gate / up launch holds two products: 2 x 184.68 GFLOP).
     o = blk.ops
-    h = torch.randn(TOKENS, FFN, device=dev).to(torch.bfloat16)
+    one = 2 * TOKENS * HID * FFN
+    h, g, u = o.a16w4_gate_up_silu(blk.x, blk.gate, blk.up, (FFN, HID), save=True)
+    dg, du = o.a16w4_dx_silu_bwd(blk.dy, *blk.down, (HID, FFN), g, u)
+    dxb = torch.empty((TOKENS, HID), dtype=torch.bfloat16, device=dev)
     kern = {}
     for name, fn, fl in [
-        ("fwd_gate_up", lambda: o.a16w4_forward(blk.x, *blk.gate, (FFN, HID)), 2 * TOKENS * HID * FFN),
-        ("fwd_down", lambda: o.a16w4_forward(h, *blk.down, (HID, FFN)), 2 * TOKENS * HID * FFN),
-        ("dx_gate_up", lambda: o.a16w4_dx(h, *blk.gate, (FFN, HID)), 2 * TOKENS * HID * FFN),
-        ("dx_down", lambda: o.a16w4_dx(blk.dy, *blk.down, (HID, FFN)), 2 * TOKENS * HID * FFN),
+        ("fwd_gate_up_silu", lambda: o.a16w4_gate_up_silu(blk.x, blk.gate, blk.up, (FFN, HID), save=True), 2 * one),
+        ("fwd_down", lambda: o.a16w4_forward(h, *blk.down, (HID, FFN)), one),
+        ("dx_down_silu_bwd", lambda: o.a16w4_dx_silu_bwd(blk.dy, *blk.down, (HID, FFN), g, u), one),
+        ("dx_gate", lambda: o.a16w4_dx(dg, *blk.gate, (FFN, HID), out=dxb), one),
+        ("dx_up_acc", lambda: o.a16w4_dx(du, *blk.up, (FFN, HID), out=dxb, accumulate=True), one),
+        # the same products as separate launches with a plain store (what the layers run on their own)
+        ("fwd_gate_or_up", lambda: o.a16w4_forward(blk.x, *blk.gate, (FFN, HID)), one),
+        ("dx_down", lambda: o.a16w4_dx(blk.dy, *blk.down, (HID, FFN)), one),
     ]:
         sec = event_time(fn, 50)
-        kern[name] = {"us": sec * 1e6, "TFLOP/s": fl / sec / 1e12, "frac_mfma_bf16": fl / sec / PEAK_BF16}
-    # weighted by launches per step: 2 fwd gate/up, 1 fwd down, 2 dx gate/up, 1 dx down
-    tot = 2 * kern["fwd_gate_up"]["us"] + kern["fwd_down"]["us"] + 2 * kern["dx_gate_up"]["us"] + kern["dx_down"]["us"]
+        kern[name] = {"us": sec * 1e6, "GFLOP": fl / 1e9, "TFLOP/s": fl / sec / 1e12, "frac_mfma_bf16": fl / sec / PEAK_BF16}
+    step_launches = ("fwd_gate_up_silu", "fwd_down", "dx_down_silu_bwd", "dx_gate", "dx_up_acc")
+    tot = sum(kern[k]["us"] for k in step_launches)
+    # per 184.68 GFLOP product: six of them in the five launches
     avg_us = tot / 6
-    achieved = 2 * TOKENS * HID * FFN / (avg_us * 1e-6) / 1e12
-    roofline = {"bound": "mfma", "kernel": "A16W4 dequant-GEMM: gemm_fwd_direct_kernel<2, false> (forward), gemm_kernel<1> (dX)",
+    achieved = one / (avg_us * 1e-6) / 1e12
+    roofline = {"bound": "mfma", "kernel": "A16W4 dequant-GEMM: gemm_fwd_direct_kernel<2, *> (forward), gemm_kernel<1> (dX)",
                 "achieved": achieved, "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": achieved * 1e12 / PEAK_BF16,
-                "avg_launch_us": avg_us, "flop_per_launch": 2 * TOKENS * HID * FFN, "traffic": gemm_traffic_bytes(),
+                "avg_launch_us": avg_us, "flop_per_launch": one,
+                "note": "per product of 2*2048*4096*11008 flop: total time of the step's five GEMM launches / 6 (the gate/up launch holds two)",
+                "traffic": gemm_traffic_bytes(),
                 "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated on a copy)"}
+    # the step with the glue as tensor-library kernels, for comparison
+    for _ in range(20):
+        blk.step_unfused()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(50):
+        blk.step_unfused()
+    torch.cuda.synchronize()
+    unfused_ms = (time.perf_counter() - t0) / 50 * 1e3
+    del g, u, dg, du, dxb
 
     line = {
         "metric": "A16W4 GEMM TFLOP/s (7B MLP, 2048 tok)", "value": value, "unit": "TFLOP/s",
@@ -747,6 +790,8 @@ def main():
                    "tokens": TOKENS, "flop_per_step": MLP_FLOP},
         "roofline": roofline,
         "gemm_kernels": kern,
+        "step_layer_by_layer": {"ms_per_step": unfused_ms, "TFLOP/s": MLP_FLOP / (unfused_ms * 1e-3) / 1e12,
+                                "what": "six GEMM launches + six bf16 tensor-library kernels (silu, three products, silu backward, add)"},
     }
     if not args.only_mlp:
         ceil = bench_ceiling(dev, blk, h)

@@ -150,6 +150,31 @@ int lq_a16w4_gate_up_silu(const void *x, const void *codes_gate, const void *sca
                           const void *codes_up, const void *scales_up, const void *zeros_up, void *h, int64_t M,
                           int64_t N, int64_t K, int group, void *stream);
 
+/* The gated MLP block in training, three entry points that take the tensor-library glue between the six
+ * products of `down(silu(gate(x)) * up(x))` and its backward into the GEMM epilogues. In the reference that
+ * block is transformers' LlamaMLP with its three nn.Linear replaced by QLinearA16W4 (main0.py:300-343), i.e.
+ * QLinearFunctionW4.forward / backward (utils/quant.py:112-146) around bf16 silu, products and an addition
+ * run by autograd; there is no counterpart function.
+ *   lq_a16w4_gate_up_silu_save: lq_a16w4_gate_up_silu that also stores the two products it forms,
+ *     g = X . deq(Wgate)^T and u = X . deq(Wup)^T (bf16 [M,N] each, rounded from the same fp32 sums h is formed
+ *     from), which the backward pass needs. Up to 16 tokens: one GEMV pass per product plus the fused pass.
+ *   lq_a16w4_dx_silu_bwd: the backward of the down projection with the backward of h = silu(g) * u as its
+ *     epilogue. P = dY . deq(Wdown) [M,K] is rounded to bf16 (it is the dh autograd would hand on) and
+ *       dg = bf16(P * u * s * (1 + g * (1 - s))),  du = bf16(P * g * s),  s = 1 / (1 + exp(-g))
+ *     are stored instead of it (fp32 arithmetic on the bf16 values of P, g, u; one rounding each, where the
+ *     tensor operations round silu(g) and P * u to bf16 in between). g, u, dg_out, du_out: bf16 [M,K].
+ *   lq_a16w4_dx_acc: dx_inout = bf16(dx_inout + bf16(dY . deq(W))): the second of the two products that
+ *     both flow into the block's input gradient; the same bits as lq_a16w4_dx followed by a bf16 addition.
+ * Shapes and alignment as lq_a16w4_dx / lq_a16w4_gate_up_silu; all outputs 16-byte aligned. */
+int lq_a16w4_gate_up_silu_save(const void *x, const void *codes_gate, const void *scales_gate, const void *zeros_gate,
+                               const void *codes_up, const void *scales_up, const void *zeros_up, void *h, void *g_out,
+                               void *u_out, int64_t M, int64_t N, int64_t K, int group, void *stream);
+int lq_a16w4_dx_silu_bwd(const void *dy, const void *codes, const void *scales, const void *zeros, const void *g,
+                         const void *u, void *dg_out, void *du_out, int64_t M, int64_t N, int64_t K, int group,
+                         void *stream);
+int lq_a16w4_dx_acc(const void *dy, const void *codes, const void *scales, const void *zeros, void *dx_inout,
+                    int64_t M, int64_t N, int64_t K, int group, void *stream);
+
 /* Which kernel lq_a16w4_fwd(_ws) (backward = 0) or lq_a16w4_dx(_ws) (backward = 1) would run for a
  * shape and a workspace size, and how it would cut the reduction; launches nothing. *kernel is
  * one of LQ_PLAN_*; *splits > 1 means a split reduction of *steps_per_split 64-deep steps per slice

@@ -71,7 +71,18 @@ struct GemmParams {
     // measurement aid (null in normal use): workgroup w writes the shader-cycle counter and the
     // 100 MHz real-time counter at its start and end to clk[4 w .. 4 w + 3]
     unsigned long long *clk;
+    // MODE_W4_DX epilogue forms (on the bf16-rounded product P, 8 columns per lane):
+    //   EP_STORE   c = P
+    //   EP_ADD     c = bf16(c + P)                                   (the second of two products that share their output)
+    //   EP_SILU_BW c  = bf16(P * u * s * (1 + g * (1 - s))),  s = 1 / (1 + exp(-g))      (gradient of the gate product)
+    //              c2 = bf16(P * g * s)                                                 (gradient of the up product)
+    //              for P = the gradient of h = silu(g) * u; ep_g, ep_u: bf16 [M, C]
+    int ep_mode;
+    const unsigned short *ep_g, *ep_u;
+    unsigned short *c2;
 };
+
+enum { EP_STORE = 0, EP_ADD = 1, EP_SILU_BW = 2 };
 
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void gbl_void;
@@ -553,7 +564,40 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             const int row = it * RPI + ep_row;
             const u32x4_t o = *reinterpret_cast<const u32x4_t *>(ep + row * EP + ep_chunk * 16);
             const int mm = m0 + wm * TM + j * 32 + row;
-            if (mm < p.M && c_lane < p.C) *reinterpret_cast<u32x4_t *>(out + (long long)mm * p.C + c_lane) = o;
+            if (mm < p.M && c_lane < p.C) {
+                const long long off = (long long)mm * p.C + c_lane;
+                if (MODE == MODE_W4_DX && p.ep_mode == EP_ADD) {
+                    const u32x4_t old = *reinterpret_cast<const u32x4_t *>(out + off);
+                    u32x4_t sum;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        sum[e] = lq_pack_bf16(lq_bf16_lo(old[e]) + lq_bf16_lo(o[e]), lq_bf16_hi(old[e]) + lq_bf16_hi(o[e]));
+                    *reinterpret_cast<u32x4_t *>(out + off) = sum;
+                } else if (MODE == MODE_W4_DX && p.ep_mode == EP_SILU_BW) {
+                    const u32x4_t g8 = *reinterpret_cast<const u32x4_t *>(p.ep_g + off);
+                    const u32x4_t u8 = *reinterpret_cast<const u32x4_t *>(p.ep_u + off);
+                    u32x4_t dg, du;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float rg[2], ru[2];
+#pragma unroll
+                        for (int hh = 0; hh < 2; ++hh) {
+                            const float d = hh ? lq_bf16_hi(o[e]) : lq_bf16_lo(o[e]);
+                            const float g = hh ? lq_bf16_hi(g8[e]) : lq_bf16_lo(g8[e]);
+                            const float u = hh ? lq_bf16_hi(u8[e]) : lq_bf16_lo(u8[e]);
+                            const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-g));
+                            rg[hh] = d * u * (sg * (1.0f + g * (1.0f - sg)));
+                            ru[hh] = d * (g * sg);
+                        }
+                        dg[e] = lq_pack_bf16(rg[0], rg[1]);
+                        du[e] = lq_pack_bf16(ru[0], ru[1]);
+                    }
+                    *reinterpret_cast<u32x4_t *>(out + off) = dg;
+                    *reinterpret_cast<u32x4_t *>(p.c2 + off) = du;
+                } else {
+                    *reinterpret_cast<u32x4_t *>(out + off) = o;
+                }
+            }
         }
     }
     if (p.clk && threadIdx.x == 0) {
@@ -616,8 +660,8 @@ long long lq_gemm_fwd_direct128_workgroups(int M, int N);
 int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scales, const void *zeros, const void *bias,
                               void *y, int M, int N, int K, hipStream_t st, unsigned long long *clk, bool narrow);
 int lq_gemm_fwd_gate_up_launch(const void *x, const void *codes_g, const void *scales_g, const void *zeros_g,
-                               const void *codes_u, const void *scales_u, const void *zeros_u, void *h, int M, int N, int K,
-                               hipStream_t st);
+                               const void *codes_u, const void *scales_u, const void *zeros_u, void *h, void *g_out, void *u_out,
+                               int M, int N, int K, hipStream_t st);
 
 // int8 GEMM with 256 x 256 tiles (lq_gemm_i8.hip)
 long long lq_gemm_i8_256_workgroups(int M, int N);
@@ -817,21 +861,45 @@ static int a16w4_fwd_impl(const char *who, const void *x, const void *codes, con
     return launch_split_reduce(p, plan.splits, (hipStream_t)stream, who);
 }
 
-extern "C" int lq_a16w4_gate_up_silu(const void *x, const void *codes_gate, const void *scales_gate, const void *zeros_gate,
-                                     const void *codes_up, const void *scales_up, const void *zeros_up, void *h, int64_t M,
-                                     int64_t N, int64_t K, int group, void *stream) {
-    const char *who = "lq_a16w4_gate_up_silu";
+static int gate_up_impl(const char *who, const void *x, const void *codes_gate, const void *scales_gate, const void *zeros_gate,
+                        const void *codes_up, const void *scales_up, const void *zeros_up, void *h, void *g_out, void *u_out,
+                        int64_t M, int64_t N, int64_t K, int group, void *stream) {
     int rc = check_w4_common(who, x, codes_gate, scales_gate, zeros_gate, h, M, N, K, group);
     if (rc) return rc;
     rc = check_w4_common(who, x, codes_up, scales_up, zeros_up, h, M, N, K, group);
     if (rc) return rc;
     LQ_REQUIRE(N % 16 == 0, "%s: N=%lld must be a multiple of 16", who, (long long)N);
-    if (M <= 16)
+    LQ_REQUIRE((g_out == nullptr) == (u_out == nullptr) && lq_aligned(g_out, 16) && lq_aligned(u_out, 16),
+               "%s: g_out and u_out are given together, 16-byte aligned", who);
+    if (M <= 16) {
+        if (g_out) {
+            // the two products on their own (one GEMV pass each), then the fused pass for h
+            rc = lq_gemv_a16w4_launch(x, codes_gate, scales_gate, zeros_gate, nullptr, g_out, (int)M, (int)N, (int)K, (hipStream_t)stream);
+            if (rc) return rc;
+            rc = lq_gemv_a16w4_launch(x, codes_up, scales_up, zeros_up, nullptr, u_out, (int)M, (int)N, (int)K, (hipStream_t)stream);
+            if (rc) return rc;
+        }
         return lq_gemv_a16w4_gate_up_launch(x, codes_gate, scales_gate, zeros_gate, codes_up, scales_up, zeros_up, h, (int)M, (int)N,
                                             (int)K, (hipStream_t)stream);
+    }
     LQ_REQUIRE(K % 256 == 0, "%s: K=%lld must be a multiple of 256 for more than 16 tokens", who, (long long)K);
-    return lq_gemm_fwd_gate_up_launch(x, codes_gate, scales_gate, zeros_gate, codes_up, scales_up, zeros_up, h, (int)M, (int)N,
-                                      (int)K, (hipStream_t)stream);
+    return lq_gemm_fwd_gate_up_launch(x, codes_gate, scales_gate, zeros_gate, codes_up, scales_up, zeros_up, h, g_out, u_out, (int)M,
+                                      (int)N, (int)K, (hipStream_t)stream);
+}
+
+extern "C" int lq_a16w4_gate_up_silu(const void *x, const void *codes_gate, const void *scales_gate, const void *zeros_gate,
+                                     const void *codes_up, const void *scales_up, const void *zeros_up, void *h, int64_t M,
+                                     int64_t N, int64_t K, int group, void *stream) {
+    return gate_up_impl("lq_a16w4_gate_up_silu", x, codes_gate, scales_gate, zeros_gate, codes_up, scales_up, zeros_up, h, nullptr,
+                        nullptr, M, N, K, group, stream);
+}
+
+extern "C" int lq_a16w4_gate_up_silu_save(const void *x, const void *codes_gate, const void *scales_gate, const void *zeros_gate,
+                                          const void *codes_up, const void *scales_up, const void *zeros_up, void *h, void *g_out,
+                                          void *u_out, int64_t M, int64_t N, int64_t K, int group, void *stream) {
+    LQ_REQUIRE(g_out && u_out, "lq_a16w4_gate_up_silu_save: null pointer argument");
+    return gate_up_impl("lq_a16w4_gate_up_silu_save", x, codes_gate, scales_gate, zeros_gate, codes_up, scales_up, zeros_up, h, g_out,
+                        u_out, M, N, K, group, stream);
 }
 
 extern "C" int lq_a16w4_fwd(const void *x, const void *codes, const void *scales, const void *zeros,
@@ -847,15 +915,25 @@ extern "C" int lq_a16w4_fwd_ws(const void *x, const void *codes, const void *sca
                           workspace && workspace_bytes > 0 ? (size_t)workspace_bytes : 0, stream);
 }
 
+struct DxEpilogue {
+    int mode = EP_STORE;
+    const void *g = nullptr, *u = nullptr;
+    void *c2 = nullptr;
+};
+
 static int a16w4_dx_impl(const char *who, const void *dy, const void *codes, const void *scales, const void *zeros,
                          void *dx, int64_t M, int64_t N, int64_t K, int group, void *workspace, size_t ws_bytes,
-                         void *stream, unsigned long long *clk = nullptr) {
+                         void *stream, unsigned long long *clk = nullptr, const DxEpilogue &ep = DxEpilogue()) {
     int rc = check_w4_common(who, dy, codes, scales, zeros, dx, M, N, K, group);
     if (rc) return rc;
     LQ_REQUIRE(N % 64 == 0, "%s: N=%lld must be a multiple of 64", who, (long long)N);
     LQ_REQUIRE(!workspace || lq_aligned(workspace, 16), "%s: the workspace must be 16-byte aligned", who);
     GemmParams p = {};
     p.clk = clk;
+    p.ep_mode = ep.mode;
+    p.ep_g = (const unsigned short *)ep.g; p.ep_u = (const unsigned short *)ep.u; p.c2 = (unsigned short *)ep.c2;
+    // the epilogue forms other than a plain store live in the GEMM kernel only: no split reduction with them
+    if (ep.mode != EP_STORE) workspace = nullptr;
     p.a = dy; p.b = codes; p.scales = (const unsigned short *)scales; p.zeros = (const unsigned short *)zeros;
     p.c = dx;
     p.M = (int)M; p.C = (int)K; p.R = (int)N; p.Kw = (int)K;
@@ -959,6 +1037,24 @@ extern "C" int lq_a16w4_plan(int backward, int64_t M, int64_t N, int64_t K, int6
 extern "C" int lq_a16w4_dx(const void *dy, const void *codes, const void *scales, const void *zeros, void *dx,
                            int64_t M, int64_t N, int64_t K, int group, void *stream) {
     return a16w4_dx_impl("lq_a16w4_dx", dy, codes, scales, zeros, dx, M, N, K, group, nullptr, 0, stream);
+}
+
+extern "C" int lq_a16w4_dx_acc(const void *dy, const void *codes, const void *scales, const void *zeros, void *dx_inout,
+                               int64_t M, int64_t N, int64_t K, int group, void *stream) {
+    DxEpilogue ep;
+    ep.mode = EP_ADD;
+    return a16w4_dx_impl("lq_a16w4_dx_acc", dy, codes, scales, zeros, dx_inout, M, N, K, group, nullptr, 0, stream, nullptr, ep);
+}
+
+extern "C" int lq_a16w4_dx_silu_bwd(const void *dh_dy, const void *codes, const void *scales, const void *zeros, const void *g,
+                                    const void *u, void *dg_out, void *du_out, int64_t M, int64_t N, int64_t K, int group,
+                                    void *stream) {
+    LQ_REQUIRE(g && u && du_out && lq_aligned(g, 16) && lq_aligned(u, 16) && lq_aligned(du_out, 16),
+               "lq_a16w4_dx_silu_bwd: g, u and du_out must be given, 16-byte aligned");
+    DxEpilogue ep;
+    ep.mode = EP_SILU_BW;
+    ep.g = g; ep.u = u; ep.c2 = du_out;
+    return a16w4_dx_impl("lq_a16w4_dx_silu_bwd", dh_dy, codes, scales, zeros, dg_out, M, N, K, group, nullptr, 0, stream, nullptr, ep);
 }
 
 extern "C" int lq_a16w4_dx_ws(const void *dy, const void *codes, const void *scales, const void *zeros, void *dx,

@@ -64,6 +64,8 @@ struct FwdParams {
     const unsigned short *scales2;
     const unsigned short *zeros2;
     unsigned short *y;           // bf16 [M, N]
+    // gate / up mode, training form: the two products themselves (bf16 [M, N] each) are stored as well when given
+    unsigned short *g_out, *u_out;
     int M, N, K;
     int tiles_m, tiles_n;
     // measurement aid (null in normal use): workgroup w writes the shader-cycle counter and the
@@ -392,30 +394,36 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
                 const int c = c0 + wave * WN + 8 * q + 4 * h + e;
                 bias_n[q][e] = (!GU && p.bias && c < p.N) ? lq_bf16_bits_to_f32(p.bias[c]) : 0.0f;
             }
+        // which = 0: the output (H, or Y with one matrix); 1, 2 (gate / up mode with g_out): the two products
+        const int n_out = (GU && p.g_out) ? 3 : 1;
+        for (int which = 0; which < n_out; ++which) {
+            unsigned short *dst = which == 0 ? p.y : which == 1 ? p.g_out : p.u_out;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < 4; ++j) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                float v[4];
+                for (int q = 0; q < 4; ++q) {
+                    float v[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float g = acc[0][j][4 * q + e];
-                    if constexpr (GU) {
-                        v[e] = g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * acc[NT - 1][j][4 * q + e];
-                    } else {
-                        v[e] = g;
-                        if (p.bias) v[e] += bias_n[q][e];
+                    for (int e = 0; e < 4; ++e) {
+                        const float g = acc[0][j][4 * q + e];
+                        if constexpr (GU) {
+                            const float u = acc[NT - 1][j][4 * q + e];
+                            v[e] = which == 0 ? g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u : which == 1 ? g : u;
+                        } else {
+                            v[e] = g;
+                            if (p.bias) v[e] += bias_n[q][e];
+                        }
                     }
+                    u32x2_t o = {lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3])};
+                    *reinterpret_cast<u32x2_t *>(ep + r * EP + (8 * q + 4 * h) * 2) = o;
                 }
-                u32x2_t o = {lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3])};
-                *reinterpret_cast<u32x2_t *>(ep + r * EP + (8 * q + 4 * h) * 2) = o;
-            }
 #pragma unroll
-            for (int it = 0; it < 2; ++it) {
-                const int row = it * 16 + ep_row;
-                const u32x4_t o = *reinterpret_cast<const u32x4_t *>(ep + row * EP + ep_chunk * 16);
-                const int mm = m0 + j * 32 + row;
-                if (mm < p.M && c_lane < p.N) *reinterpret_cast<u32x4_t *>(p.y + (long long)mm * p.N + c_lane) = o;
+                for (int it = 0; it < 2; ++it) {
+                    const int row = it * 16 + ep_row;
+                    const u32x4_t o = *reinterpret_cast<const u32x4_t *>(ep + row * EP + ep_chunk * 16);
+                    const int mm = m0 + j * 32 + row;
+                    if (mm < p.M && c_lane < p.N) *reinterpret_cast<u32x4_t *>(dst + (long long)mm * p.N + c_lane) = o;
+                }
             }
         }
     } else {
@@ -507,13 +515,14 @@ int lq_gemm_fwd_direct_launch(const void *x, const void *codes, const void *scal
 
 // Called by lq_a16w4_gate_up_silu (lq_gemm.hip) after argument validation: K % 256 == 0, N % 16 == 0, M > 16.
 int lq_gemm_fwd_gate_up_launch(const void *x, const void *codes_g, const void *scales_g, const void *zeros_g,
-                               const void *codes_u, const void *scales_u, const void *zeros_u, void *h, int M, int N, int K,
-                               hipStream_t st) {
+                               const void *codes_u, const void *scales_u, const void *zeros_u, void *h, void *g_out, void *u_out,
+                               int M, int N, int K, hipStream_t st) {
     FwdParams p = {};
     p.x = (const unsigned char *)x;
     p.w = (const unsigned char *)codes_g; p.scales = (const unsigned short *)scales_g; p.zeros = (const unsigned short *)zeros_g;
     p.w2 = (const unsigned char *)codes_u; p.scales2 = (const unsigned short *)scales_u; p.zeros2 = (const unsigned short *)zeros_u;
     p.y = (unsigned short *)h;
+    p.g_out = (unsigned short *)g_out; p.u_out = (unsigned short *)u_out;
     p.M = M; p.N = N; p.K = K;
     return launch_direct<2, true>(p, st, "lq_a16w4_gate_up_silu");
 }

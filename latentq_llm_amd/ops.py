@@ -160,9 +160,10 @@ def a16w4_forward_static(x, codes, scales, zeros, shape, out, bias=None):
     return out
 
 
-def a16w4_gate_up_silu(x, gate, up, shape, out=None):
+def a16w4_gate_up_silu(x, gate, up, shape, out=None, save=False):
     """h[M,N] = silu(X . deq(Wgate)^T) * (X . deq(Wup)^T) in one launch (lq_a16w4_gate_up_silu); gate and up are
-    (codes, scales, zeros) triples of two [N, K] matrices. Needs K % 256 == 0 above 16 tokens."""
+    (codes, scales, zeros) triples of two [N, K] matrices. Needs K % 256 == 0 above 16 tokens.
+    save=True (lq_a16w4_gate_up_silu_save) also stores the two products and returns (h, g, u)."""
     N, K = shape
     _chk(x, torch.bfloat16, "x")
     if x.dim() != 2 or x.shape[1] != K:
@@ -177,16 +178,45 @@ def a16w4_gate_up_silu(x, gate, up, shape, out=None):
         _chk(out, torch.bfloat16, "out")
         if tuple(out.shape) != (M, N):
             raise ValueError(f"out must be [{M},{N}]")
-    if M == 0:
-        return out
-    with torch.cuda.device(x.device):
-        _C.call("lq_a16w4_gate_up_silu", x.data_ptr(), gate[0].data_ptr(), gate[1].data_ptr(), gate[2].data_ptr(),
-                up[0].data_ptr(), up[1].data_ptr(), up[2].data_ptr(), out.data_ptr(), M, N, K, GROUP, _stream(x))
-    return out
+    g = torch.empty_like(out) if save else None
+    u = torch.empty_like(out) if save else None
+    if M:
+        with torch.cuda.device(x.device):
+            if save:
+                _C.call("lq_a16w4_gate_up_silu_save", x.data_ptr(), gate[0].data_ptr(), gate[1].data_ptr(), gate[2].data_ptr(),
+                        up[0].data_ptr(), up[1].data_ptr(), up[2].data_ptr(), out.data_ptr(), g.data_ptr(), u.data_ptr(),
+                        M, N, K, GROUP, _stream(x))
+            else:
+                _C.call("lq_a16w4_gate_up_silu", x.data_ptr(), gate[0].data_ptr(), gate[1].data_ptr(), gate[2].data_ptr(),
+                        up[0].data_ptr(), up[1].data_ptr(), up[2].data_ptr(), out.data_ptr(), M, N, K, GROUP, _stream(x))
+    return (out, g, u) if save else out
 
 
-def a16w4_dx(dy, codes, scales, zeros, shape, out=None):
-    """dX[M,K] = dY[M,N] . deq(W)[N,K]."""
+def a16w4_dx_silu_bwd(dy, codes, scales, zeros, shape, g, u):
+    """The backward of a gated MLP's down projection with the backward of h = silu(g) * u as its epilogue
+    (lq_a16w4_dx_silu_bwd): returns (dg, du), bf16 [M, K] each, for dy [M, N] and the saved products g, u [M, K]."""
+    N, K = shape
+    _chk(dy, torch.bfloat16, "dy")
+    if dy.dim() != 2 or dy.shape[1] != N:
+        raise ValueError(f"dy must be [M,{N}], got {tuple(dy.shape)}")
+    _codes_ok(codes, N, K)
+    _qparam_ok(scales, zeros, N, K)
+    M = dy.shape[0]
+    for t, name in ((g, "g"), (u, "u")):
+        _chk(t, torch.bfloat16, name)
+        if tuple(t.shape) != (M, K):
+            raise ValueError(f"{name} must be [{M},{K}]")
+    dg = torch.empty((M, K), dtype=torch.bfloat16, device=dy.device)
+    du = torch.empty((M, K), dtype=torch.bfloat16, device=dy.device)
+    if M:
+        with torch.cuda.device(dy.device):
+            _C.call("lq_a16w4_dx_silu_bwd", dy.data_ptr(), codes.data_ptr(), scales.data_ptr(), zeros.data_ptr(), g.data_ptr(),
+                    u.data_ptr(), dg.data_ptr(), du.data_ptr(), M, N, K, GROUP, _stream(dy))
+    return dg, du
+
+
+def a16w4_dx(dy, codes, scales, zeros, shape, out=None, accumulate=False):
+    """dX[M,K] = dY[M,N] . deq(W)[N,K]; accumulate=True: out = bf16(out + bf16(dY . deq(W))) (lq_a16w4_dx_acc)."""
     N, K = shape
     _chk(dy, torch.bfloat16, "dy")
     if dy.dim() != 2 or dy.shape[1] != N:
@@ -202,6 +232,13 @@ def a16w4_dx(dy, codes, scales, zeros, shape, out=None):
             raise ValueError(f"out must be [{M},{K}]")
         dx = out
     if M == 0:
+        return dx
+    if accumulate:
+        if out is None:
+            raise ValueError("accumulate=True needs out")
+        with torch.cuda.device(dy.device):
+            _C.call("lq_a16w4_dx_acc", dy.data_ptr(), codes.data_ptr(), scales.data_ptr(), zeros.data_ptr(), dx.data_ptr(),
+                    M, N, K, GROUP, _stream(dy))
         return dx
     with torch.cuda.device(dy.device):
         keep, ws, ws_bytes = _workspace(dy, M, K)

@@ -664,13 +664,153 @@ def test_fused_mlp_module_matches_the_three_layers(hip_lib):
     plain = blk.mlp
     fused = make_fused_mlp(blk).mlp
     assert isinstance(fused, QuantLlamaMLP) and fused.gate_proj is plain.gate_proj
-    for tokens in ((2, 3), (4, 128)):  # 6 tokens: composed path; 512 tokens: fused kernel
+    # 6 tokens: the fused GEMV pass; 40 tokens: the composed path (silu and product on the two forward results);
+    # 512 tokens: the fused MFMA kernel
+    for tokens in ((2, 3), (2, 20), (4, 128)):
         x = randn_bf16(tokens + (hid,), 9).cuda()
-        want, got = plain(x), fused(x)
+        with torch.no_grad():
+            want, got = plain(x), fused(x)
         assert got.shape == want.shape == tokens + (hid,)
         err = rel_l2(got.float(), want.float())
         print(f"{tokens}: fused MLP vs layer by layer rel_l2={err:.3e}")
         assert err <= REL_L2_TOL
+
+
+def _mlp_layers(Q, hid, ffn, train):
+    def layer(n, k, seed):
+        _, packed, scales, zeros = make_w4(n, k, seed)
+        m = Q.QLinearA16W4(k, n, bias=False, lbit=16)
+        m.zeros.data, m.scales.data, m.wshape = zeros.clone(), scales.clone(), [n, k]
+        m.weight.set_value(packed, [m.scales, m.zeros, m.wshape])
+        m = m.bfloat16().cuda()
+        m.to("cuda")
+        if train:
+            m.weight.requires_grad = True
+            m.add_hook()
+        return m, (packed, scales, zeros)
+    return layer(ffn, hid, 1), layer(ffn, hid, 2), layer(hid, ffn, 3)
+
+
+def test_fused_mlp_composed_path_with_odd_hidden_size(hip_lib):
+    """A hidden size that is no multiple of 256 takes the composed path at every token count above 16."""
+    from latentq_llm_amd import quant as Q
+    from latentq_llm_amd.fused_mlp import QuantLlamaMLP
+    (g, _), (u, _), (d, _) = _mlp_layers(Q, 384, 512, train=False)
+    fused = QuantLlamaMLP(g, d, u)
+    for tokens in (20, 200):
+        x = randn_bf16((tokens, 384), tokens).cuda()
+        with torch.no_grad():
+            want = d(torch.nn.functional.silu(g(x)) * u(x))
+            got = fused(x)
+        assert rel_l2(got.float(), want.float()) <= REL_L2_TOL
+
+
+@pytest.mark.parametrize("tokens,hid,ffn", [(300, 256, 512), (12, 256, 512), (520, 512, 1408), (40, 384, 512)])
+def test_fused_mlp_training_step(hip_lib, tokens, hid, ffn):
+    """A QuantLlamaMLP whose layers are being trained: output, input gradient and the three weight gradients against
+    the float64 composition, and against the same block run layer by layer through autograd; the hooks' dict_temp
+    is drained; a second backward accumulates. (hid = 384 is not a multiple of 256: the layers' own forward.)"""
+    from latentq_llm_amd import ops, quant as Q
+    from latentq_llm_amd.fused_mlp import QuantLlamaMLP
+    (g, gw), (u, uw), (d, dw_) = _mlp_layers(Q, hid, ffn, train=True)
+    fused = QuantLlamaMLP(g, d, u)
+    x_cpu = randn_bf16((tokens, hid), 5)
+    dy_cpu = randn_bf16((tokens, hid), 6)
+    x = x_cpu.cuda().requires_grad_(True)
+    y = fused(x)
+    y.backward(dy_cpu.cuda())
+    assert len(Q.dict_temp) == 0
+    # float64 composition on the dequantised weights
+    Wg = ops.a16w4_dequant(gw[0].cuda(), gw[1].cuda(), gw[2].cuda(), (ffn, hid)).double().cpu()
+    Wu = ops.a16w4_dequant(uw[0].cuda(), uw[1].cuda(), uw[2].cuda(), (ffn, hid)).double().cpu()
+    Wd = ops.a16w4_dequant(dw_[0].cuda(), dw_[1].cuda(), dw_[2].cuda(), (hid, ffn)).double().cpu()
+    xd = x_cpu.double().requires_grad_(True)
+    gg, uu = xd @ Wg.t(), xd @ Wu.t()
+    hh = torch.nn.functional.silu(gg) * uu
+    yy = hh @ Wd.t()
+    gg.retain_grad(); uu.retain_grad(); hh.retain_grad()
+    yy.backward(dy_cpu.double())
+    errs = {
+        "y": rel_l2(y.detach().cpu(), yy.detach()),
+        "dx": rel_l2(x.grad.cpu(), xd.grad),
+        "dW_down": rel_l2(d.weight.grad.cpu(), dy_cpu.double().t() @ hh.detach()),
+        "dW_up": rel_l2(u.weight.grad.cpu(), uu.grad.t() @ x_cpu.double()),
+        "dW_gate": rel_l2(g.weight.grad.cpu(), gg.grad.t() @ x_cpu.double()),
+    }
+    print(f"fused MLP training ({tokens} tokens, {hid}/{ffn}) rel_l2 vs float64: " + " ".join(f"{k}={v:.2e}" for k, v in errs.items()))
+    assert max(errs.values()) <= REL_L2_TOL
+    # layer by layer through autograd on the same layers: same quantities within bf16 rounding
+    grads = [m.weight.grad.clone() for m in (g, u, d)]
+    for m in (g, u, d):
+        m.weight.grad = None
+    x2 = x_cpu.cuda().requires_grad_(True)
+    y2 = d(torch.nn.functional.silu(g(x2)) * u(x2))
+    y2.backward(dy_cpu.cuda())
+    assert rel_l2(y.detach().float(), y2.detach().float()) <= 6e-3 and rel_l2(x.grad.float(), x2.grad.float()) <= 6e-3
+    for a, m in zip(grads, (g, u, d)):
+        assert rel_l2(a.float(), m.weight.grad.float()) <= 6e-3
+    # accumulation over a second backward of the fused block
+    for m, a in zip((g, u, d), grads):
+        m.weight.grad = a.clone()
+    fused(x).backward(dy_cpu.cuda())
+    for a, m in zip(grads, (g, u, d)):
+        assert rel_l2(m.weight.grad.float(), 2 * a.float()) <= 1e-2
+
+
+def test_fused_mlp_inference_call_refuses_training_inputs(hip_lib):
+    from latentq_llm_amd import quant as Q
+    from latentq_llm_amd.fused_mlp import QuantLlamaMLP
+    (g, _), (u, _), (d, _) = _mlp_layers(Q, 256, 512, train=True)
+    fused = QuantLlamaMLP(g, d, u)
+    with pytest.raises(RuntimeError, match="no backward"):
+        fused.fused_gate_up(randn_bf16((20, 256), 1).cuda())
+
+
+@pytest.mark.parametrize("M,N,K", [(2048, 1024, 512), (300, 272, 256), (7, 512, 384), (16, 256, 256)])
+def test_gate_up_silu_save_stores_the_products(ops, M, N, K):
+    """The training form of the fused gate / up launch: h equals the inference form bit for bit, and the stored
+    products are X . deq(W)^T of the two matrices (float64 bar; above 16 tokens also the bf16 rounding of the very
+    sums h was formed from: silu(g) * u recomputed from them stays within 2 bf16 ulps of h)."""
+    _, pg, sg, zg = make_w4(N, K, 1)
+    _, pu, su, zu = make_w4(N, K, 2)
+    gate, up = (dev(pg), dev(sg), dev(zg)), (dev(pu), dev(su), dev(zu))
+    x = dev(randn_bf16((M, K), 3))
+    h0 = ops.a16w4_gate_up_silu(x, gate, up, (N, K))
+    h, g, u = ops.a16w4_gate_up_silu(x, gate, up, (N, K), save=True)
+    assert torch.equal(h, h0)
+    Wg = ops.a16w4_dequant(*gate, (N, K)).double()
+    Wu = ops.a16w4_dequant(*up, (N, K)).double()
+    assert rel_l2(g, x.double() @ Wg.t()) < 3e-3 and rel_l2(u, x.double() @ Wu.t()) < 3e-3
+    re = torch.nn.functional.silu(g.double()) * u.double()
+    assert bool(((h.double() - re).abs() <= re.abs() * 2.0 ** -6 + 1e-6).all())
+
+
+@pytest.mark.parametrize("M,N,K", [(2048, 1024, 512), (100, 256, 384), (520, 1408, 512)])
+def test_dx_epilogue_forms(ops, M, N, K):
+    """lq_a16w4_dx_acc = lq_a16w4_dx followed by a bf16 addition, bit for bit; lq_a16w4_dx_silu_bwd against the fp32
+    formula on the bf16-rounded product (1 ulp: exp and reciprocal are the hardware's)."""
+    codes, packed, scales, zeros = make_w4(N, K, 3)
+    w = (dev(packed), dev(scales), dev(zeros))
+    dy = dev(randn_bf16((M, N), 4))
+    base = dev(randn_bf16((M, K), 5, 30.0))
+    p = ops.a16w4_dx(dy, *w, (N, K))
+    acc = base.clone()
+    ops.a16w4_dx(dy, *w, (N, K), out=acc, accumulate=True)
+    assert torch.equal(acc, base + p)
+    g, u = dev(randn_bf16((M, K), 6, 2.0)), dev(randn_bf16((M, K), 7))
+    dg, du = ops.a16w4_dx_silu_bwd(dy, *w, (N, K), g, u)
+    pf, gf, uf = p.double(), g.double(), u.double()
+    sg = torch.sigmoid(gf)
+    want_dg = pf * uf * sg * (1 + gf * (1 - sg))
+    want_du = pf * gf * sg
+    assert rel_l2(dg, want_dg) < 3e-3 and rel_l2(du, want_du) < 3e-3
+    # elementwise: within 2 bf16 ulps of the size of the factors (silu'(g) passes through zero near g = -1.28, so the
+    # bound is relative to |P u| and |P g|, not to the result)
+    for got, want, scale in ((dg, want_dg, (pf * uf).abs() * 1.1), (du, want_du, (pf * gf).abs())):
+        diff = (got.double() - want).abs()
+        # (the absolute term: P here comes from a launch that may cut the reduction differently, and where the sum
+        # cancels the two fp32 sums differ by more than a bf16 ulp of the small result)
+        assert bool((diff <= scale * 2.0 ** -7 + 2e-5 * (1 + uf.abs() + gf.abs())).all())
 
 
 @pytest.mark.parametrize("N,K", [(1, 8), (12, 64), (100, 1032), (2048, 8192)])
