@@ -358,6 +358,24 @@ int lq_gradq8_quant(const void *dw, int8_t *q_inout, void *scale_inout, int accu
                     const void *noise_or_null, uint64_t philox_seed, uint64_t philox_offset, void *stream);
 
 /* ---------------------------------------------------------------------------
+ * Weight gradient of a quantised linear layer, dW[N,K] = dY[M,N]^T . X[M,K] (bf16, fp32 accumulation):
+ * `grad_output.t().mm(input)` of QLinearFunctionW4.backward and its A8W8 / QAT siblings (reference
+ * utils/quant.py:141-142, 207, 248, 289, 370). Both operands are read as they lie in memory (no transposed
+ * copy). dy: bf16 [M,N]; x: bf16 [M,K]; M % 64 == 0, N % 8 == 0; dy, x and the output 16-byte aligned.
+ *   lq_weight_grad:      dw_out = bf16(dW), bf16 [N,K], K % 8 == 0.
+ *   lq_weight_grad_acc8: the product with the add_ form of the 8-bit gradient accumulator as its epilogue
+ *     (GradientQTensor.add_, utils/quant.py:891-898, reached from backward_hook_fn :398-411 on every
+ *     micro-batch after the first): with d = bf16(dW),
+ *       x = bf16(bf16(q * scale[n]) + d),  q[n,k] = clamp(rint(bf16(bf16(x / scale[n]) + noise[n,k])), -128, 127)
+ *     in place; exactly lq_weight_grad followed by lq_gradq8_quant(accumulate = 1) with the same noise
+ *     arguments, without dW ever being stored. q_inout: int8 [N,K]; scale: bf16 [N] (read); K % 16 == 0.
+ * ------------------------------------------------------------------------- */
+int lq_weight_grad(const void *dy, const void *x, void *dw_out, int64_t M, int64_t N, int64_t K, void *stream);
+int lq_weight_grad_acc8(const void *dy, const void *x, int8_t *q_inout, const void *scale, int64_t M, int64_t N,
+                        int64_t K, const void *noise_or_null, uint64_t philox_seed, uint64_t philox_offset,
+                        void *stream);
+
+/* ---------------------------------------------------------------------------
  * Layout converters (device side).
  * GPTQ layout (reference PTQ/quant/quant_linear.py:343-389): qweight is
  * int32[K/8, N] with code(k, n) at bits 4*(k%8) of word [k/8, n].

@@ -14,67 +14,20 @@
 // row before its first element can be quantised; rows of up to 12 288 elements stay in registers in between,
 // longer ones are read a second time (from L2).
 #include "lq_common.h"
+#include "lq_gradq8_math.h"
 
 namespace {
 
-__device__ __forceinline__ float bf16r(float v) { return lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(v)); }
-
-// byte SEL of `old` replaced by sat_u8(rne(v)) (v_cvt_pk_u8_f32: saturates to 0..255, NaN -> 0)
-template <int SEL>
-__device__ __forceinline__ unsigned cvt_pk_u8(float v, unsigned old) {
-    unsigned r;
-    asm("v_cvt_pk_u8_f32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "n"(SEL), "v"(old));
-    return r;
-}
-
-__device__ __forceinline__ float bf16_of(const u32x4_t v, int j) { return (j & 1) ? lq_bf16_hi(v[j >> 1]) : lq_bf16_lo(v[j >> 1]); }
-
-// 16 consecutive elements (two 16-byte pieces of dW, 16 old int8, one Philox block or two pieces of noise).
-//
-// kFast (2^-40 <= s <= 2^40): only bf16(x / s) is needed, x and s are bf16 numbers, and the quotient of two
-// 8-bit significands is never closer than 2^-17 (relative) to a bf16 rounding tie (a tie has a 9-bit odd
-// significand t, and s t = x has no solution with x below 2^8), while x RN(1/s) is within 2^-23 of it: the
-// product rounds to the same bf16 number as the IEEE quotient. Where the quotient is a bf16 subnormal that
-// argument fails, and there the sum with the noise and the final code are the same for both anyway. Infinities
-// and NaN go the same way through the product as through the quotient.
-// clamp(rint(y), -128, 127) is taken as sat_u8(rne(y + 128)) - 128: y is a bf16 number, so y + 128 is exact
-// in fp32 whenever |y| >= 2^-8, below that both forms give 0, and ties keep their parity. NaN -> -128.
-template <bool kPhilox, bool kAcc, bool kFast>
-__device__ __forceinline__ u32x4_t quant16(const u32x4_t v0, const u32x4_t v1, const u32x4_t old, const u32x4_t n0,
-                                           const u32x4_t n1, float s, float r, unsigned long long counter,
-                                           unsigned long long seed) {
-    unsigned w[4] = {0u, 0u, 0u, 0u};
-    if (kPhilox) {
-        const lq_u4 A = lq_philox4x32_10((unsigned)counter, (unsigned)(counter >> 32), 0u, 0u, (unsigned)seed,
-                                         (unsigned)(seed >> 32));
-        w[0] = A.x; w[1] = A.y; w[2] = A.z; w[3] = A.w;
-    }
-    unsigned o[4] = {0u, 0u, 0u, 0u};
+// Largest magnitude as a bit pattern: magnitudes of bf16 numbers order like unsigned integers and every NaN pattern
+// lies above infinity, so that a NaN anywhere in the row ends up in the maximum (as the tensor library's amax does).
+__device__ __forceinline__ unsigned absmax8(const u32x4_t v, unsigned m) {
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-        float x = j < 8 ? bf16_of(v0, j) : bf16_of(v1, j - 8);
-        if (kAcc) {
-            const int qi = (int)(signed char)((old[j >> 2] >> (8 * (j & 3))) & 0xFFu);
-            x = bf16r(bf16r((float)qi * s) + x);
-        }
-        float nz;
-        if (kPhilox) nz = fmaf((float)((w[j >> 2] >> (8 * (j & 3))) & 0xFFu), 0x1p-8f, 0x1p-9f - 0.5f);  // (2b - 255) / 512
-        else nz = j < 8 ? bf16_of(n0, j) : bf16_of(n1, j - 8);
-        const float q = kFast ? x * r : x / s;
-        const float y = bf16r(bf16r(q) + nz) + 128.0f;
-        switch (j & 3) {
-            case 0: o[j >> 2] = cvt_pk_u8<0>(y, o[j >> 2]); break;
-            case 1: o[j >> 2] = cvt_pk_u8<1>(y, o[j >> 2]); break;
-            case 2: o[j >> 2] = cvt_pk_u8<2>(y, o[j >> 2]); break;
-            default: o[j >> 2] = cvt_pk_u8<3>(y, o[j >> 2]); break;
-        }
+    for (int j = 0; j < 4; ++j) {
+        const unsigned a = v[j] & 0x7FFF7FFFu;
+        const unsigned lo = a & 0xFFFFu, hi = a >> 16;
+        m = m > lo ? m : lo;
+        m = m > hi ? m : hi;
     }
-    return u32x4_t{o[0] ^ 0x80808080u, o[1] ^ 0x80808080u, o[2] ^ 0x80808080u, o[3] ^ 0x80808080u};
-}
-
-__device__ __forceinline__ float absmax8(const u32x4_t v, float m) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) m = fmaxf(m, fmaxf(fabsf(lq_bf16_lo(v[j])), fabsf(lq_bf16_hi(v[j]))));
     return m;
 }
 
@@ -89,7 +42,7 @@ __global__ __launch_bounds__(256) void gradq8_kernel(const unsigned short *__res
                                                      unsigned long long offset) {
     constexpr int R = 256 / T;      // rows per workgroup
     constexpr int STEP = 16 * T;    // elements of a row the row's threads take per piece
-    __shared__ float red[4];
+    __shared__ unsigned red[4];
     const int tid = threadIdx.x % T;
     const long long n_raw = (long long)blockIdx.x * R + threadIdx.x / T;
     const bool live = n_raw < N;    // rows past the end still take part in the barrier
@@ -116,27 +69,37 @@ __global__ __launch_bounds__(256) void gradq8_kernel(const unsigned short *__res
     }
     float s;
     if (!kAcc) {
-        float m = 0.0f;
+        unsigned mb = 0u;
         if (kPieces > 0) {
 #pragma unroll
-            for (int i = 0; i < kPieces; ++i) m = absmax8(h1[i], absmax8(h0[i], m));
+            for (int i = 0; i < kPieces; ++i) mb = absmax8(h1[i], absmax8(h0[i], mb));
         } else {
             for (long long k = (long long)tid * 16; k < K; k += STEP)
-                m = absmax8(*reinterpret_cast<const u32x4_t *>(row + k + 8), absmax8(*reinterpret_cast<const u32x4_t *>(row + k), m));
+                mb = absmax8(*reinterpret_cast<const u32x4_t *>(row + k + 8), absmax8(*reinterpret_cast<const u32x4_t *>(row + k), mb));
         }
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+        for (int o = 32; o > 0; o >>= 1) {
+            const unsigned other = (unsigned)__shfl_xor((int)mb, o);
+            mb = mb > other ? mb : other;
+        }
         if constexpr (T > 64) {
             // waves of one row are neighbours: wave w belongs to row group w / (T / 64)
             const int wave = threadIdx.x >> 6;
-            if ((threadIdx.x & 63) == 0) red[wave] = m;
+            if ((threadIdx.x & 63) == 0) red[wave] = mb;
             __syncthreads();
-            if constexpr (T == 256) m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-            else m = fmaxf(red[wave & ~1], red[wave | 1]);
+            if constexpr (T == 256) {
+                const unsigned a = red[0] > red[1] ? red[0] : red[1], b = red[2] > red[3] ? red[2] : red[3];
+                mb = a > b ? a : b;
+            } else {
+                mb = red[wave & ~1] > red[wave | 1] ? red[wave & ~1] : red[wave | 1];
+            }
         }
+        const float m = __uint_as_float(mb << 16);
         const float vmax = bf16r(m * 4.0f);
         const float lo = bf16r(1e-5f);
-        s = bf16r(fmaxf(vmax, lo) * (1.0f / 127.0f));
+        // a NaN row maximum stays NaN through the floor (torch.clamp keeps it): the row's scale and with it the
+        // dequantised gradient are NaN, as in the reference
+        s = vmax != vmax ? vmax : bf16r(fmaxf(vmax, lo) * (1.0f / 127.0f));
         if (tid == 0 && live) scale[n] = lq_f32_to_bf16_bits(s);
     } else {
         s = lq_bf16_bits_to_f32(scale[n]);

@@ -48,7 +48,7 @@ class _FusedMLPTrain(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        from .quant import backward_hook_fn, dict_temp
+        from .quant import _pending_dw, backward_hook_fn, dict_temp
         x2, g, u, h = ctx.saved_tensors
         mlp = ctx.mlp
         gate, up, down = mlp.gate_proj, mlp.up_proj, mlp.down_proj
@@ -61,7 +61,7 @@ class _FusedMLPTrain(torch.autograd.Function):
             ops.a16w4_dx(du, *_w4(up), (inter, K), out=dx, accumulate=True)
         for layer, dyl, xin in ((down, dy, h), (up, du, x2), (gate, dg, x2)):
             if layer.hook_handle is not None:
-                dict_temp.append(ops.weight_grad(dyl, xin))
+                dict_temp.append(_pending_dw(dyl, xin))
                 backward_hook_fn(layer, None, None)
         return dx, None
 

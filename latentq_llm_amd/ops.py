@@ -463,13 +463,46 @@ def transpose_bf16(x):
     return out
 
 
+def _weight_grad_native_ok(dy, x, k_mult=8):
+    return (dy.is_cuda and x.is_cuda and dy.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and dy.dim() == 2
+            and x.dim() == 2 and dy.is_contiguous() and x.is_contiguous() and dy.shape[0] == x.shape[0]
+            and dy.shape[0] > 0 and dy.shape[0] % 64 == 0 and dy.shape[1] % 8 == 0 and x.shape[1] % k_mult == 0
+            and dy.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0)
+
+
 def weight_grad(dy, x):
-    """dW = dY^T X for 2-D bf16 operands: the vendor GEMM on a transposed copy of dY when the
-    shapes allow it, on the strided view otherwise."""
+    """dW = dY^T X for 2-D operands: the library's own GEMM (lq_weight_grad: both operands read as they lie in
+    memory) for bf16 GPU operands with a multiple of 64 tokens, the tensor library's product otherwise."""
+    if _weight_grad_native_ok(dy, x):
+        N, K = dy.shape[1], x.shape[1]
+        dw = torch.empty((N, K), dtype=torch.bfloat16, device=dy.device)
+        with torch.cuda.device(dy.device):
+            _C.call("lq_weight_grad", dy.data_ptr(), x.data_ptr(), dw.data_ptr(), dy.shape[0], N, K, _stream(dy))
+        return dw
     if (dy.is_cuda and dy.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and dy.dim() == 2 and dy.is_contiguous()
             and dy.shape[0] % 8 == 0 and dy.shape[1] % 8 == 0 and dy.shape[0] >= 256):
         return transpose_bf16(dy).mm(x)
     return dy.t().mm(x)
+
+
+def weight_grad_acc8(dy, x, q, scale, noise=None, seed: int = 0, offset: int = 0):
+    """q = quant(dequant(q) + dY^T X) in place (lq_weight_grad_acc8): the weight-gradient GEMM with the add_ form of
+    the 8-bit gradient accumulator as its epilogue. dy bf16 [M,N], x bf16 [M,K], q int8 [N,K], scale bf16 [N,1]."""
+    if not _weight_grad_native_ok(dy, x, 16):
+        raise ValueError("weight_grad_acc8 needs contiguous bf16 GPU operands, M % 64 == 0, N % 8 == 0, K % 16 == 0")
+    N, K = dy.shape[1], x.shape[1]
+    _chk(q, torch.int8, "q")
+    _chk(scale, torch.bfloat16, "scale")
+    if tuple(q.shape) != (N, K) or scale.numel() != N:
+        raise ValueError("q must be [N, K] and scale hold N entries")
+    if noise is not None:
+        _chk(noise, torch.bfloat16, "noise")
+        if tuple(noise.shape) != (N, K):
+            raise ValueError("noise must be [N, K]")
+    with torch.cuda.device(dy.device):
+        _C.call("lq_weight_grad_acc8", dy.data_ptr(), x.data_ptr(), q.data_ptr(), scale.data_ptr(), dy.shape[0], N, K,
+                None if noise is None else noise.data_ptr(), seed & (2**64 - 1), offset & (2**64 - 1), _stream(dy))
+    return q
 
 
 def repack_gptq_to_native(qweight, shape):

@@ -143,7 +143,7 @@ def Qfunc_8bit_res(tensor, residual_handle, qscales):
     if (FUSED_LATENT and not isinstance(residual_handle, ResidualTensor) and tensor.is_cuda and tensor.dim() == 2
             and tensor.dtype == torch.bfloat16 and tensor.is_contiguous() and tensor.shape[1] % 8 == 0
             and tensor.data_ptr() % 16 == 0 and torch.is_tensor(qscales) and qscales.dtype == torch.bfloat16
-            and qscales.is_contiguous() and qscales.numel() == tensor.shape[0]):
+            and qscales.is_contiguous() and qscales.dim() == 2 and tuple(qscales.shape) == (tensor.shape[0], 1)):
         # the chain below as one pass (same roundings)
         if residual_handle is not None:
             residual_handle.data = tensor.to(residual_handle.dtype)
@@ -156,6 +156,29 @@ def Qfunc_8bit_res(tensor, residual_handle, qscales):
     elif residual_handle is not None:
         residual_handle.data = tensor.to(residual_handle.dtype)
     return q.clamp_(-128, 127).to(torch.int8)
+
+
+# ---------------------------------------------------------------------- pending weight gradient --
+class _PendingWeightGrad(object):
+    """dW = dY^T X of one backward, not formed yet: the autograd Functions hand this to the backward hook through
+    dict_temp, and the hook either forms the product straight into an int8 gradient accumulator
+    (``GradientQTensor.add_product_``: the GEMM's epilogue does the accumulation and dW is never stored) or
+    materialises the bf16 tensor (``tensor()``), which is what every other consumer gets."""
+    __slots__ = ("dy", "x")
+
+    def __init__(self, dy, x):
+        self.dy, self.x = dy, x
+
+    def tensor(self):
+        return ops.weight_grad(self.dy, self.x)
+
+
+def _pending_dw(grad_output, input):
+    """What a Function's backward appends to dict_temp: the pending product where the library's own GEMM can form it
+    (contiguous bf16 GPU operands, a multiple of 64 tokens), the product itself otherwise."""
+    if FUSED_GRADQ and ops._weight_grad_native_ok(grad_output, input):
+        return _PendingWeightGrad(grad_output, input)
+    return ops.weight_grad(grad_output, input)
 
 
 # ------------------------------------------------------------------------ autograd: A16W4 --
@@ -200,7 +223,7 @@ class QLinearFunctionW4(torch.autograd.Function):
             grad_input = ops.a16w4_dx(dy, weight_d, scales, zeros, shape)
             if grad_input.dtype != input.dtype:
                 grad_input = grad_input.to(input.dtype)
-        dict_temp.append(ops.weight_grad(grad_output, input))  # dW = dY^T X (utils/quant.py:141-142)
+        dict_temp.append(_pending_dw(dy, _as_bf16_2d(input)))  # dW = dY^T X (utils/quant.py:141-142)
         if bias is not None and ctx.needs_input_grad[_BIAS_FLAG]:
             grad_bias = grad_output.sum(0)
         return grad_input, None, None, grad_bias
@@ -290,8 +313,7 @@ def _a8w8_backward_common(ctx, grad_output, input_f, weight_f, bias, detach_dw):
     grad_input = grad_bias = None
     if ctx.needs_input_grad[0]:
         grad_input = grad_output.mm(weight_f)
-    dw = ops.weight_grad(grad_output, input_f)
-    dict_temp.append(dw.data if detach_dw else dw)
+    dict_temp.append(_pending_dw(grad_output, input_f))
     if bias is not None and ctx.needs_input_grad[_BIAS_FLAG]:
         grad_bias = grad_output.sum(0)
     return grad_input, None, None, grad_bias
@@ -432,6 +454,11 @@ def backward_hook_fn(module, grad_out, grad_in):
     assert len(dict_temp) == 1
     dw = dict_temp.pop()
     g = module.weight.grad
+    if isinstance(dw, _PendingWeightGrad):
+        if isinstance(g, GradientQTensor) and g.acc_ite > 0 and g.can_add_product(dw.dy, dw.x):
+            g.add_product_(dw.dy, dw.x)
+            return
+        dw = dw.tensor()
     if isinstance(g, GradientQTensor):
         if g.acc_ite == 0:
             g.set_value(dw)
@@ -804,8 +831,18 @@ class GradientQTensor(object):
     a running counter shared by all instances); ``noise=`` injects a bf16 tensor instead. Anything
     else (CPU tensors, other dtypes, FUSED_GRADQ off) runs the tensor-op chain with ``uniform_``."""
 
-    noise_seed = 0x6B0D
+    # Key of the rounding-noise stream. None: taken from torch.initial_seed() at first use, so that
+    # torch.manual_seed() before training changes the noise as it does for the reference's uniform_(); set it to
+    # an integer to fix the stream by hand. The counter offset is a host-side count passed with every launch: a
+    # launch captured into a HIP graph would replay the same noise, so accumulators must not be captured.
+    noise_seed = None
     _noise_offset = 0  # Philox blocks consumed so far by all instances
+
+    @classmethod
+    def _seed(cls):
+        if cls.noise_seed is None:
+            cls.noise_seed = torch.initial_seed() & (2 ** 64 - 1)
+        return cls.noise_seed
 
     def __init__(self, shape, bit=8):
         self.acc_ite = 0
@@ -831,7 +868,7 @@ class GradientQTensor(object):
         if not accumulate:
             self.qdata = torch.empty(fdata.shape, dtype=torch.int8, device=fdata.device)
             self.scale = torch.empty((fdata.shape[0], 1), dtype=torch.bfloat16, device=fdata.device)
-        ops.gradq8_quant(fdata, self.qdata, self.scale, accumulate, noise=noise, seed=cls.noise_seed, offset=cls._noise_offset)
+        ops.gradq8_quant(fdata, self.qdata, self.scale, accumulate, noise=noise, seed=cls._seed(), offset=cls._noise_offset)
         if noise is None:
             cls._noise_offset += (fdata.numel() + 15) // 16
 
@@ -872,6 +909,24 @@ class GradientQTensor(object):
             self._hip_quant(fdata, True, noise)
         else:
             self.quant(self.dequant() + fdata, noise)
+
+    def can_add_product(self, dy, x):
+        """Whether add_product_ applies: an 8-bit accumulator that already holds a micro-batch, on the GPU, and
+        operands the weight-gradient GEMM takes."""
+        return (FUSED_GRADQ and self.bit == 8 and isinstance(self.qdata, torch.Tensor) and self.qdata.is_cuda
+                and self.qdata.is_contiguous() and self.qdata.dtype == torch.int8 and self.scale is not None
+                and self.scale.dtype == torch.bfloat16 and self.scale.is_contiguous()
+                and getattr(self, "fdtype", None) == torch.bfloat16 and ops._weight_grad_native_ok(dy, x, 16)
+                and tuple(self.qdata.shape) == (dy.shape[1], x.shape[1]))
+
+    def add_product_(self, dy, x, noise=None):
+        """add_(dy.t().mm(x)) without the product ever being stored: the GEMM's epilogue re-quantises
+        dequant() + dW in place (ops.weight_grad_acc8), bit for bit what add_ does with the bf16 product."""
+        cls = GradientQTensor
+        self.acc_ite += 1
+        ops.weight_grad_acc8(dy, x, self.qdata, self.scale, noise=noise, seed=cls._seed(), offset=cls._noise_offset)
+        if noise is None:
+            cls._noise_offset += (self.qdata.numel() + 15) // 16
 
     def get_value(self):
         return self.qdata if self.bit > 8 else self.dequant()

@@ -392,14 +392,15 @@ void lqo_gradq8(const uint16_t *dw, int8_t *q, uint16_t *scale, int accumulate, 
         float s;
         if (!accumulate) {
             float m = 0.0f;
-            for (int64_t k = 0; k < K; ++k) {
+            for (int64_t k = 0; k < K && m == m; ++k) {
                 float a = fabsf(bf16_to_f32(dw[n * K + k]));
-                if (a > m) m = a;
+                if (a != a || a > m) m = a; /* data.abs().amax() returns NaN for a row that holds one */
             }
             float vmax = bf16_round(m * 4.0f);
             float lo = bf16_round(1e-5f);
             volatile float inv = 1.0f / 127.0f;
-            s = bf16_round((vmax > lo ? vmax : lo) * inv);
+            /* torch.clamp(vmax, min = 1e-5) keeps a NaN */
+            s = vmax != vmax ? vmax : bf16_round((vmax > lo ? vmax : lo) * inv);
             scale[n] = f32_to_bf16(s);
         } else {
             s = bf16_to_f32(scale[n]);

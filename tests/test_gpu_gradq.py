@@ -165,6 +165,55 @@ def test_qlinear_a16w4_with_8bit_gradient_accumulation(Q):
     assert (m.weight.data != before).any()
 
 
+def test_8bit_accumulation_through_the_gemm_epilogue_equals_the_separate_pass(Q, ops):
+    """With a multiple of 64 tokens the backward hook forms dW straight into the int8 accumulator from the second
+    micro-batch on (GradientQTensor.add_product_: the weight-gradient GEMM's epilogue). The stored codes and scales
+    equal, bit for bit, set_value / add_ applied to the separately formed bf16 products with the same noise stream."""
+    N, K, M = 128, 256, 192
+    codes, packed, scales, zeros = make_w4(N, K, 31)
+    m = Q.QLinearA16W4(K, N, bias=False, lbit=0, gbit=8)
+    m.zeros.data, m.scales.data, m.wshape = zeros.clone(), scales.clone(), [N, K]
+    m.weight.set_value(packed, [m.scales, m.zeros, m.wshape])
+    m = m.bfloat16().cuda()
+    m.to("cuda")
+    m.weight.requires_grad = True
+    m.add_hook()
+    x = randn_bf16((M, K), 32).cuda().requires_grad_(True)
+    dys = [randn_bf16((M, N), 33 + i).cuda() for i in range(3)]
+    cls = Q.GradientQTensor
+    saved = (cls.noise_seed, cls._noise_offset)
+    calls = []
+    real = ops.weight_grad_acc8
+    try:
+        cls.noise_seed, cls._noise_offset = 4242, 1000
+        ops.weight_grad_acc8 = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
+        for dy in dys:
+            m(x).backward(dy)
+        g = m.weight.grad
+        assert g.acc_ite == 3 and len(calls) == 2 and len(Q.dict_temp) == 0
+        # the same three micro-batches through the separate passes
+        ref = cls([N, K], bit=8)
+        cls.noise_seed, cls._noise_offset = 4242, 1000
+        ref.set_value(ops.weight_grad(dys[0], x.detach()))
+        for dy in dys[1:]:
+            ref.add_(ops.weight_grad(dy, x.detach()))
+        assert torch.equal(g.scale, ref.scale) and torch.equal(g.qdata, ref.qdata)
+    finally:
+        ops.weight_grad_acc8 = real
+        cls.noise_seed, cls._noise_offset = saved
+
+
+def test_noise_seed_follows_torch_manual_seed(Q):
+    cls = Q.GradientQTensor
+    saved = (cls.noise_seed, cls._noise_offset)
+    try:
+        cls.noise_seed = None
+        torch.manual_seed(987654321)
+        assert cls._seed() == 987654321 and cls.noise_seed == 987654321
+    finally:
+        cls.noise_seed, cls._noise_offset = saved
+
+
 # --------------------------------------------------------------- 8-bit weights in the optimizer --
 def _a8w8_layer(Q, N, K, lbit, seed):
     g = torch.Generator().manual_seed(seed)

@@ -461,6 +461,21 @@ def test_gradq8_oracle_matches_torch_bf16_tensor_ops(N, K, std):
     assert np.abs(q.astype(int)).max() <= 128 and (q != 0).mean() > 0.5
 
 
+def test_gradq8_nan_row_gives_nan_scale_as_the_tensor_chain():
+    """A NaN in a row of dW: data.abs().amax() and torch.clamp keep it, so the row's scale (and with it the
+    dequantised gradient) is NaN in the reference's chain; the restatement does the same, other rows are untouched."""
+    N, K = 4, 64
+    dw = randn_bf16((N, K), 2, 0.01)
+    dw[2, 17] = float("nan")
+    nz = (torch.rand(N, K, generator=torch.Generator().manual_seed(3)) - 0.5).to(torch.bfloat16)
+    want_q, want_s = tr.gradq8_set(dw, nz)
+    q, s = co.gradq8(bits(dw), None, None, False, N, K, noise=bits(nz))
+    assert torch.isnan(want_s[2]).all() and np.isnan(co.bf16_bits_to_f32(s)[2])
+    keep = [0, 1, 3]
+    assert np.array_equal(s[keep], bits(want_s).reshape(-1)[keep])
+    assert np.array_equal(q.reshape(N, K)[keep], want_q.numpy()[keep])
+
+
 def test_gradq8_philox_noise_definition():
     """Without injected noise element i draws (2 b_i - 255) / 512, b_i = byte i & 3 of word (i >> 2) & 3 of the
     Philox block with counter offset + i / 16 (recomputed here from the pinned block function): 256 equally
