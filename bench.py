@@ -271,11 +271,26 @@ def bench_a8w8(device):
         sec = event_time(lambda: ops.a8w8_forward(x8, w8, sx, sw), 20)
         out.append({"M": M, "N": N, "K": K, "us": sec * 1e6, "TOP/s": 2 * M * N * K / sec / 1e12,
                     "frac_mfma_i8": 2 * M * N * K / sec / PEAK_I8})
-    # the activation quantiser in front of the GEMM (bf16 -> int8, clamp value on the device)
+    # what the int8 matrix pipes deliver with nothing else in the loop (random and all-zero operands, two waves per SIMD)
+    ceil = {}
+    for name, zero in (("random_operands", False), ("zero_operands", True)):
+        tops, ghz = mfma_loop_i8(device, zero)
+        ceil[f"mfma_loop_i8_{name}"] = {"TOP/s": tops, "clock_GHz": ghz}
+    loop = ceil["mfma_loop_i8_random_operands"]["TOP/s"]
+    for rec in out:
+        rec["achieved_over_ceiling"] = rec["TOP/s"] / loop
+    out.append({"ceiling": ceil})
+    # the activation quantisers in front of the GEMM (bf16 -> int8): given clamp value, the tensor's own maximum
+    # found on the device (two launches), one scale per token row
     x = torch.randn(M, 8192, device=device).to(torch.bfloat16)
     clampv = x.float().abs().max().reshape(1)
     sec = event_time(lambda: ops.act_quant_i8(x, clampv), 20)
     out.append({"act_quant": [M, 8192], "us": sec * 1e6, "GB/s": 3 * x.numel() / sec / 1e9})
+    sec = event_time(lambda: ops.act_quant_i8_dynamic(x), 20)
+    out.append({"act_quant_dynamic": [M, 8192], "us": sec * 1e6, "GB/s": 5 * x.numel() / sec / 1e9,
+                "bytes_per_element": 5, "what": "max pass (2 B read) + quantise pass (2 B read, 1 B written)"})
+    sec = event_time(lambda: ops.act_quant_i8_per_token(x), 20)
+    out.append({"act_quant_per_token": [M, 8192], "us": sec * 1e6, "GB/s": 3 * x.numel() / sec / 1e9})
     return out
 
 
@@ -320,8 +335,9 @@ def bench_adam8(device):
 
 
 def bench_dw(device):
-    """dW = dY^T X of the two MLP shapes (not part of `value`): the vendor GEMM on the strided view, as
-    the reference calls it, against the transposed-copy form the drop-in modules use."""
+    """dW = dY^T X of the two MLP shapes (not part of `value`): the library's own GEMM (operands read as they lie),
+    the same with the int8 accumulator's add_ as its epilogue, and for scale the vendor GEMM on the strided view (as
+    the reference calls it) and on a transposed copy of dY."""
     from latentq_llm_amd import ops
     out = []
     for (N, K) in [(FFN, HID), (HID, FFN)]:
@@ -329,11 +345,16 @@ def bench_dw(device):
         x = torch.randn(TOKENS, K, device=device).to(torch.bfloat16)
         flop = 2 * TOKENS * N * K
         t_ref = event_time(lambda: dy.t().mm(x), 20)
-        t_tr = event_time(lambda: ops.transpose_bf16(dy), 20)
+        t_tr = event_time(lambda: ops.transpose_bf16(dy).mm(x), 20)
         t_new = event_time(lambda: ops.weight_grad(dy, x), 20)
+        q8 = torch.zeros((N, K), dtype=torch.int8, device=device)
+        sc = torch.full((N, 1), 1e-3, dtype=torch.bfloat16, device=device)
+        t_acc = event_time(lambda: ops.weight_grad_acc8(dy, x, q8, sc, seed=1, offset=0), 20)
         out.append({"N": N, "K": K, "strided_mm_us": t_ref * 1e6, "strided_mm_TFLOP/s": flop / t_ref / 1e12,
-                    "transpose_us": t_tr * 1e6, "transpose_GB/s": 4 * TOKENS * N / t_tr / 1e9,
-                    "weight_grad_us": t_new * 1e6, "weight_grad_TFLOP/s": flop / t_new / 1e12})
+                    "transposed_copy_mm_us": t_tr * 1e6, "transposed_copy_mm_TFLOP/s": flop / t_tr / 1e12,
+                    "weight_grad_us": t_new * 1e6, "weight_grad_TFLOP/s": flop / t_new / 1e12,
+                    "frac_mfma_bf16": flop / t_new / PEAK_BF16,
+                    "weight_grad_acc8_us": t_acc * 1e6, "weight_grad_acc8_TFLOP/s": flop / t_acc / 1e12})
     return out
 
 
@@ -369,6 +390,30 @@ def mfma_loop(device, zero_operands, wgs_per_cu=2, seconds=0.004):
     sec = event_time(lambda: run(iters), 5, warm=3, warm_seconds=0.1)
     flop = waves * iters * 8 * 32768.0
     return flop / sec / 1e12, _clock_ghz(clocks, waves)
+
+
+def mfma_loop_i8(device, zero_operands, wgs_per_cu=2):
+    """The MFMA-only loop on the int8 instruction (lq_calib_mfma_loop_i8): (TOP/s, granted shader clock in GHz)."""
+    import ctypes
+    from latentq_llm_amd import _C
+    n = 1 << 20
+    if zero_operands:
+        a = torch.zeros(n, dtype=torch.int8, device=device)
+        b = torch.zeros(n, dtype=torch.int8, device=device)
+    else:
+        a = torch.randint(-127, 128, (n,), dtype=torch.int8, device=device)
+        b = torch.randint(-127, 128, (n,), dtype=torch.int8, device=device)
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    waves = 4 * cus * wgs_per_cu
+    clocks = torch.zeros(4 * waves, dtype=torch.int64, device=device)
+    sink = torch.zeros(waves, dtype=torch.int32, device=device)
+    nw = ctypes.c_int64()
+    st = torch.cuda.current_stream().cuda_stream
+    iters = 20000
+    sec = event_time(lambda: _C.call("lq_calib_mfma_loop_i8", a.data_ptr(), b.data_ptr(), n, iters, wgs_per_cu, clocks.data_ptr(),
+                                     clocks.numel(), sink.data_ptr(), ctypes.addressof(nw), st), 5, warm=3, warm_seconds=0.1)
+    ops_total = waves * iters * 8 * 65536.0
+    return ops_total / sec / 1e12, _clock_ghz(clocks, waves)
 
 
 def gemm_clock(device, backward, a, w, shape):

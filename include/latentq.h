@@ -219,6 +219,15 @@ int lq_a8w8_fwd_qs(const void *x, const void *w, const float *sx, const void *qs
                    const void *bias_or_null, void *y, int32_t *acc_or_null, int64_t M, int64_t N,
                    int64_t K, void *stream);
 
+/* Input gradient of an 8-bit-weight layer from its int8 codes: dX[M,K] = dY[M,N] . Wf[N,K] with
+ * Wf[n,k] = bf16(w[n,k] * qscales[n]), the dequantised weight the reference's backward materialises
+ * (`weight_d.to(dtype) * qscales`, utils/quant.py:200-206, 239-245, 281-288) and multiplies with
+ * `grad_output.mm(weight_forward)`; here it is formed tile by tile inside the GEMM and never stored.
+ * dy: bf16 [M,N]; w: int8 [N,K]; qscales_bf16: bf16 [N]; dx: bf16 [M,K]; N % 64 == 0, K % 128 == 0; dy, w, dx
+ * 16-byte aligned. fp32 accumulation, one bf16 rounding of the result. */
+int lq_a8w8_dx(const void *dy, const void *w, const void *qscales_bf16, void *dx, int64_t M, int64_t N, int64_t K,
+               void *stream);
+
 /* Per-tensor symmetric activation quantizer used in front of lq_a8w8_fwd:
  *   x8 = clamp(round_half_even(x * (127/clampv)), -128, 127)
  * (reference utils/quant.py:264-266). x: bf16[n]; clampv: DEVICE fp32 scalar;
@@ -424,6 +433,10 @@ int lq_calib_read(const void *src, int64_t nbytes, int workgroups, void *sink, v
  * ------------------------------------------------------------------------- */
 int lq_calib_mfma_loop(const void *a, const void *b, int64_t n_elems, int64_t iters, int workgroups_per_cu,
                        uint64_t *clocks, int64_t clocks_capacity, float *sink, int64_t *waves, void *stream);
+/* lq_calib_mfma_loop on the int8 matrix instruction of lq_a8w8_fwd (32x32x32, int32 accumulators): a and b are
+ * n_bytes of int8 each; work per wave: iters x 8 x 65536 operations; sink: int32[waves]. */
+int lq_calib_mfma_loop_i8(const void *a, const void *b, int64_t n_bytes, int64_t iters, int workgroups_per_cu,
+                          uint64_t *clocks, int64_t clocks_capacity, int32_t *sink, int64_t *waves, void *stream);
 int lq_calib_gemm_clocks(int backward, const void *a, const void *codes, const void *scales, const void *zeros,
                          void *out, int64_t M, int64_t N, int64_t K, int group, uint64_t *clocks,
                          int64_t clocks_capacity, int64_t *workgroups, void *stream);

@@ -28,6 +28,7 @@ SIGNATURES = {
     "lq_a16w4_plan": [_i32, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp],
     "lq_a16w4_dequant": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp],
     "lq_a8w8_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
+    "lq_a8w8_dx": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "lq_act_quant_i8": [_vp, _vp, _vp, _i64, _vp],
     "lq_act_quant_i8_dynamic": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp],
     "lq_act_quant_i8_per_token": [_vp, _vp, _vp, _i64, _i64, _vp],
@@ -48,6 +49,7 @@ SIGNATURES = {
     "lq_calib_copy": [_vp, _vp, _i64, _vp],
     "lq_calib_read": [_vp, _i64, _i32, _vp, _vp],
     "lq_calib_mfma_loop": [_vp, _vp, _i64, _i64, _i32, _vp, _i64, _vp, _vp, _vp],
+    "lq_calib_mfma_loop_i8": [_vp, _vp, _i64, _i64, _i32, _vp, _i64, _vp, _vp, _vp],
     "lq_calib_gemm_clocks": [_i32, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp, _vp],
     "lq_transpose_bf16": [_vp, _vp, _i64, _i64, _vp],
     "lq_latent_w4_reconstruct": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],

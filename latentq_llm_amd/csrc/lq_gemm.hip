@@ -3,6 +3,7 @@
 //   MODE_W4_FWD : Y[M,N]  = X[M,K]  . deq(W)[N,K]^T     (bf16 MFMA, int4 W dequantised into LDS)
 //   MODE_W4_DX  : dX[M,K] = dY[M,N] . deq(W)[N,K]       (same, W tile transposed on the way out of LDS)
 //   MODE_I8     : acc     = X8[M,K] . W8[N,K]^T         (int8 MFMA, int32 accumulate, scaled epilogue)
+//   MODE_W8_DX  : dX[M,K] = dY[M,N] . (W8 * qs)[N,K]    (MODE_W4_DX with int8 codes and one bf16 scale per row n)
 //
 // (The forward pass of large grids runs the weights-direct kernel of lq_gemm_fwd.hip instead.)
 //
@@ -46,7 +47,7 @@
 
 namespace {
 
-enum { MODE_W4_FWD = 0, MODE_W4_DX = 1, MODE_I8 = 2 };
+enum { MODE_W4_FWD = 0, MODE_W4_DX = 1, MODE_I8 = 2, MODE_W8_DX = 3 };
 
 struct GemmParams {
     const void *a;        // activations: bf16 [M, R] or int8 [M, R]
@@ -112,6 +113,7 @@ __device__ __forceinline__ int dx_slot(int row, int c32, int half) {
 
 template <int MODE, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
+    constexpr bool kDx = MODE == MODE_W4_DX || MODE == MODE_W8_DX;  // reduction over n, weight tile kept in [n][k] order
     constexpr int NT = 64 * WM * WN;           // threads per role
     constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
     constexpr int FM = TM / 32, FN = TN / 32;  // 32x32 fragments per wave tile
@@ -188,9 +190,9 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
         constexpr int BPT = (MODE == MODE_I8) ? BN * 8 / NT : 1;
         constexpr int NW = (MODE == MODE_W4_FWD) ? BN * 8 / NT : 1;  // tile has BN rows x 8 words
         static_assert(MODE != MODE_W4_FWD || NW == 2 || NW == 4 || NW == 8, "bad fwd staging split");
-        static_assert(MODE != MODE_W4_DX || (BN == 128 && NT == 256), "dX staging: 64 rows x 4 threads");
+        static_assert(!kDx || (BN == 128 && NT == 256), "dX staging: 64 rows x 4 threads");
         constexpr int NSZ = 1;
-        constexpr int NWORDS = (MODE == MODE_W4_DX) ? 4 : NW;
+        constexpr int NWORDS = (MODE == MODE_W4_DX) ? 4 : (MODE == MODE_W8_DX) ? 8 : NW;
 
         const unsigned char *b_src[MODE == MODE_I8 ? BPT : 1];
         int b_dst[MODE == MODE_I8 ? BPT : 1];
@@ -217,6 +219,12 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             b_src[0] = (const unsigned char *)p.b + (long long)gr * (p.Kw / 2) + b_w0 * 4 + (long long)k0 * 32;
             s_src[0] = p.scales + (long long)gr * groups_per_row + k0 / 2;  // k0 is even: a group is two steps
             z_src[0] = p.zeros + (long long)gr * groups_per_row + k0 / 2;
+        } else if constexpr (MODE == MODE_W8_DX) {
+            b_row = tid >> 2;  // n within the tile
+            b_w0 = tid & 3;    // 32 of the tile's 128 output columns k = 32 code bytes
+            b_src[0] = (const unsigned char *)p.b + ((long long)k0 * 64 + b_row) * p.Kw + c0 + b_w0 * 32;
+            s_src[0] = p.scales + ((long long)k0 * 64 + b_row);  // one scale per weight row n
+            z_src[0] = nullptr;
         } else {
             b_row = tid >> 2;  // n within the tile (the tile offset along n is added per tile)
             b_w0 = tid & 3;    // 32 of the tile's 128 output columns k
@@ -253,6 +261,13 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
                 }
                 S.s[0] = s_src[0][kt >> 1];
                 S.z[0] = z_src[0][kt >> 1];
+            } else if constexpr (MODE == MODE_W8_DX) {
+                const long long row_off = (long long)kt * 64;
+                const u32x4_t v0 = *reinterpret_cast<const u32x4_t *>(b_src[0] + row_off * p.Kw);
+                const u32x4_t v1 = *reinterpret_cast<const u32x4_t *>(b_src[0] + row_off * p.Kw + 16);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { S.w[i] = v0[i]; S.w[4 + i] = v1[i]; }
+                S.s[0] = s_src[0][row_off];
             } else {
                 const long long row_off = (long long)kt * 64;
                 u32x4_t v = *reinterpret_cast<const u32x4_t *>(b_src[0] + row_off * (p.Kw / 2));
@@ -279,6 +294,21 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
                     u32x4_t v = {lq_pack_bf16(f[0], f[1]), lq_pack_bf16(f[2], f[3]), lq_pack_bf16(f[4], f[5]),
                                  lq_pack_bf16(f[6], f[7])};
                     *reinterpret_cast<u32x4_t *>(lb + b_row * ROWB + ((ch ^ swz(b_row)) << 4)) = v;
+                }
+            } else if constexpr (MODE == MODE_W8_DX) {
+                // bf16(w8 * qs), the weight the reference's backward multiplies with (utils/quant.py:200-201): the
+                // byte + 128 converts with one instruction, and fma(u, s, -128 s) is the exact product (16 bits)
+                const float s = lq_bf16_bits_to_f32(S.s[0]);
+                const float off = -128.0f * s;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const unsigned a = S.w[2 * w] ^ 0x80808080u, b = S.w[2 * w + 1] ^ 0x80808080u;
+                    u32x4_t v = {lq_pack_bf16(fmaf((float)((a >> 0) & 0xFFu), s, off), fmaf((float)((a >> 8) & 0xFFu), s, off)),
+                                 lq_pack_bf16(fmaf((float)((a >> 16) & 0xFFu), s, off), fmaf((float)((a >> 24) & 0xFFu), s, off)),
+                                 lq_pack_bf16(fmaf((float)((b >> 0) & 0xFFu), s, off), fmaf((float)((b >> 8) & 0xFFu), s, off)),
+                                 lq_pack_bf16(fmaf((float)((b >> 16) & 0xFFu), s, off), fmaf((float)((b >> 24) & 0xFFu), s, off))};
+                    const int c32 = b_w0 * 2 + (w >> 1);  // 32-byte piece of the 256-byte row
+                    *reinterpret_cast<u32x4_t *>(lb + b_row * 256 + dx_slot(b_row, c32, w & 1)) = v;
                 }
             } else {
                 const float s = lq_bf16_bits_to_f32(S.s[0]);
@@ -382,7 +412,7 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
     // wave are (k0, n0) = (0, 0), (16, 0), (0, 8), (16, 8); a second read 4 rows further down
     // completes the 8 n of the operand.
     int dx_off[FN];
-    if constexpr (MODE == MODE_W4_DX) {
+    if constexpr (kDx) {
         const int i16 = lane & 15, blk = lane >> 4;
         const int row_lane = 8 * (blk >> 1) + (i16 >> 2), colblk = blk & 1;  // row_lane & 3 is the row's j
 #pragma unroll
@@ -396,7 +426,7 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
 #pragma unroll
         for (int i = 0; i < FM; ++i)
             af[i] = *reinterpret_cast<const u32x4_t *>(la + a_frag[ks] + i * 32 * AROW);
-        if constexpr (MODE == MODE_W4_DX) {
+        if constexpr (kDx) {
 #pragma unroll
             for (int i = 0; i < FN; ++i) {
                 const v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)(lb + dx_off[i] + ks * 4096));
@@ -566,14 +596,14 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             const int mm = m0 + wm * TM + j * 32 + row;
             if (mm < p.M && c_lane < p.C) {
                 const long long off = (long long)mm * p.C + c_lane;
-                if (MODE == MODE_W4_DX && p.ep_mode == EP_ADD) {
+                if (kDx && p.ep_mode == EP_ADD) {
                     const u32x4_t old = *reinterpret_cast<const u32x4_t *>(out + off);
                     u32x4_t sum;
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         sum[e] = lq_pack_bf16(lq_bf16_lo(old[e]) + lq_bf16_lo(o[e]), lq_bf16_hi(old[e]) + lq_bf16_hi(o[e]));
                     *reinterpret_cast<u32x4_t *>(out + off) = sum;
-                } else if (MODE == MODE_W4_DX && p.ep_mode == EP_SILU_BW) {
+                } else if (kDx && p.ep_mode == EP_SILU_BW) {
                     const u32x4_t g8 = *reinterpret_cast<const u32x4_t *>(p.ep_g + off);
                     const u32x4_t u8 = *reinterpret_cast<const u32x4_t *>(p.ep_u + off);
                     u32x4_t dg, du;
@@ -1062,6 +1092,24 @@ extern "C" int lq_a16w4_dx_ws(const void *dy, const void *codes, const void *sca
                               void *stream) {
     return a16w4_dx_impl("lq_a16w4_dx_ws", dy, codes, scales, zeros, dx, M, N, K, group, workspace,
                          workspace && workspace_bytes > 0 ? (size_t)workspace_bytes : 0, stream);
+}
+
+// dX of an 8-bit-weight layer straight from the int8 codes: the staged dX kernel with the weight waves forming
+// bf16(w8 * qs[n]) instead of dequantising int4 groups.
+extern "C" int lq_a8w8_dx(const void *dy, const void *w, const void *qscales_bf16, void *dx, int64_t M, int64_t N, int64_t K,
+                          void *stream) {
+    LQ_REQUIRE(dy && w && qscales_bf16 && dx, "lq_a8w8_dx: null pointer argument");
+    LQ_REQUIRE(M > 0 && N > 0 && K > 0 && M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && N * K < (1ll << 40),
+               "lq_a8w8_dx: M, N, K must be positive (M=%lld N=%lld K=%lld)", (long long)M, (long long)N, (long long)K);
+    LQ_REQUIRE(N % 64 == 0 && K % 128 == 0, "lq_a8w8_dx: N=%lld must be a multiple of 64 and K=%lld of 128", (long long)N, (long long)K);
+    LQ_REQUIRE(lq_aligned(dy, 16) && lq_aligned(w, 16) && lq_aligned(dx, 16) && lq_aligned(qscales_bf16, 2),
+               "lq_a8w8_dx: dy, w and dx must be 16-byte aligned");
+    GemmParams p = {};
+    p.a = dy; p.b = w; p.scales = (const unsigned short *)qscales_bf16; p.c = dx;
+    p.M = (int)M; p.C = (int)K; p.R = (int)N; p.Kw = (int)K;
+    const W4Plan plan = plan_dx(M, N, K, 0, lq_device_cu_count());
+    return plan.kernel == LQ_PLAN_STAGED_256 ? launch_gemm<MODE_W8_DX, 256, 128, 2, 2>(p, (hipStream_t)stream, "lq_a8w8_dx")
+                                             : launch_gemm<MODE_W8_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, "lq_a8w8_dx");
 }
 
 static int a8w8_fwd_impl(const void *x, const void *w, const float *sx, const void *sw, bool sw_bf16, const void *bias_or_null,

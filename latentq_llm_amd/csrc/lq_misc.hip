@@ -221,6 +221,61 @@ __global__ __launch_bounds__(256, 2) void mfma_loop_kernel(const u32x4_t *__rest
     }
 }
 
+// The same loop on the int8 matrix instruction of the A8W8 kernels (32x32x32, int32 accumulators).
+__global__ __launch_bounds__(256, 2) void mfma_loop_i8_kernel(const u32x4_t *__restrict__ a, const u32x4_t *__restrict__ b,
+                                                              long long n16, long long iters, unsigned long long *__restrict__ clk,
+                                                              int *__restrict__ sink) {
+    const int lane = threadIdx.x & 63;
+    const long long wv = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    u32x4_t af[4], bf[2];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) af[j] = a[((wv * 4 + j) * 64 + lane) % n16];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) bf[i] = b[((wv * 2 + i) * 64 + lane) % n16];
+    i32x16_t acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0;
+    const unsigned long long t0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+    for (long long it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf[i]), __builtin_bit_cast(i32x4_t, af[j]),
+                                                                 acc[i][j], 0, 0, 0);
+    }
+    const unsigned long long t1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) s += acc[i][j][q];
+    if (lane == 0) {
+        clk[4 * wv] = t0; clk[4 * wv + 1] = t1; clk[4 * wv + 2] = r0; clk[4 * wv + 3] = r1;
+        sink[wv] = s;
+    }
+}
+
+extern "C" int lq_calib_mfma_loop_i8(const void *a, const void *b, int64_t n_bytes, int64_t iters, int workgroups_per_cu,
+                                     uint64_t *clocks, int64_t clocks_capacity, int32_t *sink, int64_t *waves, void *stream) {
+    LQ_REQUIRE(a && b && clocks && sink && waves, "lq_calib_mfma_loop_i8: null pointer argument");
+    LQ_REQUIRE(n_bytes >= 8192 && n_bytes % 16 == 0 && lq_aligned(a, 16) && lq_aligned(b, 16) && lq_aligned(clocks, 8),
+               "lq_calib_mfma_loop_i8: operands need at least 8192 bytes, a multiple of 16, 16-byte aligned");
+    LQ_REQUIRE(iters > 0 && (workgroups_per_cu == 1 || workgroups_per_cu == 2), "lq_calib_mfma_loop_i8: iters > 0, 1 or 2 workgroups per unit");
+    const long long wgs = (long long)lq_device_cu_count() * workgroups_per_cu;
+    LQ_REQUIRE(16 * wgs <= clocks_capacity, "lq_calib_mfma_loop_i8: clocks must hold %lld values", 16 * wgs);
+    *waves = 4 * wgs;
+    hipLaunchKernelGGL(mfma_loop_i8_kernel, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream, (const u32x4_t *)a,
+                       (const u32x4_t *)b, (long long)(n_bytes / 16), (long long)iters, (unsigned long long *)clocks, sink);
+    return lq_check_launch("lq_calib_mfma_loop_i8");
+}
+
 extern "C" int lq_calib_mfma_loop(const void *a, const void *b, int64_t n_elems, int64_t iters, int workgroups_per_cu,
                                   uint64_t *clocks, int64_t clocks_capacity, float *sink, int64_t *waves, void *stream) {
     LQ_REQUIRE(a && b && clocks && sink && waves, "lq_calib_mfma_loop: null pointer argument");

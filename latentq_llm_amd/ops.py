@@ -317,6 +317,27 @@ def a8w8_forward(x8, w8, sx, sw, bias=None, want_acc: bool = False):
     return (y, acc) if want_acc else y
 
 
+def a8w8_dx_ok(dy, w8, qscales):
+    """Whether a8w8_dx takes these operands (the layers fall back to the dense product otherwise)."""
+    return (dy.is_cuda and dy.dtype == torch.bfloat16 and dy.dim() == 2 and dy.is_contiguous() and w8.is_cuda
+            and w8.dtype == torch.int8 and w8.dim() == 2 and w8.is_contiguous() and qscales.is_cuda
+            and qscales.dtype == torch.bfloat16 and qscales.is_contiguous() and qscales.numel() == w8.shape[0]
+            and dy.shape[1] == w8.shape[0] and w8.shape[0] % 64 == 0 and w8.shape[1] % 128 == 0 and dy.shape[0] > 0
+            and dy.data_ptr() % 16 == 0 and w8.data_ptr() % 16 == 0)
+
+
+def a8w8_dx(dy, w8, qscales):
+    """dX[M,K] = dY[M,N] . bf16(W8 * qscales)[N,K] from the int8 codes (lq_a8w8_dx)."""
+    if not a8w8_dx_ok(dy, w8, qscales):
+        raise ValueError("a8w8_dx needs contiguous GPU operands: dy bf16 [M,N], w8 int8 [N,K], qscales bf16 [N], N % 64 == 0, K % 128 == 0")
+    M, N = dy.shape
+    K = w8.shape[1]
+    dx = torch.empty((M, K), dtype=torch.bfloat16, device=dy.device)
+    with torch.cuda.device(dy.device):
+        _C.call("lq_a8w8_dx", dy.data_ptr(), w8.data_ptr(), qscales.data_ptr(), dx.data_ptr(), M, N, K, _stream(dy))
+    return dx
+
+
 def act_quant_i8(x, clampv):
     """int8 activations clamp(rne(x*127/clampv)); clampv is a 1-element fp32 GPU tensor (no host sync)."""
     _chk(x, torch.bfloat16, "x")

@@ -43,6 +43,9 @@ FUSED_ADAM8 = True
 # The 8-bit gradient accumulator (row scales + stochastic rounding to int8, and the accumulate form) as
 # one HIP pass per micro-batch; False runs the reference's tensor operations with torch's uniform_ noise.
 FUSED_GRADQ = True
+# The input gradient of an 8-bit-weight layer from its int8 codes (the dequantised weight formed inside the GEMM);
+# False materialises W8 * qscales and multiplies densely, as the reference does.
+FUSED_A8W8_DX = True
 EXT_type = torch.bfloat16  # utils/quant.py:722
 
 # dW travels from the autograd Functions to the full-backward hook through this list
@@ -309,10 +312,23 @@ def _fake_quant_activation(input, clampv):
     return (input * s).round_().clamp_(-128, 127).div_(s)
 
 
-def _a8w8_backward_common(ctx, grad_output, input_f, weight_f, bias, detach_dw):
+def _a8w8_backward_common(ctx, grad_output, input_f, weight_f, bias, detach_dw=False):
+    """grad_input = dY . Wf and dW = dY^T . Xf on the dequantised operands (utils/quant.py:203-210). weight_f is the
+    dense weight, or an (int8 codes, qscales) pair: then dX comes from the codes (ops.a8w8_dx: bf16(W8 * qs) is formed
+    inside the GEMM, the values the reference's `weight_d.to(dtype) * qscales` holds) whenever the kernel takes the
+    shapes. detach_dw is kept for the call sites' symmetry with the reference (the product has no history here)."""
     grad_input = grad_bias = None
     if ctx.needs_input_grad[0]:
-        grad_input = grad_output.mm(weight_f)
+        if isinstance(weight_f, tuple):
+            w8, qscales = weight_f
+            dy = grad_output if grad_output.is_contiguous() else grad_output.contiguous()
+            qs = qscales.detach().reshape(-1)
+            if FUSED_A8W8_DX and ops.a8w8_dx_ok(dy, w8, qs):
+                grad_input = ops.a8w8_dx(dy, w8, qs)
+            else:
+                grad_input = grad_output.mm((w8.to(grad_output.dtype) * qscales).to(grad_output.dtype))
+        else:
+            grad_input = grad_output.mm(weight_f)
     dict_temp.append(_pending_dw(grad_output, input_f))
     if bias is not None and ctx.needs_input_grad[_BIAS_FLAG]:
         grad_bias = grad_output.sum(0)
@@ -338,8 +354,7 @@ class QLinearFunctionA8W8_static(torch.autograd.Function):
         input, weight_d, bias = ctx.saved_tensors
         clampv, qscales = ctx.save_qparamaw
         input_f = _fake_quant_activation(input, clampv)
-        weight_f = weight_d.to(input.dtype) * qscales
-        return _a8w8_backward_common(ctx, grad_output, input_f, weight_f, bias, detach_dw=False)
+        return _a8w8_backward_common(ctx, grad_output, input_f, (weight_d, qscales), bias, detach_dw=False)
 
 
 class QLinearFunctionA8W8_dynamic0(torch.autograd.Function):
@@ -358,8 +373,7 @@ class QLinearFunctionA8W8_dynamic0(torch.autograd.Function):
         input, weight_d, bias = ctx.saved_tensors
         work, qscales = ctx.save_qparamaw
         input_f = _fake_quant_activation(input, work[0].to(input.dtype))  # clampv = input.max(), a 0-dim tensor
-        weight_f = weight_d.to(input.dtype) * qscales
-        return _a8w8_backward_common(ctx, grad_output, input_f, weight_f, bias, detach_dw=True)
+        return _a8w8_backward_common(ctx, grad_output, input_f, (weight_d, qscales), bias, detach_dw=True)
 
 
 class QLinearFunctionA8W8_dynamic(torch.autograd.Function):
@@ -382,8 +396,7 @@ class QLinearFunctionA8W8_dynamic(torch.autograd.Function):
         # x8 * (clampv / 127.): the quantiser left that bf16-valued alpha in scale[1]; per token: the row scales
         s = scale.view(-1, 1) if per_token else scale[1]
         input_f = x8.to(grad_output.dtype) * s.to(grad_output.dtype)
-        weight_f = (weight_d.to(grad_output.dtype) * qscales).to(grad_output.dtype)
-        return _a8w8_backward_common(ctx, grad_output, input_f, weight_f, bias, detach_dw=True)
+        return _a8w8_backward_common(ctx, grad_output, input_f, (weight_d, qscales), bias, detach_dw=True)
 
 
 class QLinearFunctionA8W8_static_eval(torch.autograd.Function):

@@ -456,6 +456,33 @@ def test_a8w8_per_token_forward_matches_float64(ops):
     assert torch.equal(y, y32)  # bf16 scales widened in the epilogue = the fp32 copy of them
 
 
+@pytest.mark.parametrize("M,N,K", [(2048, 2048, 2048), (300, 64, 128), (2048, 8192, 2048), (100, 2048, 8192), (520, 192, 384)])
+def test_a8w8_dx_from_int8_codes(ops, M, N, K):
+    """dX = dY . bf16(W8 * qs): the weight tile is formed inside the GEMM. Against the float64 product with that
+    bf16 weight (rel-L2, printed), and exactly for integer-valued operands with power-of-two scales."""
+    g = torch.Generator().manual_seed(N + K)
+    w8 = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+    qs = ((torch.randn(N, generator=g) * 0.01).abs() + 1e-3).to(torch.bfloat16)
+    dy = randn_bf16((M, N), 3)
+    dx = ops.a8w8_dx(dev(dy), dev(w8), dev(qs)).cpu()
+    wf = (w8.to(torch.bfloat16) * qs[:, None]).to(torch.bfloat16)  # what the reference's backward materialises
+    want = dy.double() @ wf.double()
+    err = rel_l2(dx, want)
+    print(f"a8w8_dx {M}x{N}x{K}: rel_l2={err:.3e} max_abs={float((dx.double() - want).abs().max()):.3e}")
+    assert err < 4e-3
+    # exact case: a few rows of dY one-hot with power-of-two values, scales powers of two: dX rows are scaled weight rows
+    dy1 = torch.zeros((M, N), dtype=torch.bfloat16)
+    rows = [0, M // 2, M - 1]
+    cols = [0, N // 3, N - 1]
+    for r_, c_ in zip(rows, cols):
+        dy1[r_, c_] = 2.0
+    qs2 = torch.tensor([2.0 ** ((i % 5) - 7) for i in range(N)], dtype=torch.bfloat16)
+    dx1 = ops.a8w8_dx(dev(dy1), dev(w8), dev(qs2)).cpu()
+    for r_, c_ in zip(rows, cols):
+        assert torch.equal(dx1[r_].float(), 2.0 * w8[c_].float() * qs2[c_].float())
+    assert not dx1[1].any()
+
+
 # ------------------------------------------------------------------ repack --
 @pytest.mark.parametrize("N,K", [(16, 128), (100, 384), (4096, 1024)])
 def test_repack_round_trip(ops, co, N, K):

@@ -180,6 +180,30 @@ def test_qlinear_a8w8_per_token(Q):
     assert rel_l2(m.weight.grad.float().cpu(), dy.double().t() @ xq) < 1e-2
 
 
+def test_qlinear_a8w8_backward_from_codes_equals_dense_path(Q):
+    """The A8W8 training Function's input gradient comes from the int8 codes (lq_a8w8_dx); with the switch off the
+    dequantised weight is materialised and multiplied densely, as the reference does: same result within the fp32
+    accumulation order."""
+    N, K, M = 256, 384, 200
+    m, w8, qs = _a8w8_layer(Q, N, K, 31, bias=False)
+    m.weight.requires_grad = True
+    m.add_hook()
+    x_cpu, dy = randn_bf16((M, K), 3), randn_bf16((M, N), 4).cuda()
+    grads = []
+    for fused in (True, False):
+        Q.FUSED_A8W8_DX = fused
+        try:
+            x = x_cpu.cuda().requires_grad_(True)
+            m.weight.grad = None
+            m(x).backward(dy)
+            grads.append(x.grad.clone())
+        finally:
+            Q.FUSED_A8W8_DX = True
+    assert rel_l2(grads[0].float(), grads[1].float()) < 3e-3
+    wf = (w8.to(torch.bfloat16) * qs).to(torch.bfloat16).double()
+    assert rel_l2(grads[0].cpu(), dy.cpu().double() @ wf) < 4e-3
+
+
 def test_qlinear_qat_forward(Q):
     N, K, M = 64, 128, 33
     m = Q.QLinearQAT(K, N, bias=False, lbit=16, gbit=16)
