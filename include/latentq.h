@@ -262,7 +262,7 @@ int lq_act_quant_i8_per_token(const void *x, int8_t *x8, float *sx, int64_t M, i
  * from MyAdam.update_step (:1141):
  *   codes[n,k] = clamp(round_half_even(bf16(latent[n,k] / qscales[n])), -128, 127)      NaN -> 0
  * latent: bf16[N,K], 16-byte aligned; qscales: bf16[N]; codes: int8[N,K], 8-byte aligned; K % 8 == 0.
- * (With a 4-bit residual codec, lbit = 4, the layer keeps the reference's chain of tensor operations.) */
+ * (With a 4-bit residual codec, lbit = 4: lq_latent_w8_requant.) */
 int lq_w8_requant(const void *latent, const void *qscales, int8_t *codes, int64_t N, int64_t K, void *stream);
 
 /* ---------------------------------------------------------------------------
@@ -314,6 +314,20 @@ int lq_latent_w4_reconstruct(const void *codes, const void *scales, const void *
 int lq_latent_w4_requant(const void *latent, const void *scales, const void *zeros, void *codes_out,
                          int32_t *residual_out, int64_t N, int64_t K, int group, int k1, float b1, int k2, float b2,
                          int k3, void *stream);
+
+/* The same two passes for an 8-bit-weight layer whose latent is codes + 4-bit residual (QuantTensor(wbit = 8,
+ * lbit = 4)): one bf16 scale per weight row instead of scale and zero per group.
+ *   lq_latent_w8_reconstruct: latent = bf16(bf16(value(nibble) * s[n]) + bf16(q * s[n]))
+ *     replaces ResidualTensor.add((p.data * p.qparam).to(dtype)), utils/quant.py:826-837, 1069-1070.
+ *   lq_latent_w8_requant: Z = bf16(t / s[n]), q = rint(Z), residual nibble and carry from bf16(Z - q),
+ *     code = clamp(q + carry, -128, 127); replaces Qfunc_8bit_res with a ResidualTensor, utils/quant.py:88-103
+ *     (+ ResidualTensor.set_value :803-811). NaN -> code 0.
+ * codes: int8 [N,K]; qscales: bf16 [N]; residual: int32 [N*K/8]; latent: bf16 [N,K]; K % 16 == 0; codes and latent
+ * 16-byte, residual 8-byte aligned. */
+int lq_latent_w8_reconstruct(const int8_t *codes, const void *qscales, const int32_t *residual, void *latent_out,
+                             int64_t N, int64_t K, int k1, float b1, int k2, float b2, int k3, void *stream);
+int lq_latent_w8_requant(const void *latent, const void *qscales, int8_t *codes_out, int32_t *residual_out, int64_t N,
+                         int64_t K, int k1, float b1, int k2, float b2, int k3, void *stream);
 
 /* ---------------------------------------------------------------------------
  * One Adam step on 8-bit block-wise moments, the chain of tensor operations of

@@ -54,6 +54,8 @@ SIGNATURES = {
     "lq_transpose_bf16": [_vp, _vp, _i64, _i64, _vp],
     "lq_latent_w4_reconstruct": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],
     "lq_latent_w4_requant": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],
+    "lq_latent_w8_reconstruct": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _f32, _i32, _f32, _i32, _vp],
+    "lq_latent_w8_requant": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _f32, _i32, _f32, _i32, _vp],
     "lq_adam8_update": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _f64, _f64, _f64, _f64, _vp],
     "lq_adam8_latent_w4_step": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32,
                                 _i32, _f32, _i32, _f32, _i32, _i32, _f32, _i32, _f32, _i32, _f64, _f64, _f64, _f64, _vp],

@@ -13,6 +13,12 @@
 //   reconstruct:  w = bf16(bf16(q - z) * s);  r = bf16(bf16(value(nibble)) * s);  latent = bf16(r + w)
 //   requant:      Z = bf16(bf16(t / s) + z);  q = rint(Z);  f = bf16(Z - q)
 //                 (nibble, carry) = codec(f);  code = clamp(bf16(q + carry), 0, 15)
+//
+// The 8-bit-weight layer keeps its latent the same way (int8 codes, one bf16 scale per row, the same residual words):
+//   reconstruct:  w = bf16(q * s);  r = bf16(bf16(value(nibble)) * s);  latent = bf16(r + w)
+//                 (ResidualTensor.add((p.data * p.qparam).to(dtype)), utils/quant.py:826-837, 1069-1070)
+//   requant:      Z = bf16(t / s);  q = rint(Z);  f = bf16(Z - q);  (nibble, carry) = codec(f)
+//                 code = clamp(q + carry, -128, 127)                  (Qfunc_8bit_res, utils/quant.py:88-103)
 #include "lq_latent_math.h"
 
 namespace {
@@ -87,6 +93,95 @@ __global__ __launch_bounds__(256) void latent_requant_kernel(const u32x4_t *__re
     residual[L] = rout;
 }
 
+// ---- 8-bit weights: a thread owns 16 consecutive elements of one row (16 code bytes, two residual words) ----
+__global__ __launch_bounds__(256) void latent_w8_reconstruct_kernel(const u32x4_t *__restrict__ codes,
+                                                                    const unsigned short *__restrict__ qscales,
+                                                                    const u32x2_t *__restrict__ residual,
+                                                                    u32x4_t *__restrict__ latent, long long n_chunks,
+                                                                    long long chunks_per_row, CodecParams p) {
+    __shared__ float vtab[16];
+    lq_latent_fill_value_table(vtab, p);
+    __syncthreads();
+    const long long L = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (L >= n_chunks) return;
+    const u32x4_t cw = codes[L];
+    const u32x2_t rw = residual[L];
+    const float s = lq_bf16_bits_to_f32(qscales[L / chunks_per_row]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        float v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int e = 8 * i + k;
+            const float q = (float)(int)(signed char)((cw[e >> 2] >> (8 * (e & 3))) & 0xFFu);
+            const float w = lq_bf16r(q * s);
+            const float r = lq_bf16r(vtab[(rw[i] >> (28 - 4 * k)) & 0xFu] * s);
+            v[k] = r + w;
+        }
+        latent[L * 2 + i] = u32x4_t{lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3]), lq_pack_bf16(v[4], v[5]),
+                                    lq_pack_bf16(v[6], v[7])};
+    }
+}
+
+template <bool kFast>
+__device__ __forceinline__ void requant_w8_thread(const u32x4_t (&in)[2], float s, float r, const CodecParams p, u32x4_t &cout,
+                                                  u32x2_t &rout) {
+    unsigned cw[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        unsigned rword = 0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float t = (k & 1) ? lq_bf16_hi(in[i][k >> 1]) : lq_bf16_lo(in[i][k >> 1]);
+            const float quo = kFast ? t * r : t / s;
+            const float Z = lq_bf16r(quo);
+            const float q = rintf(Z);       // round half to even, as torch.round
+            const float f = lq_bf16r(Z - q);
+            bool carry;
+            const unsigned nib = nibble_of(level_3fold(f, p), carry);
+            // q + carry is an integer (bf16 holds it exactly wherever the clamp does not decide); NaN -> 0
+            const float c = q + (carry ? 1.0f : 0.0f);
+            const float cc = c == c ? __builtin_amdgcn_fmed3f(c, -128.0f, 127.0f) : 0.0f;
+            rword = (rword << 4) | nib;
+            const int e = 8 * i + k;
+            cw[e >> 2] |= ((unsigned)(int)cc & 0xFFu) << (8 * (e & 3));
+        }
+        rout[i] = rword;
+    }
+    cout = u32x4_t{cw[0], cw[1], cw[2], cw[3]};
+}
+
+__global__ __launch_bounds__(256) void latent_w8_requant_kernel(const u32x4_t *__restrict__ latent,
+                                                                const unsigned short *__restrict__ qscales,
+                                                                u32x4_t *__restrict__ codes, u32x2_t *__restrict__ residual,
+                                                                long long n_chunks, long long chunks_per_row, CodecParams p) {
+    const long long L = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (L >= n_chunks) return;
+    u32x4_t in[2];
+    in[0] = latent[L * 2];
+    in[1] = latent[L * 2 + 1];
+    const float s = lq_bf16_bits_to_f32(qscales[L / chunks_per_row]);
+    // the quotient of two bf16 numbers as a product with the reciprocal: see lq_latent_requant_elem
+    const bool fast = (fabsf(s) >= 0x1p-40f) && (fabsf(s) <= 0x1p40f);
+    const float r = 1.0f / s;
+    u32x4_t cout;
+    u32x2_t rout;
+    if (fast) requant_w8_thread<true>(in, s, r, p, cout, rout);
+    else requant_w8_thread<false>(in, s, r, p, cout, rout);
+    codes[L] = cout;
+    residual[L] = rout;
+}
+
+int check_latent_w8(const char *who, const void *a, const void *b, const void *c, const void *d, int64_t N, int64_t K, int k1,
+                    float b1, int k2, float b2, int k3) {
+    LQ_REQUIRE(a && b && c && d, "%s: null pointer argument", who);
+    LQ_REQUIRE(N > 0 && K > 0 && K % 16 == 0, "%s: need N > 0, K a positive multiple of 16", who);
+    LQ_REQUIRE(N * K / 16 <= 0x7FFFFFFFll * 256, "%s: tensor too large", who);
+    LQ_REQUIRE(k1 > 0 && k2 > 0 && k3 > 0 && b1 > 0.0f && b2 > b1 && b2 < 0.5f, "%s: need k1,k2,k3 > 0 and 0 < b1 < b2 < 0.5",
+               who);
+    return LQ_OK;
+}
+
 int check_latent(const char *who, const void *a, const void *b, const void *c, const void *d, const void *e, int64_t N,
                  int64_t K, int group, int k1, float b1, int k2, float b2, int k3) {
     LQ_REQUIRE(a && b && c && d && e, "%s: null pointer argument", who);
@@ -129,4 +224,30 @@ extern "C" int lq_latent_w4_requant(const void *latent, const void *scales, cons
                        (const u32x4_t *)latent, (const unsigned short *)scales, (const unsigned short *)zeros,
                        (u32x4_t *)codes_out, (u32x4_t *)residual_out, n_chunks, lq_codec_quant_params(k1, b1, k2, b2, k3));
     return lq_check_launch("lq_latent_w4_requant");
+}
+
+extern "C" int lq_latent_w8_reconstruct(const int8_t *codes, const void *qscales, const int32_t *residual, void *latent_out,
+                                        int64_t N, int64_t K, int k1, float b1, int k2, float b2, int k3, void *stream) {
+    int rc = check_latent_w8("lq_latent_w8_reconstruct", codes, qscales, residual, latent_out, N, K, k1, b1, k2, b2, k3);
+    if (rc) return rc;
+    LQ_REQUIRE(lq_aligned(codes, 16) && lq_aligned(residual, 8) && lq_aligned(latent_out, 16),
+               "lq_latent_w8_reconstruct: codes and latent must be 16-byte, residual 8-byte aligned");
+    const long long n_chunks = (long long)N * K / 16;
+    hipLaunchKernelGGL(latent_w8_reconstruct_kernel, dim3((unsigned)((n_chunks + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const u32x4_t *)codes, (const unsigned short *)qscales, (const u32x2_t *)residual, (u32x4_t *)latent_out,
+                       n_chunks, (long long)(K / 16), lq_codec_dequant_params(k1, b1, k2, b2, k3));
+    return lq_check_launch("lq_latent_w8_reconstruct");
+}
+
+extern "C" int lq_latent_w8_requant(const void *latent, const void *qscales, int8_t *codes_out, int32_t *residual_out, int64_t N,
+                                    int64_t K, int k1, float b1, int k2, float b2, int k3, void *stream) {
+    int rc = check_latent_w8("lq_latent_w8_requant", latent, qscales, codes_out, residual_out, N, K, k1, b1, k2, b2, k3);
+    if (rc) return rc;
+    LQ_REQUIRE(lq_aligned(latent, 16) && lq_aligned(codes_out, 16) && lq_aligned(residual_out, 8),
+               "lq_latent_w8_requant: latent and codes must be 16-byte, residual 8-byte aligned");
+    const long long n_chunks = (long long)N * K / 16;
+    hipLaunchKernelGGL(latent_w8_requant_kernel, dim3((unsigned)((n_chunks + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const u32x4_t *)latent, (const unsigned short *)qscales, (u32x4_t *)codes_out, (u32x2_t *)residual_out,
+                       n_chunks, (long long)(K / 16), lq_codec_quant_params(k1, b1, k2, b2, k3));
+    return lq_check_launch("lq_latent_w8_requant");
 }

@@ -614,3 +614,34 @@ def latent_w4_requant(latent, scales, zeros, residual_int, shape, k1, b1, k2, b2
         _C.call("lq_latent_w4_requant", latent.data_ptr(), scales.data_ptr(), zeros.data_ptr(), codes.data_ptr(),
                 residual_int.data_ptr(), N, K, 128, int(k1), float(b1), int(k2), float(b2), int(k3), _stream(latent))
     return codes
+
+
+def latent_w8_reconstruct(codes, qscales, residual_int, k1, b1, k2, b2, k3):
+    """Latent weight of an 8-bit-weight layer with a 4-bit residual (lq_latent_w8_reconstruct): bf16 [N, K] from the
+    int8 codes [N, K], the bf16 row scales and the residual words."""
+    _chk(codes, torch.int8, "codes")
+    _chk(qscales, torch.bfloat16, "qscales")
+    _chk(residual_int, torch.int32, "residual_int")
+    if codes.dim() != 2 or qscales.numel() != codes.shape[0] or residual_int.numel() != codes.numel() // 8:
+        raise ValueError("codes must be [N, K], qscales hold N entries and residual_int N*K/8 words")
+    N, K = codes.shape
+    out = torch.empty((N, K), dtype=torch.bfloat16, device=codes.device)
+    with torch.cuda.device(codes.device):
+        _C.call("lq_latent_w8_reconstruct", codes.data_ptr(), qscales.data_ptr(), residual_int.data_ptr(), out.data_ptr(), N, K,
+                int(k1), float(b1), int(k2), float(b2), int(k3), _stream(codes))
+    return out
+
+
+def latent_w8_requant(latent, qscales, residual_int, k1, b1, k2, b2, k3):
+    """Re-quantise the bf16 latent of an 8-bit-weight layer: returns the int8 codes and overwrites residual_int."""
+    _chk(latent, torch.bfloat16, "latent")
+    _chk(qscales, torch.bfloat16, "qscales")
+    _chk(residual_int, torch.int32, "residual_int")
+    if latent.dim() != 2 or qscales.numel() != latent.shape[0] or residual_int.numel() != latent.numel() // 8:
+        raise ValueError("latent must be [N, K], qscales hold N entries and residual_int N*K/8 words")
+    N, K = latent.shape
+    codes = torch.empty((N, K), dtype=torch.int8, device=latent.device)
+    with torch.cuda.device(latent.device):
+        _C.call("lq_latent_w8_requant", latent.data_ptr(), qscales.data_ptr(), codes.data_ptr(), residual_int.data_ptr(), N, K,
+                int(k1), float(b1), int(k2), float(b2), int(k3), _stream(latent))
+    return codes

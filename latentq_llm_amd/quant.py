@@ -151,6 +151,18 @@ def Qfunc_8bit_res(tensor, residual_handle, qscales):
         if residual_handle is not None:
             residual_handle.data = tensor.to(residual_handle.dtype)
         return ops.w8_requant(tensor, qscales)
+    if (FUSED_LATENT and isinstance(residual_handle, ResidualTensor) and tensor.is_cuda and tensor.dim() == 2
+            and tensor.dtype == torch.bfloat16 and tensor.is_contiguous() and tensor.shape[1] % 16 == 0
+            and tensor.data_ptr() % 16 == 0 and torch.is_tensor(qscales) and qscales.dtype == torch.bfloat16
+            and qscales.is_contiguous() and qscales.dim() == 2 and tuple(qscales.shape) == (tensor.shape[0], 1)
+            and residual_handle.residual_int.is_cuda):
+        # the chain below with the residual codec inside, as one pass (lq_latent_w8_requant; same roundings)
+        p1, y1, p2, y2 = three_fold_curve_4bit(residual_handle.mu)
+        codes = ops.latent_w8_requant(tensor, qscales.view(-1), residual_handle.residual_int.view(-1), p1, y1, p2 - p1, y2, 8 - p2)
+        residual_handle.weight_scale = qscales
+        residual_handle.lock_mu = residual_handle.mu
+        residual_handle.init = False
+        return codes
     q = tensor / qscales
     q.round_()
     if isinstance(residual_handle, ResidualTensor):
@@ -1057,6 +1069,14 @@ class MyAdam(torch.optim.Adam):
         """Latent weight of a QuantTensor: dequantised codes + residual (utils/quant.py:1066-1079)."""
         if isinstance(p.residual, ResidualTensor):
             if p.wbit == 8:
+                r, qs = p.residual, p.qparam
+                if (FUSED_LATENT and not r.init and dtype == torch.bfloat16 and p.data.is_cuda and p.data.dtype == torch.int8
+                        and p.data.dim() == 2 and p.data.is_contiguous() and p.data.shape[1] % 16 == 0
+                        and torch.is_tensor(qs) and qs.dtype == torch.bfloat16 and qs.is_contiguous()
+                        and tuple(qs.shape) == (p.data.shape[0], 1) and r.weight_scale is not None
+                        and r.weight_scale.data_ptr() == qs.data_ptr() and r.residual_int.is_cuda):
+                    p1, y1, p2, y2 = three_fold_curve_4bit(r.lock_mu)
+                    return ops.latent_w8_reconstruct(p.data, qs.view(-1), r.residual_int.view(-1), p1, y1, p2 - p1, y2, 8 - p2)
                 return p.residual.add((p.data * p.qparam).to(dtype))
             if p.wbit == 4:
                 r = p.residual

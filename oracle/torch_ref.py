@@ -198,6 +198,37 @@ def quant_8bit_res(latent, qscales, carry=None):
     return q.clamp(-128, 127).to(torch.int8), res
 
 
+@torch.no_grad()
+def latent_w8_reconstruct(codes, qscales, residual_int, curve):
+    """Latent weight of an 8-bit-weight layer in lbit = 4 mode, the reference's chain on CPU tensors:
+    (p.data * p.qparam).to(bf16) (utils/quant.py:1069-1070) + ResidualTensor.add (:826-837) with the residual decoded by
+    the C restatement of the codec. codes int8 [N,K], qscales bf16 [N,1]."""
+    import numpy as np
+    from . import c_oracle as co
+    p1, y1, p2, y2 = curve
+    w = (codes * qscales).to(torch.bfloat16)
+    r_bits = co.residual_dequant(residual_int.numpy().view(np.uint32), 0, p1, y1, p2 - p1, y2, 8 - p2)
+    r = torch.from_numpy(r_bits.view(np.int16).copy()).view(torch.bfloat16)
+    r = (r.view(codes.shape) * qscales).to(torch.bfloat16)
+    return r.add(w)
+
+
+@torch.no_grad()
+def latent_w8_requant(latent, qscales, curve):
+    """Qfunc_8bit_res with a ResidualTensor handle (utils/quant.py:88-103, 803-811) on CPU tensors: returns
+    (codes int8 [N,K], residual words int32)."""
+    import numpy as np
+    from . import c_oracle as co
+    p1, y1, p2, y2 = curve
+    q = latent / qscales
+    q.round_()
+    f = (latent / qscales - q).to(torch.bfloat16).contiguous()
+    words, carry_bits = co.residual_quant(f.view(torch.int16).numpy().view(np.uint16), 0, p1, y1, p2 - p1, y2, 8 - p2)
+    carry = torch.from_numpy(carry_bits.view(np.int16).copy()).view(torch.bfloat16).view(latent.shape)
+    q += carry
+    return q.clamp_(-128, 127).to(torch.int8), torch.from_numpy(words.view(np.int32).copy())
+
+
 # --------------------------------------------------------------- 8-bit gradient accumulator ---
 def gradq8_find_param(data):
     """GradientQTensor.find_param, utils/quant.py:856-861 (bit = 8)."""

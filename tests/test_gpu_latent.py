@@ -64,6 +64,86 @@ def test_requant_matches_the_tensor_op_chain(ops, N, K, mu):
     assert float(err.max()) <= 0.25, float(err.max())
 
 
+@pytest.mark.parametrize("mu", [0, 1, 2, 3])
+@pytest.mark.parametrize("N,K", [(8, 16), (40, 400), (256, 1024)])
+def test_w8_latent_passes_match_the_tensor_op_chain(ops, N, K, mu):
+    """8-bit weights with a 4-bit residual: reconstruct and re-quantise as single passes against the reference's chain
+    of bf16 tensor operations on the CPU around the C codec, bit for bit; with saturating rows, exact halves, carries,
+    a NaN, and scales outside the range of the reciprocal form."""
+    from oracle import torch_ref as tr
+    p1, y1, p2, y2 = CURVES[mu]
+    g = torch.Generator().manual_seed(N + K + mu)
+    codes = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+    qs = ((torch.randn(N, 1, generator=g) * 0.01).abs() + 1e-3).to(torch.bfloat16)
+    if N > 4:
+        qs[2], qs[3] = 2.0 ** -50, 2.0 ** 45
+    residual = torch.randint(-2 ** 31, 2 ** 31 - 1, (N * K // 8,), generator=g, dtype=torch.int64).to(torch.int32)
+    want = tr.latent_w8_reconstruct(codes, qs, residual, CURVES[mu])
+    got = ops.latent_w8_reconstruct(codes.cuda(), qs.cuda(), residual.cuda(), p1, y1, p2 - p1, y2, 8 - p2)
+    assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16))
+    noise = torch.rand((N, K), generator=g) - 0.5
+    latent = (codes.float() + noise * 1.2) * qs.float()
+    latent.view(-1)[::37] = ((codes.float() + 0.5) * qs.float()).view(-1)[::37]
+    latent.view(-1)[5::101] = (300.0 * qs.float().expand(N, K)).reshape(-1)[5::101]
+    latent.view(-1)[7::103] = (-300.0 * qs.float().expand(N, K)).reshape(-1)[7::103]
+    latent = latent.to(torch.bfloat16)
+    if N > 4:
+        latent[4, 3] = float("nan")
+    want_codes, want_res = tr.latent_w8_requant(latent.clone(), qs, CURVES[mu])
+    res = torch.empty(N * K // 8, dtype=torch.int32, device="cuda")
+    got_codes = ops.latent_w8_requant(latent.cuda(), qs.cuda(), res, p1, y1, p2 - p1, y2, 8 - p2)
+    keep = ~torch.isnan(latent.float())
+    assert torch.equal(got_codes.cpu()[keep], want_codes[keep])
+    assert int(got_codes.cpu()[~keep].abs().sum()) == 0      # NaN -> code 0
+    if bool(keep.all()):
+        assert torch.equal(res.cpu(), want_res)
+    else:
+        words_ok = keep.view(-1, 8).all(dim=1)
+        assert torch.equal(res.cpu()[words_ok], want_res[words_ok])
+
+
+def _run_steps_w8(Q, fused, steps=4):
+    Q.FUSED_LATENT = fused
+    torch.manual_seed(0)
+    N, K = 128, 256
+    g = torch.Generator().manual_seed(5)
+    w8 = torch.randint(-120, 121, (N, K), generator=g, dtype=torch.int8)
+    qs = ((torch.randn(N, 1, generator=g) * 0.01).abs() + 2e-3).to(torch.bfloat16)
+    layer = Q.QLinearA8W8(K, N, bias=False, lbit=4, gbit=16)
+    layer.qscales.data = qs.clone()
+    layer.weight.set_value(w8, layer.qscales)
+    layer = layer.bfloat16().cuda()
+    layer.to("cuda")
+    layer.weight.requires_grad = True
+    layer.add_hook()
+    opt = Q.MyAdam([{"params": [layer.weight]}], lr=2e-3, betas=(0.9, 0.999), obit=16, mu_updata_f=20)
+    x = randn_bf16((64, K), 11).cuda().requires_grad_(True)
+    tgt = randn_bf16((64, N), 12).cuda()
+    for _ in range(steps):
+        y = layer(x)
+        ((y.float() - tgt.float()) ** 2).mean().backward()
+        opt.step()
+    return layer.weight.data.clone().cpu(), layer.weight.residual.residual_int.clone().cpu(), w8
+
+
+def test_optimizer_steps_on_8bit_weights_fused_equals_unfused(hip_lib, monkeypatch):
+    from latentq_llm_amd import ops as O
+    from latentq_llm_amd import quant as Q
+    calls = {"reconstruct": 0, "requant": 0}
+    rec, req = O.latent_w8_reconstruct, O.latent_w8_requant
+    monkeypatch.setattr(O, "latent_w8_reconstruct", lambda *a, **k: (calls.__setitem__("reconstruct", calls["reconstruct"] + 1), rec(*a, **k))[1])
+    monkeypatch.setattr(O, "latent_w8_requant", lambda *a, **k: (calls.__setitem__("requant", calls["requant"] + 1), req(*a, **k))[1])
+    try:
+        c1, r1, w8 = _run_steps_w8(Q, True)
+        assert calls == {"reconstruct": 3, "requant": 4}  # the first step has no stored residual yet
+        c0, r0, _ = _run_steps_w8(Q, False)
+        assert calls == {"reconstruct": 3, "requant": 4}
+    finally:
+        Q.FUSED_LATENT = True
+    assert torch.equal(c1, c0) and torch.equal(r1, r0)
+    assert not torch.equal(c1, w8)  # the steps did move the weights
+
+
 def _run_steps(Q, fused, steps=4):
     Q.FUSED_LATENT = fused
     torch.manual_seed(0)
