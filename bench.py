@@ -140,20 +140,20 @@ MLP_FLOP = 6 * 2 * TOKENS * HID * FFN  # 1 108.1 GFLOP
 # with profiles/gemm_a16w4_c2_counters.md from two counter runs of
 #   rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --profile-target gemm     (then WRITE_SIZE)
 # each scaled by what the same counter reads for the 256 MiB calibration copy of the same run.
-PMC_LAUNCHES = {"fwd_gate_up": 2, "fwd_down": 1, "dx_gate_up": 2, "dx_down": 1}  # per MLP step
+PMC_LAUNCHES = ("fwd_gate_up_silu", "fwd_down", "dx_down_silu_bwd", "dx_gate", "dx_up_acc")  # the five launches of a step
 
 
 def gemm_traffic_bytes():
-    """Launch-weighted mean HBM bytes (read + written) per GEMM launch of the MLP step, or None when
-    the counter summary is missing."""
+    """Mean HBM bytes (read + written) per product of the MLP step (its five launches hold six), or None when the
+    counter summary is missing."""
     path = os.path.join(ROOT, "profiles", "gemm_a16w4_c2_counters.json")
     try:
         with open(path) as f:
             mb = json.load(f)["hbm_MB_per_launch"]
-        tot = sum(n * (mb[k]["read"] + mb[k]["written"]) for k, n in PMC_LAUNCHES.items())
+        tot = sum(mb[k]["read"] + mb[k]["written"] for k in PMC_LAUNCHES)
     except (OSError, KeyError, ValueError):
         return None
-    return tot * 1e6 / sum(PMC_LAUNCHES.values())
+    return tot * 1e6 / 6
 
 
 def _requant_sets(device, N, K, nb, seed0):
@@ -537,32 +537,40 @@ def profile_target(device, which, launches=10):
         _C.call("lq_calib_copy", src.data_ptr(), dst.data_ptr(), nbytes, st)
     del src, dst
     if which == "gemm":
+        # every launch of the benchmark step, and the plain-store forms of the same products, 10 times each in this order
+        # (launches that share a kernel name and grid are told apart by their position in the sequence)
         blk = MLPBlock(device)
         h = torch.randn(TOKENS, FFN, device=device).to(torch.bfloat16)
         for _ in range(launches):
-            o.a16w4_forward(blk.x, *blk.gate, (FFN, HID))
+            o.a16w4_forward(blk.x, *blk.gate, (FFN, HID))                      # 1 forward gate (or up), plain
         for _ in range(launches):
-            o.a16w4_forward(h, *blk.down, (HID, FFN))
+            o.a16w4_forward(h, *blk.down, (HID, FFN))                          # 2 forward down
         for _ in range(launches):
-            o.a16w4_dx(h, *blk.gate, (FFN, HID))
+            o.a16w4_dx(h, *blk.gate, (FFN, HID))                               # 3 dX gate, plain store
         for _ in range(launches):
-            o.a16w4_dx(blk.dy, *blk.down, (HID, FFN))
-        # the fused product silu(gate(x)) * up(x) (inference form, then the training form that also stores the two
-        # products), the down dX with the silu backward epilogue, the accumulating dX, and the 128 x 128-tile
-        # instance of the forward kernel
+            o.a16w4_dx(blk.dy, *blk.down, (HID, FFN))                          # 4 dX down, plain store
         hbuf = torch.empty((TOKENS, FFN), dtype=torch.bfloat16, device=device)
         for _ in range(launches):
-            o.a16w4_gate_up_silu(blk.x, blk.gate, blk.up, (FFN, HID), out=hbuf)
+            _, g_, u_ = o.a16w4_gate_up_silu(blk.x, blk.gate, blk.up, (FFN, HID), out=hbuf, save=True)  # 5 fused gate / up, stores g, u, h
         for _ in range(launches):
-            _, g_, u_ = o.a16w4_gate_up_silu(blk.x, blk.gate, blk.up, (FFN, HID), out=hbuf, save=True)
-        for _ in range(launches):
-            dg_, du_ = o.a16w4_dx_silu_bwd(blk.dy, *blk.down, (HID, FFN), g_, u_)
+            dg_, du_ = o.a16w4_dx_silu_bwd(blk.dy, *blk.down, (HID, FFN), g_, u_)  # 6 dX down with the silu-backward epilogue
         dxb = torch.zeros((TOKENS, HID), dtype=torch.bfloat16, device=device)
         for _ in range(launches):
-            o.a16w4_dx(du_, *blk.up, (FFN, HID), out=dxb, accumulate=True)
+            o.a16w4_dx(du_, *blk.up, (FFN, HID), out=dxb, accumulate=True)     # 7 dX up, accumulating
         x1536 = torch.randn(1536, HID, device=device).to(torch.bfloat16)
         for _ in range(launches):
-            o.a16w4_forward(x1536, *blk.gate, (FFN, HID))
+            o.a16w4_forward(x1536, *blk.gate, (FFN, HID))                      # 8 forward gate at 1536 tokens (128 x 128 tiles)
+    elif which == "dw":
+        # the weight-gradient GEMM on the two MLP shapes: plain store, then the int8 accumulate epilogue
+        for (N, K) in [(FFN, HID), (HID, FFN)]:
+            dy = torch.randn(TOKENS, N, device=device).to(torch.bfloat16)
+            x = torch.randn(TOKENS, K, device=device).to(torch.bfloat16)
+            q8 = torch.zeros((N, K), dtype=torch.int8, device=device)
+            sc = torch.full((N, 1), 1e-3, dtype=torch.bfloat16, device=device)
+            for _ in range(launches):
+                o.weight_grad(dy, x)
+            for i in range(launches):
+                o.weight_grad_acc8(dy, x, q8, sc, seed=1, offset=i)
     elif which == "requant":
         # the benchmark size (8192 x 2048), then 4 and 16 times as many rows: steady state against launch cost
         for rows in (8192, 4 * 8192, 16 * 8192):
@@ -748,7 +756,7 @@ def main():
     ap.add_argument("--settle-ms", type=float, default=150.0, help="untimed steps run for at least this long before the warm-up")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-mlp", action="store_true", help="skip the side measurements (requant, GEMV, A8W8)")
-    ap.add_argument("--profile-target", choices=["gemm", "requant", "gemv", "a8w8", "latent", "adam8", "gradq8", "ceiling"],
+    ap.add_argument("--profile-target", choices=["gemm", "requant", "gemv", "a8w8", "latent", "adam8", "gradq8", "dw", "ceiling"],
                     help="run only a short fixed launch sequence of one kernel family (for rocprofv3); prints nothing except for 'ceiling'")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -814,7 +822,7 @@ def main():
                 "avg_launch_us": avg_us, "flop_per_launch": one,
                 "note": "per product of 2*2048*4096*11008 flop: total time of the step's five GEMM launches / 6 (the gate/up launch holds two)",
                 "traffic": gemm_traffic_bytes(),
-                "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated on a copy)"}
+                "traffic_unit": "HBM bytes per product: the five launches' rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated on a copy, / 6"}
     # the step with the glue as tensor-library kernels, for comparison
     for _ in range(20):
         blk.step_unfused()
