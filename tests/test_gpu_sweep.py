@@ -99,3 +99,63 @@ def test_forward_128x128_direct_kernel_identity_is_exact_dequant(ops):
     x = torch.eye(K, device="cuda", dtype=torch.bfloat16)
     y = ops.a16w4_forward(x, *w, (N, K))
     assert torch.equal(y, ops.a16w4_dequant(*w, (N, K)).t().contiguous())
+
+
+def _dw_shapes(seed, n):
+    rng = random.Random(seed)
+    out = []
+    for _ in range(n):
+        M = 64 * rng.randint(1, 40)
+        N = 8 * rng.randint(1, 700) if rng.random() < 0.6 else rng.choice([256, 4096, 11008])
+        K = 16 * rng.randint(1, 300) if rng.random() < 0.6 else rng.choice([256, 4096, 11008])
+        if N * K > 24e6:
+            K = 16 * max(1, int(24e6 // N) // 16)
+        out.append((M, N, K))
+    return out
+
+
+@pytest.mark.parametrize("M,N,K", _dw_shapes(5, 24))
+def test_weight_grad_random_shapes(ops, M, N, K):
+    """dW = dY^T X over random shapes (partial tiles along both output dimensions, 1 to 40 reduction steps) against
+    the fp32 product on the GPU; the int8 accumulate epilogue against the stand-alone pass on the stored product."""
+    g = torch.Generator(device="cuda").manual_seed(M + N + K)
+    dy = (torch.randn(M, N, device="cuda", generator=g) * 0.05).to(torch.bfloat16)
+    x = torch.randn(M, K, device="cuda", generator=g).to(torch.bfloat16)
+    dw = ops.weight_grad(dy, x)
+    ref = dy.float().t() @ x.float()
+    assert ((dw.float() - ref).norm() / ref.norm()).item() < TOL
+    q = torch.randint(-100, 100, (N, K), device="cuda", generator=g, dtype=torch.int8)
+    s = (torch.rand(N, 1, device="cuda", generator=g) * 0.01 + 1e-3).to(torch.bfloat16)
+    q2 = q.clone()
+    ops.weight_grad_acc8(dy, x, q, s, seed=3, offset=M)
+    ops.gradq8_quant(dw, q2, s, True, seed=3, offset=M)
+    assert torch.equal(q, q2)
+
+
+@pytest.mark.parametrize("M,N,K", _shapes(7, 16, [17, 100, 256, 300, 1024, 2050], [4096, 8192, 11008], 24))
+def test_dx_epilogues_and_int8_dx_random_shapes(ops, M, N, K):
+    """The accumulate and SiLU-backward epilogues of the dX kernel and the dX from int8 codes over random shapes."""
+    if N % 64:
+        N = (N // 64 + 1) * 64
+    _, packed, scales, zeros = make_w4(N, K, M + N + K)
+    w = (packed.cuda(), scales.cuda(), zeros.cuda())
+    g = torch.Generator(device="cuda").manual_seed(M * 3 + 2)
+    dy = torch.randn(M, N, device="cuda", generator=g).to(torch.bfloat16)
+    base = torch.randn(M, K, device="cuda", generator=g).to(torch.bfloat16)
+    W = ops.a16w4_dequant(*w, (N, K)).float()
+    ref = dy.float() @ W
+    acc = base.clone()
+    ops.a16w4_dx(dy, *w, (N, K), out=acc, accumulate=True)
+    want = base.float() + ref
+    assert ((acc.float() - want).norm() / want.norm()).item() < TOL
+    gg = torch.randn(M, K, device="cuda", generator=g).to(torch.bfloat16)
+    uu = torch.randn(M, K, device="cuda", generator=g).to(torch.bfloat16)
+    dg, du = ops.a16w4_dx_silu_bwd(dy, *w, (N, K), gg, uu)
+    sg = torch.sigmoid(gg.float())
+    for got, wnt in ((dg, ref * uu.float() * sg * (1 + gg.float() * (1 - sg))), (du, ref * gg.float() * sg)):
+        assert ((got.float() - wnt).norm() / wnt.norm()).item() < 2 * TOL
+    w8 = torch.randint(-128, 128, (N, K), device="cuda", generator=g, dtype=torch.int8)
+    qs = (torch.rand(N, device="cuda", generator=g) * 0.01 + 1e-3).to(torch.bfloat16)
+    dx8 = ops.a8w8_dx(dy, w8, qs)
+    ref8 = dy.float() @ (w8.to(torch.bfloat16) * qs[:, None]).to(torch.bfloat16).float()
+    assert ((dx8.float() - ref8).norm() / ref8.norm()).item() < TOL
