@@ -288,6 +288,46 @@ def test_a16w4_fwd_integer_exact(ops, co):
     assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("N,K", [(64, 256), (256, 4096), (8224, 1024), (512, 11008), (11008, 512)])
+@pytest.mark.parametrize("M", [1, 3, 4, 7, 8, 13, 16])
+def test_gemv_one_hot_tokens_give_the_exact_dequantised_weights(ops, co, N, K, M):
+    """Decode path at bit level: token m is one-hot at a column k_m, so y[m, n] = s (P - (128 + z) S) with
+    P = 128 + q and S = 1, i.e. s (q - z) formed exactly in fp32 and rounded once: the reference's dequantised weight
+    W[n, k_m] bit for bit (integer zeros). Shapes and token counts walk through every GEMV configuration (2 to 16
+    waves, 4 / 8 / 16 staged rows, one and two row tiles, scales through LDS, tail batches of fewer than 4 groups)."""
+    codes, packed, scales, zeros = make_w4(N, K, N + K + M)
+    ks = [(37 * m + 5) * 131 % K for m in range(M)]
+    ks[0], ks[-1] = (0, K - 1) if M > 1 else (K - 1, K - 1)
+    x = torch.zeros((M, K), dtype=torch.bfloat16)
+    for m, k in enumerate(ks):
+        x[m, k] = 1.0
+    got = ops.a16w4_forward(dev(x), dev(packed), dev(scales), dev(zeros), (N, K))
+    want = co.dequant(packed.numpy(), bits(scales), bits(zeros), N, K)  # [N, K] bf16 bits
+    for m, k in enumerate(ks):
+        assert np.array_equal(bits(got[m]), want[:, k]), (m, k)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 256, 4096), (4, 512, 1024), (8, 8224, 512), (16, 256, 11008), (16, 8224, 384)])
+def test_gemv_integer_exact(ops, M, N, K):
+    """Power-of-two scales, integer zeros and small-integer activations: every partial sum of the decode kernel is
+    exact in fp32, so the output equals the exact product (which bf16 holds) whatever the order of summation."""
+    g = torch.Generator().manual_seed(M + N + K)
+    codes = torch.randint(0, 16, (N, K), generator=g, dtype=torch.uint8)
+    packed = util.pack_codes(codes)
+    G = N * K // 128
+    scales = torch.tensor([2.0 ** -(i % 2) for i in range(G)], dtype=torch.bfloat16).reshape(G, 1)
+    zeros = torch.randint(6, 10, (G, 1), generator=g).to(torch.bfloat16)
+    x = torch.zeros((M, K), dtype=torch.bfloat16)
+    nz = torch.randint(0, K, (M, 12), generator=g)
+    for m in range(M):
+        x[m, nz[m]] = (2 * torch.randint(0, 2, (12,), generator=g) - 1).to(torch.bfloat16)  # |sum| <= 12 * 9, steps of 1/2
+    got = ops.a16w4_forward(dev(x), dev(packed), dev(scales), dev(zeros), (N, K)).cpu()
+    W = (codes.double().reshape(G, 128) - zeros.double()) * scales.double()
+    want = x.double() @ W.reshape(N, K).t()
+    assert float(want.abs().max()) < 128 and torch.equal(want, want.to(torch.bfloat16).double())
+    assert torch.equal(got.double(), want)
+
+
 # ---------------------------------------------------------------- A16W4 dX --
 @pytest.mark.parametrize("M,N,K", [(17, 64, 128), (64, 128, 256), (130, 192, 384), (300, 320, 512), (1024, 3072, 768),
                                    (4, 128, 256)])
