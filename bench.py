@@ -5,7 +5,7 @@
 
 One "step" is one pass of the A16W4 Llama-2-7B MLP block at 4 x 512 = 2048 bf16 tokens:
 forward  down(silu(gate(x)) * up(x))  and the dX backward through all three projections
-(six dequant-GEMM products, 1108.1 GFLOP, in the five launches the fused training block makes:
+(six dequant-GEMM products, 1108.1 GFLOP, in the four launches the fused training block makes:
 the bf16 glue of autograd sits in the GEMM epilogues), with synthetic seeded weights and
 activations already resident in HBM. The headline value is GEMM TFLOP/s of that step. The same JSON line also
 carries the kernel roofline of the dominant kernel (measured with HIP events on the launch
@@ -107,14 +107,14 @@ class MLPBlock:
         self.dy = torch.randn(TOKENS, HID, generator=g).to(torch.bfloat16).to(device)
 
     def step(self):
-        """The block as latentq_llm_amd.fused_mlp.QuantLlamaMLP runs it in training: five launches, the bf16 glue
-        of autograd (silu, three products, silu backward, the sum of the two input gradients) in the GEMM epilogues."""
+        """The block as latentq_llm_amd.fused_mlp.QuantLlamaMLP runs it in training: four launches, the bf16 glue
+        of autograd (silu, three products, silu backward) in the GEMM epilogues and the sum of the two input
+        gradients in one reduction over both products."""
         o = self.ops
         h, g, u = o.a16w4_gate_up_silu(self.x, self.gate, self.up, (FFN, HID), save=True)
         y = o.a16w4_forward(h, *self.down, (HID, FFN))
         dg, du = o.a16w4_dx_silu_bwd(self.dy, *self.down, (HID, FFN), g, u)
-        dx = o.a16w4_dx(dg, *self.gate, (FFN, HID))
-        o.a16w4_dx(du, *self.up, (FFN, HID), out=dx, accumulate=True)
+        dx = o.a16w4_dx_pair(dg, self.gate, du, self.up, (FFN, HID))
         return y, dx
 
     def step_unfused(self):
@@ -140,11 +140,11 @@ MLP_FLOP = 6 * 2 * TOKENS * HID * FFN  # 1 108.1 GFLOP
 # with profiles/gemm_a16w4_c2_counters.md from two counter runs of
 #   rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --profile-target gemm     (then WRITE_SIZE)
 # each scaled by what the same counter reads for the 256 MiB calibration copy of the same run.
-PMC_LAUNCHES = ("fwd_gate_up_silu", "fwd_down", "dx_down_silu_bwd", "dx_gate", "dx_up_acc")  # the five launches of a step
+PMC_LAUNCHES = ("fwd_gate_up_silu", "fwd_down", "dx_down_silu_bwd", "dx_gate_up_pair")  # the four launches of a step
 
 
 def gemm_traffic_bytes():
-    """Mean HBM bytes (read + written) per product of the MLP step (its five launches hold six), or None when the
+    """Mean HBM bytes (read + written) per product of the MLP step (its four launches hold six), or None when the
     counter summary is missing."""
     path = os.path.join(ROOT, "profiles", "gemm_a16w4_c2_counters.json")
     try:
@@ -557,9 +557,11 @@ def profile_target(device, which, launches=10):
         dxb = torch.zeros((TOKENS, HID), dtype=torch.bfloat16, device=device)
         for _ in range(launches):
             o.a16w4_dx(du_, *blk.up, (FFN, HID), out=dxb, accumulate=True)     # 7 dX up, accumulating
+        for _ in range(launches):
+            o.a16w4_dx_pair(dg_, blk.gate, du_, blk.up, (FFN, HID), out=dxb)   # 8 dX of gate and up in one reduction
         x1536 = torch.randn(1536, HID, device=device).to(torch.bfloat16)
         for _ in range(launches):
-            o.a16w4_forward(x1536, *blk.gate, (FFN, HID))                      # 8 forward gate at 1536 tokens (128 x 128 tiles)
+            o.a16w4_forward(x1536, *blk.gate, (FFN, HID))                      # 9 forward gate at 1536 tokens (128 x 128 tiles)
     elif which == "dw":
         # the weight-gradient GEMM on the two MLP shapes: plain store, then the int8 accumulate epilogue
         for (N, K) in [(FFN, HID), (HID, FFN)]:
@@ -792,8 +794,8 @@ def main():
     dt = (time.perf_counter() - t0) / args.steps
     value = MLP_FLOP / dt / 1e12
 
-    # Dominant kernel: the dequant-GEMM. Per-launch duration of the step's five launches from HIP events on the
-    # launch stream (the gate / up launch holds two products: 2 x 184.68 GFLOP).
+    # Dominant kernel: the dequant-GEMM. Per-launch duration of the step's four launches from HIP events on the
+    # launch stream (the gate / up launches hold two products each: 2 x 184.68 GFLOP).
     o = blk.ops
     one = 2 * TOKENS * HID * FFN
     h, g, u = o.a16w4_gate_up_silu(blk.x, blk.gate, blk.up, (FFN, HID), save=True)
@@ -804,25 +806,25 @@ def main():
         ("fwd_gate_up_silu", lambda: o.a16w4_gate_up_silu(blk.x, blk.gate, blk.up, (FFN, HID), save=True), 2 * one),
         ("fwd_down", lambda: o.a16w4_forward(h, *blk.down, (HID, FFN)), one),
         ("dx_down_silu_bwd", lambda: o.a16w4_dx_silu_bwd(blk.dy, *blk.down, (HID, FFN), g, u), one),
-        ("dx_gate", lambda: o.a16w4_dx(dg, *blk.gate, (FFN, HID), out=dxb), one),
-        ("dx_up_acc", lambda: o.a16w4_dx(du, *blk.up, (FFN, HID), out=dxb, accumulate=True), one),
+        ("dx_gate_up_pair", lambda: o.a16w4_dx_pair(dg, blk.gate, du, blk.up, (FFN, HID), out=dxb), 2 * one),
         # the same products as separate launches with a plain store (what the layers run on their own)
         ("fwd_gate_or_up", lambda: o.a16w4_forward(blk.x, *blk.gate, (FFN, HID)), one),
         ("dx_down", lambda: o.a16w4_dx(blk.dy, *blk.down, (HID, FFN)), one),
+        ("dx_gate", lambda: o.a16w4_dx(dg, *blk.gate, (FFN, HID), out=dxb), one),
+        ("dx_up_acc", lambda: o.a16w4_dx(du, *blk.up, (FFN, HID), out=dxb, accumulate=True), one),
     ]:
         sec = event_time(fn, 50)
         kern[name] = {"us": sec * 1e6, "GFLOP": fl / 1e9, "TFLOP/s": fl / sec / 1e12, "frac_mfma_bf16": fl / sec / PEAK_BF16}
-    step_launches = ("fwd_gate_up_silu", "fwd_down", "dx_down_silu_bwd", "dx_gate", "dx_up_acc")
-    tot = sum(kern[k]["us"] for k in step_launches)
-    # per 184.68 GFLOP product: six of them in the five launches
+    tot = sum(kern[k]["us"] for k in PMC_LAUNCHES)
+    # per 184.68 GFLOP product: six of them in the four launches
     avg_us = tot / 6
     achieved = one / (avg_us * 1e-6) / 1e12
     roofline = {"bound": "mfma", "kernel": "A16W4 dequant-GEMM: gemm_fwd_direct_kernel<2, *> (forward), gemm_kernel<1> (dX)",
                 "achieved": achieved, "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": achieved * 1e12 / PEAK_BF16,
                 "avg_launch_us": avg_us, "flop_per_launch": one,
-                "note": "per product of 2*2048*4096*11008 flop: total time of the step's five GEMM launches / 6 (the gate/up launch holds two)",
+                "note": "per product of 2*2048*4096*11008 flop: total time of the step's four GEMM launches / 6 (the two gate/up launches hold two each)",
                 "traffic": gemm_traffic_bytes(),
-                "traffic_unit": "HBM bytes per product: the five launches' rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated on a copy, / 6"}
+                "traffic_unit": "HBM bytes per product: the four launches' rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated on a copy, / 6"}
     # the step with the glue as tensor-library kernels, for comparison
     for _ in range(20):
         blk.step_unfused()

@@ -165,6 +165,9 @@ int lq_a16w4_gate_up_silu(const void *x, const void *codes_gate, const void *sca
  *     tensor operations round silu(g) and P * u to bf16 in between). g, u, dg_out, du_out: bf16 [M,K].
  *   lq_a16w4_dx_acc: dx_inout = bf16(dx_inout + bf16(dY . deq(W))): the second of the two products that
  *     both flow into the block's input gradient; the same bits as lq_a16w4_dx followed by a bf16 addition.
+ *   lq_a16w4_dx_pair: dx = bf16(dY1 . deq(W1) + dY2 . deq(W2)) for two layers of one shape [N,K] fed by the same
+ *     input (gate and up): one launch whose reduction runs through both products, the sum kept in fp32 (one rounding
+ *     where lq_a16w4_dx followed by lq_a16w4_dx_acc has two). dy1, dy2: bf16 [M,N]; dx: bf16 [M,K]; N % 64 == 0.
  * Shapes and alignment as lq_a16w4_dx / lq_a16w4_gate_up_silu; all outputs 16-byte aligned. */
 int lq_a16w4_gate_up_silu_save(const void *x, const void *codes_gate, const void *scales_gate, const void *zeros_gate,
                                const void *codes_up, const void *scales_up, const void *zeros_up, void *h, void *g_out,
@@ -174,6 +177,9 @@ int lq_a16w4_dx_silu_bwd(const void *dy, const void *codes, const void *scales, 
                          void *stream);
 int lq_a16w4_dx_acc(const void *dy, const void *codes, const void *scales, const void *zeros, void *dx_inout,
                     int64_t M, int64_t N, int64_t K, int group, void *stream);
+int lq_a16w4_dx_pair(const void *dy1, const void *codes1, const void *scales1, const void *zeros1, const void *dy2,
+                     const void *codes2, const void *scales2, const void *zeros2, void *dx, int64_t M, int64_t N,
+                     int64_t K, int group, void *stream);
 
 /* Which kernel lq_a16w4_fwd(_ws) (backward = 0) or lq_a16w4_dx(_ws) (backward = 1) would run for a
  * shape and a workspace size, and how it would cut the reduction; launches nothing. *kernel is

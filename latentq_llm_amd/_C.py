@@ -39,6 +39,7 @@ SIGNATURES = {
     "lq_a16w4_gate_up_silu_save": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
     "lq_a16w4_dx_silu_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
     "lq_a16w4_dx_acc": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
+    "lq_a16w4_dx_pair": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
     "lq_w8_requant": [_vp, _vp, _vp, _i64, _i64, _vp],
     "lq_residual_quant_s": [_vp, _vp, _i64, _i32, _vp],
     "lq_gradq8_quant": [_vp, _vp, _vp, _i32, _i64, _i64, _vp, _u64, _u64, _vp],

@@ -81,6 +81,10 @@ struct GemmParams {
     int ep_mode;
     const unsigned short *ep_g, *ep_u;
     unsigned short *c2;
+    // MODE_W4_DX, two products into one output: c = a * deq(b) + a2 * deq(b2), both pairs of the shape (M, R) x (R, C).
+    // The reduction runs over the first pair's R / 64 steps and then over the second's; a2 = null: one product.
+    const void *a2, *b2;
+    const unsigned short *scales2, *zeros2;
 };
 
 enum { EP_STORE = 0, EP_ADD = 1, EP_SILU_BW = 2 };
@@ -177,7 +181,9 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
     const int m0 = tile_m * BM, c0 = tile_n * BN;
     // reduction steps of this workgroup: all of them, or one slice of a split reduction
     const int k0 = p.partial ? (int)blockIdx.y * p.steps_per_split : 0;
-    const int nk = p.partial ? (p.R / RT - k0 < p.steps_per_split ? p.R / RT - k0 : p.steps_per_split) : p.R / RT;
+    const bool pair = MODE == MODE_W4_DX && p.a2 != nullptr;  // never together with a split reduction
+    const int n1 = p.R / RT;                                  // steps of the first (or only) product
+    const int nk = p.partial ? (n1 - k0 < p.steps_per_split ? n1 - k0 : p.steps_per_split) : pair ? 2 * n1 : n1;
     const int groups_per_row = p.Kw / LQ_GROUP;
 
     if (is_weight_wave) {
@@ -198,6 +204,8 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
         int b_dst[MODE == MODE_I8 ? BPT : 1];
         const unsigned short *s_src[NSZ];
         const unsigned short *z_src[NSZ];
+        const unsigned char *b_src2 = nullptr;  // W4_DX: the second product's codes, scales and zeros
+        const unsigned short *s_src2 = nullptr, *z_src2 = nullptr;
         int b_row = 0, b_w0 = 0;  // W4_FWD: LDS row and first word; W4_DX: LDS row (n) and quarter of the row
 
         if constexpr (MODE == MODE_I8) {
@@ -232,6 +240,11 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             const int g = (c0 + b_w0 * 32) / LQ_GROUP;
             s_src[0] = p.scales + ((long long)k0 * 64 + b_row) * groups_per_row + g;
             z_src[0] = p.zeros + ((long long)k0 * 64 + b_row) * groups_per_row + g;
+            if (pair) {
+                b_src2 = (const unsigned char *)p.b2 + (long long)b_row * (p.Kw / 2) + c0 / 2 + b_w0 * 16;
+                s_src2 = p.scales2 + (long long)b_row * groups_per_row + g;
+                z_src2 = p.zeros2 + (long long)b_row * groups_per_row + g;
+            }
         }
 
         struct Stage {
@@ -269,12 +282,13 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
                 for (int i = 0; i < 4; ++i) { S.w[i] = v0[i]; S.w[4 + i] = v1[i]; }
                 S.s[0] = s_src[0][row_off];
             } else {
-                const long long row_off = (long long)kt * 64;
-                u32x4_t v = *reinterpret_cast<const u32x4_t *>(b_src[0] + row_off * (p.Kw / 2));
+                const bool second = kt >= n1 && pair;
+                const long long row_off = (long long)(second ? kt - n1 : kt) * 64;
+                u32x4_t v = *reinterpret_cast<const u32x4_t *>((second ? b_src2 : b_src[0]) + row_off * (p.Kw / 2));
 #pragma unroll
                 for (int i = 0; i < 4; ++i) S.w[i] = v[i];
-                S.s[0] = s_src[0][row_off * groups_per_row];
-                S.z[0] = z_src[0][row_off * groups_per_row];
+                S.s[0] = (second ? s_src2 : s_src[0])[row_off * groups_per_row];
+                S.z[0] = (second ? z_src2 : z_src[0])[row_off * groups_per_row];
             }
         };
 
@@ -362,6 +376,7 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
         a_off[i] = (unsigned)((gr - m0) * lda + ch * 16);
     }
     const unsigned char *a_base = (const unsigned char *)p.a + m0 * lda + (long long)k0 * ROWB;
+    const unsigned char *a_base2 = pair ? (const unsigned char *)p.a2 + m0 * lda : a_base;
     // LDS-direct load: lane l of the wave writes 16 bytes at (wave-uniform base) + 16*l. Written as
     // inline assembly (M0 = LDS base, one wait state, then the load with a scalar base and a 32-bit
     // lane offset) so that the compiler's wait-count insertion does not see an LDS write it cannot
@@ -370,7 +385,11 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
     static_assert(APT % 4 == 0, "A loads are issued in four parts per tile");
     // part q (0..3) of a tile's loads: APT/4 of them
     auto issue_a_part = [&](int kt, unsigned char *la, int q) {
-        const unsigned char *src = a_base + (long long)kt * ROWB;
+        const bool second = kt >= n1 && pair;
+        const unsigned long long addr = (unsigned long long)((second ? a_base2 : a_base) + (long long)(second ? kt - n1 : kt) * ROWB);
+        // the load takes its base from scalar registers
+        const unsigned char *src = (const unsigned char *)(((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane((int)(addr >> 32)) << 32) |
+                                                           (unsigned)__builtin_amdgcn_readfirstlane((int)addr));
 #pragma unroll
         for (int i = q * (APT / 4); i < (q + 1) * (APT / 4); ++i) {
             const unsigned lds_addr = (unsigned)reinterpret_cast<size_t>((lds_void *)(la + (i * NT + wave * 64) * 16));
@@ -1074,6 +1093,28 @@ extern "C" int lq_a16w4_dx_acc(const void *dy, const void *codes, const void *sc
     DxEpilogue ep;
     ep.mode = EP_ADD;
     return a16w4_dx_impl("lq_a16w4_dx_acc", dy, codes, scales, zeros, dx_inout, M, N, K, group, nullptr, 0, stream, nullptr, ep);
+}
+
+// dx = dy1 * deq(W1) + dy2 * deq(W2) for two layers of the same shape that share their input (gate and up of an MLP
+// block): one launch whose reduction runs through the first product and on into the second, the sum kept in the fp32
+// accumulators (one rounding to bf16 where lq_a16w4_dx followed by lq_a16w4_dx_acc has two).
+extern "C" int lq_a16w4_dx_pair(const void *dy1, const void *codes1, const void *scales1, const void *zeros1, const void *dy2,
+                                const void *codes2, const void *scales2, const void *zeros2, void *dx, int64_t M, int64_t N,
+                                int64_t K, int group, void *stream) {
+    const char *who = "lq_a16w4_dx_pair";
+    int rc = check_w4_common(who, dy1, codes1, scales1, zeros1, dx, M, N, K, group);
+    if (rc) return rc;
+    rc = check_w4_common(who, dy2, codes2, scales2, zeros2, dx, M, N, K, group);
+    if (rc) return rc;
+    LQ_REQUIRE(N % 64 == 0, "%s: N=%lld must be a multiple of 64", who, (long long)N);
+    GemmParams p = {};
+    p.a = dy1; p.b = codes1; p.scales = (const unsigned short *)scales1; p.zeros = (const unsigned short *)zeros1;
+    p.a2 = dy2; p.b2 = codes2; p.scales2 = (const unsigned short *)scales2; p.zeros2 = (const unsigned short *)zeros2;
+    p.c = dx;
+    p.M = (int)M; p.C = (int)K; p.R = (int)N; p.Kw = (int)K;
+    const W4Plan plan = plan_dx(M, N, K, 0, lq_device_cu_count());
+    return plan.kernel == LQ_PLAN_STAGED_256 ? launch_gemm<MODE_W4_DX, 256, 128, 2, 2>(p, (hipStream_t)stream, who)
+                                             : launch_gemm<MODE_W4_DX, 128, 128, 2, 2>(p, (hipStream_t)stream, who);
 }
 
 extern "C" int lq_a16w4_dx_silu_bwd(const void *dh_dy, const void *codes, const void *scales, const void *zeros, const void *g,

@@ -5,7 +5,7 @@ for this package's ``QLinearA16W4`` layers (native code layout): ``forward`` is
 ``down_proj(silu(gate_proj(x)) * up_proj(x))`` with the first three operations done by
 ``lq_a16w4_gate_up_silu`` on fp32 accumulators, as the reference's Triton kernel does (:160-166).
 The reference's fused MLP is inference only. Here a block whose layers are being trained (backward hooks
-installed, or an input that needs a gradient) runs the same five launches forward and backward with the
+installed, or an input that needs a gradient) runs four launches forward and backward with the
 tensor-library glue folded into the GEMM epilogues (``_FusedMLPTrain``), and hands the three weight
 gradients to the layers' accumulators exactly as their own backward hooks would.
 """
@@ -31,8 +31,8 @@ def _w4(layer):
 class _FusedMLPTrain(torch.autograd.Function):
     """down(silu(gate(x)) * up(x)) for layers in training. Forward: the gate / up launch also stores the two
     products (lq_a16w4_gate_up_silu_save), then the down projection. Backward: the down projection's dX with the
-    backward of silu(g) * u as its epilogue (lq_a16w4_dx_silu_bwd), the gate dX, the up dX added into it
-    (lq_a16w4_dx_acc); dW of the three layers as QLinearFunctionW4.backward forms them (utils/quant.py:141-142),
+    backward of silu(g) * u as its epilogue (lq_a16w4_dx_silu_bwd), then the gate and the up dX summed in one
+    launch (lq_a16w4_dx_pair); dW of the three layers as QLinearFunctionW4.backward forms them (utils/quant.py:141-142),
     delivered through dict_temp and backward_hook_fn (utils/quant.py:398-411) layer by layer."""
 
     @staticmethod
@@ -57,8 +57,7 @@ class _FusedMLPTrain(torch.autograd.Function):
         dg, du = ops.a16w4_dx_silu_bwd(dy, *_w4(down), (mlp.outfeatures, inter), g, u)
         dx = None
         if ctx.needs_input_grad[0]:
-            dx = ops.a16w4_dx(dg, *_w4(gate), (inter, K))
-            ops.a16w4_dx(du, *_w4(up), (inter, K), out=dx, accumulate=True)
+            dx = ops.a16w4_dx_pair(dg, _w4(gate), du, _w4(up), (inter, K))
         for layer, dyl, xin in ((down, dy, h), (up, du, x2), (gate, dg, x2)):
             if layer.hook_handle is not None:
                 dict_temp.append(_pending_dw(dyl, xin))

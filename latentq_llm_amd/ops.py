@@ -248,6 +248,33 @@ def a16w4_dx(dy, codes, scales, zeros, shape, out=None, accumulate=False):
     return dx
 
 
+def a16w4_dx_pair(dy1, w1, dy2, w2, shape, out=None):
+    """dX[M,K] = bf16(dY1 . deq(W1) + dY2 . deq(W2)) in one launch (lq_a16w4_dx_pair); w1, w2 = (codes, scales, zeros)
+    of two [N, K] matrices."""
+    N, K = shape
+    for name, dy, w in (("dy1", dy1, w1), ("dy2", dy2, w2)):
+        _chk(dy, torch.bfloat16, name)
+        if dy.dim() != 2 or dy.shape[1] != N:
+            raise ValueError(f"{name} must be [M,{N}], got {tuple(dy.shape)}")
+        _codes_ok(w[0], N, K)
+        _qparam_ok(w[1], w[2], N, K)
+    if dy1.shape != dy2.shape:
+        raise ValueError("dy1 and dy2 must have the same shape")
+    M = dy1.shape[0]
+    if out is None:
+        out = torch.empty((M, K), dtype=torch.bfloat16, device=dy1.device)
+    else:
+        _chk(out, torch.bfloat16, "out")
+        if tuple(out.shape) != (M, K):
+            raise ValueError(f"out must be [{M},{K}]")
+    if M == 0:
+        return out
+    with torch.cuda.device(dy1.device):
+        _C.call("lq_a16w4_dx_pair", dy1.data_ptr(), w1[0].data_ptr(), w1[1].data_ptr(), w1[2].data_ptr(), dy2.data_ptr(),
+                w2[0].data_ptr(), w2[1].data_ptr(), w2[2].data_ptr(), out.data_ptr(), M, N, K, GROUP, _stream(dy1))
+    return out
+
+
 PLAN_KERNELS = {0: "gemv", 1: "gemv_chunks", 2: "direct_128x256", 3: "staged_128x128", 4: "staged_256x128",
                 5: "direct_128x128"}
 

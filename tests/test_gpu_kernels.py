@@ -880,6 +880,31 @@ def test_dx_epilogue_forms(ops, M, N, K):
         assert bool((diff <= scale * 2.0 ** -7 + 2e-5 * (1 + uf.abs() + gf.abs())).all())
 
 
+@pytest.mark.parametrize("M,N,K", [(2048, 1024, 512), (100, 256, 384), (520, 1408, 512), (17, 64, 128)])
+def test_dx_pair(ops, M, N, K):
+    """lq_a16w4_dx_pair = dY1 . deq(W1) + dY2 . deq(W2) in one reduction: against float64; with one of the two
+    gradients zero it is the other product's unsplit kernel bit for bit (the reduction only gains exact zeros),
+    which pins which operands go together and the order of the two halves."""
+    _, p1, s1, z1 = make_w4(N, K, 3)
+    _, p2, s2, z2 = make_w4(N, K, 13)
+    w1, w2 = (dev(p1), dev(s1), dev(z1)), (dev(p2), dev(s2), dev(z2))
+    dy1, dy2 = dev(randn_bf16((M, N), 4)), dev(randn_bf16((M, N), 14))
+    got = ops.a16w4_dx_pair(dy1, w1, dy2, w2, (N, K))
+    want = dy1.double() @ ops.a16w4_dequant(*w1, (N, K)).double() + dy2.double() @ ops.a16w4_dequant(*w2, (N, K)).double()
+    assert rel_l2(got, want) < 3e-3
+    assert bool(((got.double() - want).abs() <= want.abs() * 2.0 ** -8 + 1e-3 * N ** 0.5 * 2.0 ** -8).all())
+    zero = torch.zeros_like(dy1)
+    for a, b, single in ((dy1, zero, (dy1, w1)), (zero, dy2, (dy2, w2))):
+        base = torch.zeros((M, K), dtype=torch.bfloat16, device=dy1.device)
+        ops.a16w4_dx(single[0], *single[1], (N, K), out=base, accumulate=True)  # the unsplit kernel: 0 + P
+        assert torch.equal(ops.a16w4_dx_pair(a, w1, b, w2, (N, K)), base)
+    # the caller's buffer, and argument checks
+    out = torch.empty((M, K), dtype=torch.bfloat16, device=dy1.device)
+    assert ops.a16w4_dx_pair(dy1, w1, dy2, w2, (N, K), out=out) is out and torch.equal(out, got)
+    with pytest.raises(ValueError):
+        ops.a16w4_dx_pair(dy1, w1, dy2[:-1], w2, (N, K))
+
+
 @pytest.mark.parametrize("N,K", [(1, 8), (12, 64), (100, 1032), (2048, 8192)])
 def test_w8_requant_bit_exact(ops, co, N, K):
     """lq_w8_requant against the C restatement of Qfunc_8bit_res: random latents, ties, saturation, infinities, NaN

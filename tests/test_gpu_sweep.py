@@ -134,7 +134,8 @@ def test_weight_grad_random_shapes(ops, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", _shapes(7, 16, [17, 100, 256, 300, 1024, 2050], [4096, 8192, 11008], 24))
 def test_dx_epilogues_and_int8_dx_random_shapes(ops, M, N, K):
-    """The accumulate and SiLU-backward epilogues of the dX kernel and the dX from int8 codes over random shapes."""
+    """The accumulate and SiLU-backward epilogues of the dX kernel, two products in one reduction, and the dX from int8
+    codes over random shapes."""
     if N % 64:
         N = (N // 64 + 1) * 64
     _, packed, scales, zeros = make_w4(N, K, M + N + K)
@@ -154,6 +155,12 @@ def test_dx_epilogues_and_int8_dx_random_shapes(ops, M, N, K):
     sg = torch.sigmoid(gg.float())
     for got, wnt in ((dg, ref * uu.float() * sg * (1 + gg.float() * (1 - sg))), (du, ref * gg.float() * sg)):
         assert ((got.float() - wnt).norm() / wnt.norm()).item() < 2 * TOL
+    _, packed2, scales2, zeros2 = make_w4(N, K, M + N + K + 1)
+    w2 = (packed2.cuda(), scales2.cuda(), zeros2.cuda())
+    dy2 = torch.randn(M, N, device="cuda", generator=g).to(torch.bfloat16)
+    pair = ops.a16w4_dx_pair(dy, w, dy2, w2, (N, K))
+    want = ref + dy2.float() @ ops.a16w4_dequant(*w2, (N, K)).float()
+    assert ((pair.float() - want).norm() / want.norm()).item() < TOL
     w8 = torch.randint(-128, 128, (N, K), device="cuda", generator=g, dtype=torch.int8)
     qs = (torch.rand(N, device="cuda", generator=g) * 0.01 + 1e-3).to(torch.bfloat16)
     dx8 = ops.a8w8_dx(dy, w8, qs)
