@@ -203,6 +203,55 @@ def test_8bit_accumulation_through_the_gemm_epilogue_equals_the_separate_pass(Q,
         cls.noise_seed, cls._noise_offset = saved
 
 
+def test_fused_mlp_block_with_8bit_gradient_accumulators(Q, ops):
+    """A QuantLlamaMLP of three gbit = 8 layers: the fused backward hands its three weight-gradient products to the
+    layers' hooks (down, up, gate), the second micro-batch through the GEMM epilogue. Codes and scales equal, bit
+    for bit, the separate passes on the same products with the same noise stream."""
+    from latentq_llm_amd.fused_mlp import QuantLlamaMLP
+    hid, ffn, M = 256, 384, 128
+
+    def layer(n, k, seed):
+        _, packed, scales, zeros = make_w4(n, k, seed)
+        m = Q.QLinearA16W4(k, n, bias=False, lbit=0, gbit=8)
+        m.zeros.data, m.scales.data, m.wshape = zeros.clone(), scales.clone(), [n, k]
+        m.weight.set_value(packed, [m.scales, m.zeros, m.wshape])
+        m = m.bfloat16().cuda()
+        m.to("cuda")
+        m.weight.requires_grad = True
+        m.add_hook()
+        return m
+
+    gate, up, down = layer(ffn, hid, 41), layer(ffn, hid, 42), layer(hid, ffn, 43)
+    mlp = QuantLlamaMLP(gate, down, up)
+    x = randn_bf16((M, hid), 44).cuda().requires_grad_(True)
+    dys = [randn_bf16((M, hid), 45 + i).cuda() for i in range(2)]
+    cls = Q.GradientQTensor
+    saved = (cls.noise_seed, cls._noise_offset)
+    try:
+        cls.noise_seed, cls._noise_offset = 777, 5000
+        for dy in dys:
+            mlp(x).backward(dy)
+        assert len(Q.dict_temp) == 0
+        for m in (gate, up, down):
+            assert isinstance(m.weight.grad, cls) and m.weight.grad.acc_ite == 2
+        # the same products through the separate passes, in the hooks' order
+        w4 = lambda m: (m.weight.data, m.scales, m.zeros)
+        refs = {id(m): cls([m.wshape[0], m.wshape[1]], bit=8) for m in (gate, up, down)}
+        cls.noise_seed, cls._noise_offset = 777, 5000
+        xd = x.detach()
+        h, g, u = ops.a16w4_gate_up_silu(xd, w4(gate), w4(up), (ffn, hid), save=True)
+        for i, dy in enumerate(dys):
+            dg, du = ops.a16w4_dx_silu_bwd(dy, *w4(down), (hid, ffn), g, u)
+            for m, dyl, xin in ((down, dy, h), (up, du, xd), (gate, dg, xd)):
+                dw = ops.weight_grad(dyl, xin)
+                (refs[id(m)].set_value if i == 0 else refs[id(m)].add_)(dw)
+        for m in (gate, up, down):
+            assert torch.equal(m.weight.grad.scale, refs[id(m)].scale)
+            assert torch.equal(m.weight.grad.qdata, refs[id(m)].qdata)
+    finally:
+        cls.noise_seed, cls._noise_offset = saved
+
+
 def test_noise_seed_follows_torch_manual_seed(Q):
     cls = Q.GradientQTensor
     saved = (cls.noise_seed, cls._noise_offset)
