@@ -327,11 +327,26 @@ def bench_adam8(device):
     curve = (2, 0.1875, 3, 0.375, 3)
     sec_step = event_time(lambda: ops.adam8_latent_w4_step(grad, codes, res, scales.view(-1), zeros.view(-1), (N, K), s1, s2,
                                                            sc1, mx1, sc2, mx2, curve, curve, 0.9, 0.95, 1e-8, 1e-3), 20)
-    step_bytes = 6 * n + 32 * nblk + 4 * n // 128
+    # per element: 2 B of gradient, 2 + 2 B of moments in and out, 0.5 + 0.5 B of codes and of residual in and out
+    step_bytes = 8 * n + 32 * nblk + 4 * n // 128
+    # the same for an 8-bit-weight layer (int8 codes, one scale per row): the single kernel against its three passes
+    w8 = torch.randint(-128, 128, (N, K), device=device, dtype=torch.int8)
+    qs = ((torch.randn(N, device=device) * 0.01).abs() + 1e-3).to(torch.bfloat16)
+    sec_w8 = event_time(lambda: ops.adam8_latent_w8_step(grad, w8, res, qs, s1, s2, sc1, mx1, sc2, mx2, curve, curve,
+                                                         0.9, 0.95, 1e-8, 1e-3), 20)
+
+    def three_passes():
+        lat = ops.latent_w8_reconstruct(w8, qs, res, *curve)
+        ops.adam8_update(grad, s1, s2, sc1, mx1, sc2, mx2, 0.9, 0.95, 1e-8, 1e-3, param=lat.view(-1))
+        ops.latent_w8_requant(lat, qs, res, *curve)
+    sec_w8_3 = event_time(three_passes, 20)
+    w8_bytes = 9 * n + 32 * nblk + 2 * N  # as above with 1 + 1 B of codes
     return {"elements": n, "block": block, "bytes": nbytes, "us": sec * 1e6, "GB/s": nbytes / sec / 1e9,
             "frac_hbm": nbytes / sec / PEAK_HBM, "tensor_op_chain_us": sec_chain * 1e6,
             "latent_w4_step": {"bytes": step_bytes, "us": sec_step * 1e6, "GB/s": step_bytes / sec_step / 1e9,
-                               "frac_hbm": step_bytes / sec_step / PEAK_HBM}}
+                               "frac_hbm": step_bytes / sec_step / PEAK_HBM},
+            "latent_w8_step": {"bytes": w8_bytes, "us": sec_w8 * 1e6, "GB/s": w8_bytes / sec_w8 / 1e9,
+                               "frac_hbm": w8_bytes / sec_w8 / PEAK_HBM, "three_passes_us": sec_w8_3 * 1e6}}
 
 
 def bench_dw(device):
@@ -618,6 +633,9 @@ def profile_target(device, which, launches=10):
             o.adam8_update(grad, s1, s2, q[0], q[1], q[2], q[3], 0.9, 0.95, 1e-8, 1e-3, param=param)
             o.adam8_latent_w4_step(grad, p, res, s.view(-1), z.view(-1), (N, K), s1, s2, q[0], q[1], q[2], q[3], curve, curve,
                                    0.9, 0.95, 1e-8, 1e-3)
+            w8 = torch.randint(-128, 128, (N, K), device=device, dtype=torch.int8)
+            qs = ((torch.randn(N, device=device) * 0.01).abs() + 1e-3).to(torch.bfloat16)
+            o.adam8_latent_w8_step(grad, w8, res, qs, s1, s2, q[0], q[1], q[2], q[3], curve, curve, 0.9, 0.95, 1e-8, 1e-3)
     elif which == "gemv":
         for (N, K) in [(4096, 4096), (11008, 4096), (4096, 11008)]:
             for M in (1, 4, 16):

@@ -369,6 +369,16 @@ int lq_adam8_latent_w4_step(const void *grad, void *codes, int32_t *residual, co
                             int dk3, int qk1, float qb1, int qk2, float qb2, int qk3, double beta1, double beta2,
                             double eps, double step_size, void *stream);
 
+/* The same for an 8-bit-weight layer (QLinearA8W8 with lbit = 4): the parameter is rebuilt from the int8 codes, the
+ * per-row bf16 scales and the residual words exactly as lq_latent_w8_reconstruct does
+ * (ResidualTensor.add((p.data * p.qparam).to(dtype)), utils/quant.py:826-837, 1069-1070), updated, and re-quantised
+ * exactly as lq_latent_w8_requant does (Qfunc_8bit_res, utils/quant.py:88-103). codes: int8 [N, K], 8-byte aligned,
+ * K % 8 == 0; qscales: bf16 [N]; residual: int32 [N*K/8]; the rest as lq_adam8_latent_w4_step with n = N*K. */
+int lq_adam8_latent_w8_step(const void *grad, int8_t *codes, int32_t *residual, const void *qscales, uint8_t *state1,
+                            uint8_t *state2, float *scale1, float *max1, float *scale2, float *max2, int64_t N, int64_t K,
+                            int block_elems, int dk1, float db1, int dk2, float db2, int dk3, int qk1, float qb1, int qk2,
+                            float qb2, int qk3, double beta1, double beta2, double eps, double step_size, void *stream);
+
 /* ---------------------------------------------------------------------------
  * 8-bit gradient accumulator: GradientQTensor.find_param / quant / dequant / set_value / add_ of
  * the reference (utils/quant.py:856-898) for bit = 8 as one pass over the bf16 weight gradient,

@@ -60,6 +60,8 @@ SIGNATURES = {
     "lq_adam8_update": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _f64, _f64, _f64, _f64, _vp],
     "lq_adam8_latent_w4_step": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32,
                                 _i32, _f32, _i32, _f32, _i32, _i32, _f32, _i32, _f32, _i32, _f64, _f64, _f64, _f64, _vp],
+    "lq_adam8_latent_w8_step": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32,
+                                _i32, _f32, _i32, _f32, _i32, _i32, _f32, _i32, _f32, _i32, _f64, _f64, _f64, _f64, _vp],
 }
 
 _lib = None

@@ -43,7 +43,13 @@ struct Adam8Params {
     unsigned *codes, *residual;
     const unsigned short *wscales, *wzeros;  // per group of 128 elements
     CodecParams dequant_curve, quant_curve;
+    // latent mode of an 8-bit-weight layer: int8 codes (8 per thread), one bf16 scale per row of K elements
+    u32x2_t *codes8;
+    const unsigned short *qscales;
+    long long threads_per_row;  // K / 8
 };
+
+enum { LATENT_NONE = 0, LATENT_W4 = 1, LATENT_W8 = 2 };
 
 // minimum and maximum over the W threads that share a block (W = 16: one 16-lane row of the
 // wave, by cross-lane shuffles; W = 256: the whole workgroup, through LDS)
@@ -145,12 +151,27 @@ __device__ __forceinline__ void requant8(const float (&out)[8], float ws, float 
     }
 }
 
-template <int BS, bool LATENT>
+// The same for an 8-bit-weight layer: 8 code bytes and one residual word per thread
+template <bool kFast>
+__device__ __forceinline__ void requant8_w8(const float (&out)[8], float ws, float wr, const CodecParams pq, u32x2_t &cnew,
+                                            unsigned &rnew) {
+    unsigned cw[2] = {0u, 0u};
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        unsigned nib, byte;
+        lq_latent_w8_requant_elem<kFast>(out[k], ws, wr, pq, nib, byte);
+        rnew = (rnew << 4) | nib;
+        cw[k >> 2] |= byte << (8 * (k & 3));
+    }
+    cnew = u32x2_t{cw[0], cw[1]};
+}
+
+template <int BS, int LATENT>
 __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
     constexpr int W = BS / 8;  // threads per block of the moments
     __shared__ float red[4][2];
     __shared__ float vtab[16];  // latent mode: dequantised values of the 16 residual nibbles
-    if constexpr (LATENT) {
+    if constexpr (LATENT != LATENT_NONE) {
         lq_latent_fill_value_table(vtab, a.dequant_curve);
         __syncthreads();
     }
@@ -164,11 +185,16 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
     u32x4_t p4 = {0u, 0u, 0u, 0u};
     unsigned cword = 0, rword = 0;
     float ws = 0.0f, wz = 0.0f;
-    if constexpr (LATENT) {
+    u32x2_t c8 = {0u, 0u};
+    if constexpr (LATENT == LATENT_W4) {
         cword = a.codes[Tc];
         rword = a.residual[Tc];
         ws = lq_bf16_bits_to_f32(a.wscales[Tc >> 4]);
         wz = lq_bf16_bits_to_f32(a.wzeros[Tc >> 4]);
+    } else if constexpr (LATENT == LATENT_W8) {
+        c8 = a.codes8[Tc];
+        rword = a.residual[Tc];
+        ws = lq_bf16_bits_to_f32(a.qscales[Tc / a.threads_per_row]);
     } else if (a.param) {
         p4 = a.param[Tc];
     }
@@ -209,7 +235,7 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
         d[k] = bf16r(d[k] + a.eps);
         const float r = __builtin_amdgcn_rcpf(d[k]);
         const float q0 = m[k] * r;
-        if (!LATENT && !a.param) {
+        if (LATENT == LATENT_NONE && !a.param) {
             // Only bf16(m / d) is stored here, and the quotient of two bf16 numbers never comes closer
             // than 2^-17 (relative) to the midpoint of two bf16 values (256 m_a = (2j+1) m_b has no
             // solution with 8-bit significands), so any fp32 quotient within a few ulps rounds to the
@@ -233,8 +259,11 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
     }
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-        if constexpr (LATENT) {
+        if constexpr (LATENT == LATENT_W4) {
             const float p = bf16r(lq_latent_value(lq_code(cword, k), vtab[(rword >> (28 - 4 * k)) & 0xFu], ws, wz));
+            out[k] = bf16r(fmaf(a.neg_step, ratio[k], p));
+        } else if constexpr (LATENT == LATENT_W8) {
+            const float p = bf16r(lq_latent_w8_value(c8[k >> 2] >> (8 * (k & 3)), vtab[(rword >> (28 - 4 * k)) & 0xFu], ws));
             out[k] = bf16r(fmaf(a.neg_step, ratio[k], p));
         } else if (a.param) {
             const float p = (k & 1) ? lq_bf16_hi(p4[k >> 1]) : lq_bf16_lo(p4[k >> 1]);
@@ -243,7 +272,7 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
             out[k] = ratio[k];
         }
     }
-    if constexpr (LATENT) {
+    if constexpr (LATENT == LATENT_W4) {
         const bool fast = (ws >= 0x1p-40f) && (ws <= 0x1p40f);
         const float wr = 1.0f / ws;
         unsigned cnew = 0, rnew = 0;
@@ -251,6 +280,17 @@ __global__ __launch_bounds__(256) void adam8_update_kernel(Adam8Params a) {
         else requant8<false>(out, ws, wz, wr, a.quant_curve, cnew, rnew);
         if (live) {
             a.codes[T] = cnew;
+            a.residual[T] = rnew;
+        }
+    } else if constexpr (LATENT == LATENT_W8) {
+        const bool fast = (fabsf(ws) >= 0x1p-40f) && (fabsf(ws) <= 0x1p40f);
+        const float wr = 1.0f / ws;
+        u32x2_t cnew;
+        unsigned rnew = 0;
+        if (fast) requant8_w8<true>(out, ws, wr, a.quant_curve, cnew, rnew);
+        else requant8_w8<false>(out, ws, wr, a.quant_curve, cnew, rnew);
+        if (live) {
+            a.codes8[T] = cnew;
             a.residual[T] = rnew;
         }
     } else if (live) {
@@ -323,9 +363,9 @@ extern "C" int lq_adam8_update(const void *grad, void *param_or_null, void *dire
     adam8_scalars(a, beta1, beta2, eps, step_size);
     const unsigned blocks = (unsigned)((a.n_threads + 255) / 256);
     if (block_elems == 2048)
-        hipLaunchKernelGGL((adam8_update_kernel<2048, false>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+        hipLaunchKernelGGL((adam8_update_kernel<2048, LATENT_NONE>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
     else
-        hipLaunchKernelGGL((adam8_update_kernel<128, false>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+        hipLaunchKernelGGL((adam8_update_kernel<128, LATENT_NONE>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
     return lq_check_launch("lq_adam8_update");
 }
 
@@ -358,8 +398,42 @@ extern "C" int lq_adam8_latent_w4_step(const void *grad, void *codes, int32_t *r
     adam8_scalars(a, beta1, beta2, eps, step_size);
     const unsigned blocks = (unsigned)((a.n_threads + 255) / 256);
     if (block_elems == 2048)
-        hipLaunchKernelGGL((adam8_update_kernel<2048, true>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+        hipLaunchKernelGGL((adam8_update_kernel<2048, LATENT_W4>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
     else
-        hipLaunchKernelGGL((adam8_update_kernel<128, true>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+        hipLaunchKernelGGL((adam8_update_kernel<128, LATENT_W4>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
     return lq_check_launch("lq_adam8_latent_w4_step");
+}
+
+extern "C" int lq_adam8_latent_w8_step(const void *grad, int8_t *codes, int32_t *residual, const void *qscales, uint8_t *state1,
+                                       uint8_t *state2, float *scale1, float *max1, float *scale2, float *max2, int64_t N,
+                                       int64_t K, int block_elems, int dk1, float db1, int dk2, float db2, int dk3, int qk1,
+                                       float qb1, int qk2, float qb2, int qk3, double beta1, double beta2, double eps,
+                                       double step_size, void *stream) {
+    LQ_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "lq_adam8_latent_w8_step: need N > 0, K a positive multiple of 8");
+    const int64_t n = N * K;
+    int rc = adam8_check("lq_adam8_latent_w8_step", grad, state1, state2, scale1, max1, scale2, max2, n, block_elems);
+    if (rc) return rc;
+    LQ_REQUIRE(codes && residual && qscales, "lq_adam8_latent_w8_step: null pointer argument");
+    LQ_REQUIRE(lq_aligned(codes, 8) && lq_aligned(residual, 4) && lq_aligned(qscales, 2),
+               "lq_adam8_latent_w8_step: codes must be 8-byte, residual 4-byte aligned");
+    LQ_REQUIRE(dk1 > 0 && dk2 > 0 && dk3 > 0 && db1 > 0.0f && db2 > db1 && db2 < 0.5f && qk1 > 0 && qk2 > 0 && qk3 > 0 &&
+                   qb1 > 0.0f && qb2 > qb1 && qb2 < 0.5f,
+               "lq_adam8_latent_w8_step: need k1,k2,k3 > 0 and 0 < b1 < b2 < 0.5 for both curves");
+    Adam8Params a = {};
+    a.grad = (const u32x4_t *)grad;
+    a.state1 = (u32x2_t *)state1; a.state2 = (u32x2_t *)state2;
+    a.scale1 = scale1; a.max1 = max1; a.scale2 = scale2; a.max2 = max2;
+    a.n_threads = n / 8;
+    a.codes8 = (u32x2_t *)codes; a.residual = (unsigned *)residual;
+    a.qscales = (const unsigned short *)qscales;
+    a.threads_per_row = K / 8;
+    a.dequant_curve = lq_codec_dequant_params(dk1, db1, dk2, db2, dk3);
+    a.quant_curve = lq_codec_quant_params(qk1, qb1, qk2, qb2, qk3);
+    adam8_scalars(a, beta1, beta2, eps, step_size);
+    const unsigned blocks = (unsigned)((a.n_threads + 255) / 256);
+    if (block_elems == 2048)
+        hipLaunchKernelGGL((adam8_update_kernel<2048, LATENT_W8>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+    else
+        hipLaunchKernelGGL((adam8_update_kernel<128, LATENT_W8>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+    return lq_check_launch("lq_adam8_latent_w8_step");
 }

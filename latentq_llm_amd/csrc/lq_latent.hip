@@ -113,10 +113,7 @@ __global__ __launch_bounds__(256) void latent_w8_reconstruct_kernel(const u32x4_
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             const int e = 8 * i + k;
-            const float q = (float)(int)(signed char)((cw[e >> 2] >> (8 * (e & 3))) & 0xFFu);
-            const float w = lq_bf16r(q * s);
-            const float r = lq_bf16r(vtab[(rw[i] >> (28 - 4 * k)) & 0xFu] * s);
-            v[k] = r + w;
+            v[k] = lq_latent_w8_value(cw[e >> 2] >> (8 * (e & 3)), vtab[(rw[i] >> (28 - 4 * k)) & 0xFu], s);
         }
         latent[L * 2 + i] = u32x4_t{lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3]), lq_pack_bf16(v[4], v[5]),
                                     lq_pack_bf16(v[6], v[7])};
@@ -133,18 +130,11 @@ __device__ __forceinline__ void requant_w8_thread(const u32x4_t (&in)[2], float 
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             const float t = (k & 1) ? lq_bf16_hi(in[i][k >> 1]) : lq_bf16_lo(in[i][k >> 1]);
-            const float quo = kFast ? t * r : t / s;
-            const float Z = lq_bf16r(quo);
-            const float q = rintf(Z);       // round half to even, as torch.round
-            const float f = lq_bf16r(Z - q);
-            bool carry;
-            const unsigned nib = nibble_of(level_3fold(f, p), carry);
-            // q + carry is an integer (bf16 holds it exactly wherever the clamp does not decide); NaN -> 0
-            const float c = q + (carry ? 1.0f : 0.0f);
-            const float cc = c == c ? __builtin_amdgcn_fmed3f(c, -128.0f, 127.0f) : 0.0f;
+            unsigned nib, byte;
+            lq_latent_w8_requant_elem<kFast>(t, s, r, p, nib, byte);
             rword = (rword << 4) | nib;
             const int e = 8 * i + k;
-            cw[e >> 2] |= ((unsigned)(int)cc & 0xFFu) << (8 * (e & 3));
+            cw[e >> 2] |= byte << (8 * (e & 3));
         }
         rout[i] = rword;
     }

@@ -44,3 +44,28 @@ __device__ __forceinline__ void lq_latent_requant_elem(float t, float s, float z
     const float c = __builtin_amdgcn_fmed3f(fmaxf(q + (carry ? 1.0f : 0.0f), 0.0f), 0.0f, 15.0f);
     code = (unsigned)c;
 }
+
+// ---- 8-bit weights (int8 codes, one bf16 scale per row; utils/quant.py:88-103, 826-837, 1069-1070) ----
+// latent = bf16(bf16(value(nibble)) * s) + bf16(q * s); the caller applies the last rounding
+__device__ __forceinline__ float lq_latent_w8_value(unsigned byte, float value_bf16, float s) {
+    const float q = (float)(int)(signed char)(byte & 0xFFu);
+    return lq_bf16r(value_bf16 * s) + lq_bf16r(q * s);
+}
+
+// One element of the 8-bit re-quantiser: Z = bf16(t / s), q = rint(Z), residual nibble and carry from
+// bf16(Z - q), code byte = clamp(q + carry, -128, 127) (NaN -> 0). kFast: the quotient as the product with
+// r = 1 / s, valid for 2^-40 <= |s| <= 2^40 (see lq_latent_requant_elem).
+template <bool kFast>
+__device__ __forceinline__ void lq_latent_w8_requant_elem(float t, float s, float r, const CodecParams &pq, unsigned &nib,
+                                                          unsigned &byte) {
+    const float quo = kFast ? t * r : t / s;
+    const float Z = lq_bf16r(quo);
+    const float q = rintf(Z);  // round half to even, as torch.round
+    const float f = lq_bf16r(Z - q);
+    bool carry;
+    nib = nibble_of(level_3fold(f, pq), carry);
+    // q + carry is an integer (bf16 holds it exactly wherever the clamp does not decide); NaN -> 0
+    const float c = q + (carry ? 1.0f : 0.0f);
+    const float cc = c == c ? __builtin_amdgcn_fmed3f(c, -128.0f, 127.0f) : 0.0f;
+    byte = (unsigned)(int)cc & 0xFFu;
+}

@@ -478,6 +478,47 @@ def adam8_latent_w4_step(grad, codes, residual_int, scales, zeros, shape, state1
     return codes
 
 
+def adam8_latent_w8_step(grad, codes, residual_int, qscales, state1, state2, scale1, max1, scale2, max2,
+                         dequant_curve, quant_curve, beta1, beta2, eps, step_size):
+    """The Adam step of an 8-bit-weight layer in lbit = 4 mode in one pass: codes (int8 [N, K]), residual_int
+    (int32[N*K/8]) and the uint8 moments with their block parameters are all updated in place; qscales bf16 [N].
+    The curves are (k1, b1, k2, b2, k3) tuples: the one the residual was stored with and the current one."""
+    _chk(grad, torch.bfloat16, "grad")
+    _chk(codes, torch.int8, "codes")
+    if codes.dim() != 2 or codes.shape[1] % 8:
+        raise ValueError("codes must be int8 [N, K] with K a multiple of 8")
+    N, K = codes.shape
+    n = N * K
+    if grad.numel() != n:
+        raise ValueError("grad must hold N*K elements")
+    _chk(qscales, torch.bfloat16, "qscales")
+    if qscales.numel() != N:
+        raise ValueError("qscales must hold one value per row")
+    _chk(residual_int, torch.int32, "residual_int")
+    if residual_int.numel() != n // 8:
+        raise ValueError("residual_int must hold N*K/8 words")
+    for t, name in ((state1, "state1"), (state2, "state2")):
+        _chk(t, torch.uint8, name)
+        if t.numel() != n:
+            raise ValueError(f"{name} must hold N*K elements")
+    nblk = scale1.numel()
+    if nblk == 0 or n % nblk:
+        raise ValueError("the number of blocks must divide the number of elements")
+    for t, name in ((scale1, "scale1"), (max1, "max1"), (scale2, "scale2"), (max2, "max2")):
+        _chk(t, torch.float32, name)
+        if t.numel() != nblk:
+            raise ValueError(f"{name} must hold one value per block")
+    d, q = dequant_curve, quant_curve
+    with torch.cuda.device(grad.device):
+        _C.call("lq_adam8_latent_w8_step", grad.data_ptr(), codes.data_ptr(), residual_int.data_ptr(), qscales.data_ptr(),
+                state1.data_ptr(), state2.data_ptr(), scale1.data_ptr(), max1.data_ptr(), scale2.data_ptr(),
+                max2.data_ptr(), N, K, n // nblk,
+                int(d[0]), float(d[1]), int(d[2]), float(d[3]), int(d[4]),
+                int(q[0]), float(q[1]), int(q[2]), float(q[3]), int(q[4]),
+                float(beta1), float(beta2), float(eps), float(step_size), _stream(grad))
+    return codes
+
+
 def gradq8_quant(dw, q, scale, accumulate: bool, noise=None, seed: int = 0, offset: int = 0):
     """The 8-bit gradient accumulator in one pass (lq_gradq8_quant): dw bf16 [N, K]; q int8 [N, K] and
     scale bf16 [N, 1] are updated in place (scale only when ``accumulate`` is False). ``noise`` is an

@@ -1180,9 +1180,32 @@ class MyAdam(torch.optim.Adam):
         back to codes + residual) as one kernel, when every piece is in the form the kernel takes;
         returns False to let the separate passes run."""
         r = p.residual
-        if not (p.wbit == 4 and isinstance(r, ResidualTensor) and not r.init and p.data.is_cuda
+        if not (p.wbit in (4, 8) and isinstance(r, ResidualTensor) and not r.init and p.data.is_cuda
                 and p.data.is_contiguous() and r.residual_int.is_cuda and r.residual_int.is_contiguous()):
             return False
+        moments = (state["state1"], state["state2"], state["qmap1"], state["absmax1"], state["qmap2"], state["absmax2"])
+        if p.wbit == 8:
+            # 8-bit weights: int8 codes [N, K], one bf16 scale per row (the conditions of _latent and Qfunc_8bit_res)
+            qs = p.qparam
+            if not (p.data.dtype == torch.int8 and p.data.dim() == 2 and p.data.shape[1] % 16 == 0 and torch.is_tensor(qs)
+                    and qs.dtype == torch.bfloat16 and qs.is_contiguous() and tuple(qs.shape) == (p.data.shape[0], 1)
+                    and r.weight_scale is not None and r.weight_scale.data_ptr() == qs.data_ptr()):
+                return False
+            beta1, beta2 = config["betas"]
+            state["step"] += 1
+            step_size = config["lr"] * math.sqrt(1 - beta2 ** state["step"]) / (1 - beta1 ** state["step"])
+            p1, y1, p2, y2 = three_fold_curve_4bit(r.lock_mu)
+            q1, z1, q2, z2 = three_fold_curve_4bit(r.mu)
+            ops.adam8_latent_w8_step(grad, p.data, r.residual_int.view(-1), qs.view(-1), *moments,
+                                     (p1, y1, p2 - p1, y2, 8 - p2), (q1, z1, q2 - q1, z2, 8 - q2), beta1, beta2,
+                                     group["eps"], step_size)
+            r.weight_scale = qs
+            r.lock_mu = r.mu
+            if isinstance(p.grad, GradientQTensor):
+                p.grad.zero()
+            else:
+                p.grad = None
+            return True
         scales, zeros, shape = _flat_qparam(p.qparam)
         if not (scales.dtype == torch.bfloat16 and zeros.dtype == torch.bfloat16 and scales.is_contiguous()
                 and zeros.is_contiguous() and r.weight_scale is not None and r.weight_scale.dtype == torch.bfloat16
@@ -1193,8 +1216,7 @@ class MyAdam(torch.optim.Adam):
         step_size = config["lr"] * math.sqrt(1 - beta2 ** state["step"]) / (1 - beta1 ** state["step"])
         p1, y1, p2, y2 = three_fold_curve_4bit(r.lock_mu)
         q1, z1, q2, z2 = three_fold_curve_4bit(r.mu)
-        ops.adam8_latent_w4_step(grad, p.data, r.residual_int.view(-1), scales, zeros, tuple(shape), state["state1"],
-                                 state["state2"], state["qmap1"], state["absmax1"], state["qmap2"], state["absmax2"],
+        ops.adam8_latent_w4_step(grad, p.data, r.residual_int.view(-1), scales, zeros, tuple(shape), *moments,
                                  (p1, y1, p2 - p1, y2, 8 - p2), (q1, z1, q2 - q1, z2, 8 - q2), beta1, beta2,
                                  group["eps"], step_size)
         r.weight_scale = scales.contiguous().reshape(-1, 1)

@@ -204,3 +204,96 @@ def test_single_kernel_latent_step_equals_the_three_passes(ops, N, K, block):
         for name in a:
             assert torch.equal(a[name].view(-1), b[name].view(-1)), f"step {step}: {name} differs"
     assert not torch.equal(b["codes"].cpu(), packed)
+
+
+@pytest.mark.parametrize("N,K,block", [(64, 2048, 2048), (200, 320, 128), (1024, 4096, 2048)])
+def test_single_kernel_w8_latent_step_equals_the_three_passes(ops, N, K, block):
+    """lq_adam8_latent_w8_step against lq_latent_w8_reconstruct -> lq_adam8_update -> lq_latent_w8_requant on an
+    8-bit-weight layer (scales of both signs, one outside the range of the reciprocal product), with different curves
+    for the stored residual and for the new one, over several steps: codes, residual words, moments and block
+    parameters identical."""
+    from latentq_llm_amd import quant as q
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(N + K)
+    n = N * K
+    nblk = n // block
+    codes = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+    qs = ((torch.randn(N, generator=g) * 0.01).abs() + 1e-3).to(torch.bfloat16)
+    qs[3] = -qs[3]
+    qs[5] = 2.0 ** -50
+    qs = qs.to(dev)
+    res = torch.randint(-2**31, 2**31 - 1, (n // 8,), generator=g, dtype=torch.int64).to(torch.int32).to(dev)
+    a = {"codes": codes.clone().to(dev), "res": res.clone(), **fresh_state(n, nblk, dev)}
+    b = {"codes": codes.clone().to(dev), "res": res.clone(), **fresh_state(n, nblk, dev)}
+
+    def curve(mu):
+        p1, y1, p2, y2 = q.three_fold_curve_4bit(mu)
+        return (p1, y1, p2 - p1, y2, 8 - p2)
+    curves = [curve(0), curve(1), curve(1), curve(2), curve(0)]
+    for step in range(1, 5):
+        grad = (torch.randn(n, generator=g) * 10.0 ** torch.randint(-5, -1, (n,), generator=g).float()).to(torch.bfloat16).to(dev)
+        step_size = 2e-3 * math.sqrt(1 - 0.95 ** step) / (1 - 0.9 ** step)
+        dq, qq = curves[step - 1], curves[step]
+        latent = ops.latent_w8_reconstruct(a["codes"], qs, a["res"], *dq)
+        ops.adam8_update(grad, a["state1"], a["state2"], a["qmap1"], a["absmax1"], a["qmap2"], a["absmax2"],
+                         0.9, 0.95, 1e-8, step_size, param=latent.view(-1))
+        a["codes"] = ops.latent_w8_requant(latent, qs, a["res"], *qq)
+        ops.adam8_latent_w8_step(grad, b["codes"], b["res"], qs, b["state1"], b["state2"], b["qmap1"], b["absmax1"],
+                                 b["qmap2"], b["absmax2"], dq, qq, 0.9, 0.95, 1e-8, step_size)
+        torch.cuda.synchronize()
+        for name in a:
+            assert torch.equal(a[name].view(-1), b[name].view(-1)), f"step {step}: {name} differs"
+    assert not torch.equal(b["codes"].cpu(), codes)
+
+
+def _run_w8_module_steps(Q, fused, steps=5):
+    from tests.util import randn_bf16
+    Q.FUSED_ADAM8 = fused
+    Q.FUSED_LATENT = fused
+    torch.manual_seed(0)
+    N, K = 256, 512
+    g = torch.Generator().manual_seed(5)
+    w8 = torch.randint(-120, 121, (N, K), generator=g, dtype=torch.int8)
+    qs = ((torch.randn(N, 1, generator=g) * 0.01).abs() + 2e-3).to(torch.bfloat16)
+    layer = Q.QLinearA8W8(K, N, bias=False, lbit=4, gbit=16)
+    layer.qscales.data = qs.clone()
+    layer.weight.set_value(w8, layer.qscales)
+    layer = layer.bfloat16().cuda()
+    layer.to("cuda")
+    layer.weight.requires_grad = True
+    layer.add_hook()
+    opt = Q.MyAdam([{"params": [layer.weight]}], lr=2e-3, betas=(0.9, 0.95), obit=8, mu_updata_f=20)
+    x = randn_bf16((64, K), 11).cuda().requires_grad_(True)
+    tgt = randn_bf16((64, N), 12).cuda()
+    for _ in range(steps):
+        y = layer(x)
+        ((y.float() - tgt.float()) ** 2).mean().backward()
+        opt.step()
+    st = opt.state[layer.weight]
+    assert st["state1"].dtype == torch.uint8
+    return (layer.weight.data.clone().cpu(), layer.weight.residual.residual_int.clone().cpu(), st["state1"].clone().cpu(),
+            st["state2"].clone().cpu(), st["qmap1"].clone().cpu(), st["absmax1"].clone().cpu(), st["qmap2"].clone().cpu(),
+            st["absmax2"].clone().cpu()), w8
+
+
+def test_optimizer_steps_on_8bit_weights_with_uint8_moments(ops, monkeypatch):
+    """Whole optimizer steps of an 8-bit-weight layer in lbit = 4 mode with uint8 moments: the single-kernel step
+    runs from the second step on (the first has no stored residual yet), and codes, residual words, moments and block
+    parameters equal those of the chain of tensor operations."""
+    from latentq_llm_amd import ops as O
+    from latentq_llm_amd import quant as Q
+    calls = {"step": 0}
+    real_step = O.adam8_latent_w8_step
+    monkeypatch.setattr(O, "adam8_latent_w8_step",
+                        lambda *a, **k: (calls.__setitem__("step", calls["step"] + 1), real_step(*a, **k))[1])
+    try:
+        a, w8 = _run_w8_module_steps(Q, True)
+        assert calls == {"step": 4}
+        b, _ = _run_w8_module_steps(Q, False)
+        assert calls == {"step": 4}
+    finally:
+        Q.FUSED_ADAM8 = True
+        Q.FUSED_LATENT = True
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    assert not torch.equal(a[0], w8)
