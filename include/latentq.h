@@ -263,6 +263,12 @@ int lq_act_quant_i8_dynamic(const void *x, int8_t *x8, float *sx, float *work, i
  * x: bf16[M,K], 16-byte aligned, K % 8 == 0; x8: int8[M,K]; sx: fp32[M]. */
 int lq_act_quant_i8_per_token(const void *x, int8_t *x8, float *sx, int64_t M, int64_t K, void *stream);
 
+/* The quantised activations back as bf16 for the backward pass: out[m,k] = bf16(x8[m,k] * bf16(s)), s = scale[m]
+ * (per_token != 0) or scale[0]: the values of `x8.to(dtype) * scale.to(dtype)` that the training Function's backward
+ * multiplies dY^T with (utils/quant.py:277-280) as one pass instead of two tensor operations. x8: int8 [M,K], 16-byte
+ * aligned, K % 16 == 0; scale: fp32 [M] or [1]; out: bf16 [M,K], 16-byte aligned. */
+int lq_act_dequant_i8(const int8_t *x8, const float *scale, int per_token, void *out, int64_t M, int64_t K, void *stream);
+
 /* Per-channel int8 re-quantiser of the latent weight of an 8-bit-weight layer: the reference's
  * Qfunc_8bit_res (utils/quant.py:88-103) for a latent kept as a plain tensor (lbit 0, 16, 32), called
  * from MyAdam.update_step (:1141):

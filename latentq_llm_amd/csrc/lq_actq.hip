@@ -217,7 +217,44 @@ __global__ __launch_bounds__(256) void act_quant_token_kernel(const unsigned sho
     }
 }
 
+// The way back, for the backward pass: out = bf16(x8 * bf16(s)) with s = scale[m] (per token) or scale[0]; the values of
+// `x8.to(dtype) * s.to(dtype)`. 16 elements per thread (one row: K % 16 == 0).
+__global__ __launch_bounds__(256) void act_dequant_kernel(const u32x4_t *__restrict__ x8, const float *__restrict__ scale,
+                                                          u32x4_t *__restrict__ out, long long n_chunks, long long chunks_per_row,
+                                                          int per_token) {
+    const long long L = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (L >= n_chunks) return;
+    const float s = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(scale[per_token ? L / chunks_per_row : 0]));
+    const u32x4_t c = x8[L];
+    u32x4_t o[2];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        float v[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) v[b] = (float)(int)(signed char)((c[w] >> (8 * b)) & 0xFFu) * s;
+        o[w >> 1][2 * (w & 1)] = lq_pack_bf16(v[0], v[1]);
+        o[w >> 1][2 * (w & 1) + 1] = lq_pack_bf16(v[2], v[3]);
+    }
+    out[2 * L] = o[0];
+    out[2 * L + 1] = o[1];
+}
+
 }  // namespace
+
+extern "C" int lq_act_dequant_i8(const int8_t *x8, const float *scale, int per_token, void *out, int64_t M, int64_t K,
+                                 void *stream) {
+    LQ_REQUIRE(x8 && scale && out, "lq_act_dequant_i8: null pointer argument");
+    LQ_REQUIRE(M > 0 && K > 0 && K % 16 == 0 && M < (1ll << 31) && K < (1ll << 31),
+               "lq_act_dequant_i8: need M > 0 and K a positive multiple of 16 (M=%lld K=%lld)", (long long)M, (long long)K);
+    LQ_REQUIRE(lq_aligned(x8, 16) && lq_aligned(out, 16) && lq_aligned(scale, 4),
+               "lq_act_dequant_i8: x8 and out must be 16-byte aligned, scale 4-byte");
+    const long long n_chunks = M * K / 16;
+    const long long blocks = (n_chunks + 255) / 256;
+    LQ_REQUIRE(blocks <= 0x7FFFFFFFll, "lq_act_dequant_i8: tensor too large");
+    hipLaunchKernelGGL(act_dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const u32x4_t *)x8, scale,
+                       (u32x4_t *)out, n_chunks, (long long)(K / 16), per_token);
+    return lq_check_launch("lq_act_dequant_i8");
+}
 
 extern "C" int lq_act_quant_i8(const void *x, const float *clampv_dev, int8_t *x8, int64_t n, void *stream) {
     LQ_REQUIRE(x && clampv_dev && x8 && n >= 0, "lq_act_quant_i8: bad argument");

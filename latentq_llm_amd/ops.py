@@ -409,6 +409,30 @@ def act_quant_i8_per_token(x):
     return x8, sx
 
 
+def act_dequant_ok(x8, scale, per_token: bool) -> bool:
+    """Whether act_dequant_i8 takes these operands."""
+    return (x8.is_cuda and x8.dtype == torch.int8 and x8.dim() == 2 and x8.is_contiguous() and x8.numel() > 0
+            and x8.shape[1] % 16 == 0 and x8.data_ptr() % 16 == 0 and torch.is_tensor(scale) and scale.is_cuda
+            and scale.dtype == torch.float32 and scale.is_contiguous()
+            and scale.numel() == (x8.shape[0] if per_token else 1))
+
+
+def act_dequant_i8(x8, scale, per_token: bool):
+    """bf16(x8 * bf16(scale)) (lq_act_dequant_i8): scale fp32 [M] (per token) or one element; the values of
+    ``x8.to(torch.bfloat16) * scale.to(torch.bfloat16)``."""
+    _chk(x8, torch.int8, "x8")
+    _chk(scale, torch.float32, "scale")
+    if x8.dim() != 2 or x8.numel() == 0 or x8.shape[1] % 16:
+        raise ValueError("x8 must be a non-empty [M, K] matrix with K a multiple of 16")
+    M, K = x8.shape
+    if scale.numel() != (M if per_token else 1):
+        raise ValueError("scale must hold one value per row (per token) or one value")
+    out = torch.empty((M, K), dtype=torch.bfloat16, device=x8.device)
+    with torch.cuda.device(x8.device):
+        _C.call("lq_act_dequant_i8", x8.data_ptr(), scale.data_ptr(), 1 if per_token else 0, out.data_ptr(), M, K, _stream(x8))
+    return out
+
+
 def adam8_update(grad, state1, state2, scale1, max1, scale2, max2, beta1, beta2, eps, step_size, param=None,
                  direction=None):
     """One Adam step on uint8 block-wise moments (all updated in place). Either ``param`` (bf16, updated in

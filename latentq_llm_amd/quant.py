@@ -406,8 +406,12 @@ class QLinearFunctionA8W8_dynamic(torch.autograd.Function):
         x8, weight_d, bias = ctx.saved_tensors
         scale, qscales, per_token = ctx.save_qparamaw
         # x8 * (clampv / 127.): the quantiser left that bf16-valued alpha in scale[1]; per token: the row scales
-        s = scale.view(-1, 1) if per_token else scale[1]
-        input_f = x8.to(grad_output.dtype) * s.to(grad_output.dtype)
+        sv = scale.view(-1) if per_token else scale.view(-1)[1:2]
+        if grad_output.dtype == torch.bfloat16 and ops.act_dequant_ok(x8, sv, per_token):
+            input_f = ops.act_dequant_i8(x8, sv, per_token)  # the two tensor operations below as one pass
+        else:
+            s = scale.view(-1, 1) if per_token else scale[1]
+            input_f = x8.to(grad_output.dtype) * s.to(grad_output.dtype)
         return _a8w8_backward_common(ctx, grad_output, input_f, (weight_d, qscales), bias, detach_dw=True)
 
 

@@ -474,6 +474,32 @@ def test_act_quant_per_token_bit_exact(ops, co, shape):
     assert np.array_equal(g, want8), np.nonzero(g != want8)[0][:10]
 
 
+@pytest.mark.parametrize("shape", [(1, 16), (333, 80), (2048, 2048), (64, 8208)])
+def test_act_dequant_equals_the_two_tensor_operations(ops, shape):
+    """lq_act_dequant_i8 = x8.to(bf16) * scale.to(bf16), bit for bit, per token and per tensor (scales that are no
+    bf16 numbers, a zero, an infinity and a NaN among them)."""
+    M, K = shape
+    g = torch.Generator().manual_seed(M + K)
+    x8 = dev(torch.randint(-128, 128, shape, generator=g, dtype=torch.int8))
+    sx = (torch.rand(M, generator=g) * 0.1 + 1e-3)
+    if M > 4:
+        sx[0], sx[1], sx[2] = 0.0, float("inf"), float("nan")
+    sx = dev(sx)
+    want = x8.to(torch.bfloat16) * sx.view(-1, 1).to(torch.bfloat16)
+    got = ops.act_dequant_i8(x8, sx, True)
+    # NaNs (0 * inf, x * NaN) in the same places, whatever their payload bits; everything else bit for bit
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(got), nan)
+    diff = (got.view(torch.int16) != want.view(torch.int16)) & ~nan
+    assert int(diff.sum()) == 0, (int(diff.sum()), diff.nonzero()[:5].tolist())
+    s1 = dev(torch.tensor([3.0, 0.0123456, 7.0]))[1:2]   # an element inside a larger buffer
+    want = x8.to(torch.bfloat16) * s1[0].to(torch.bfloat16)
+    got = ops.act_dequant_i8(x8, s1, False)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    with pytest.raises(ValueError):
+        ops.act_dequant_i8(x8, sx[:-1] if M > 1 else dev(torch.zeros(2)), True)
+
+
 def test_a8w8_per_token_forward_matches_float64(ops):
     """Per-token x per-channel scaled output of the int8 GEMM (bf16 scales read in the epilogue) against the float64
     product of the dequantised operands."""
