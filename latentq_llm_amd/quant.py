@@ -441,6 +441,13 @@ class QLinearFunctionA8W8_dynamic_eval(torch.autograd.Function):
 
 
 def _qat_weight_i8(weight_f, qscales):
+    """clamp(round(weight_f / qscales), -128, 127) as int8 (utils/quant.py:345-346): one pass (lq_w8_requant, the
+    same chain as Qfunc_8bit_res without a residual) where the kernel takes the operands."""
+    if (FUSED_LATENT and weight_f.is_cuda and weight_f.dim() == 2 and weight_f.dtype == torch.bfloat16
+            and weight_f.is_contiguous() and weight_f.shape[1] % 8 == 0 and weight_f.data_ptr() % 16 == 0
+            and torch.is_tensor(qscales) and qscales.dtype == torch.bfloat16 and qscales.is_contiguous()
+            and qscales.is_cuda and tuple(qscales.shape) == (weight_f.shape[0], 1)):
+        return ops.w8_requant(weight_f, qscales)
     return (weight_f / qscales).round_().clamp_(-128, 127).to(torch.int8)
 
 
@@ -460,7 +467,12 @@ class QLinearFunctionQAT_dynamic(torch.autograd.Function):
         input, weight_f, bias = ctx.saved_tensors
         work, qscales = ctx.save_qparamaw
         input_f = _fake_quant_activation(input, work[0].to(input.dtype))
-        weight_q = (weight_f / qscales).round_().clamp_(-128, 127).mul_(qscales).to(input.dtype)
+        # the fake-quantised weight (utils/quant.py:363-365) is bf16(w8 * qscales) for the int8 codes of the forward:
+        # handed over as codes, so that the input gradient forms it inside its GEMM
+        if weight_f.dtype == torch.bfloat16 and input.dtype == torch.bfloat16:
+            weight_q = (_qat_weight_i8(weight_f, qscales), qscales)
+        else:
+            weight_q = (weight_f / qscales).round_().clamp_(-128, 127).mul_(qscales).to(input.dtype)
         return _a8w8_backward_common(ctx, grad_output, input_f, weight_q, bias, detach_dw=False)
 
 

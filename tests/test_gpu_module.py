@@ -220,6 +220,44 @@ def test_qlinear_qat_forward(Q):
     assert rel_l2(y.float().cpu(), want.float()) < 1e-2
 
 
+def test_qlinear_qat_training_step_on_library_kernels_equals_the_tensor_chain(Q):
+    """QLinearQAT forward + backward: with the weight quantised by the one-pass kernel and the input gradient formed
+    from the int8 codes, against the same layer on the tensor-operation chain. Output and weight gradient identical
+    bit for bit (same codes, same operands); the input gradient within the reduction-order tolerance."""
+    N, K, M = 128, 256, 192
+    wf = randn_bf16((N, K), 5, 0.05)
+    qs = (wf.float().abs().amax(dim=1, keepdim=True) / 127).to(torch.bfloat16)
+    x0 = randn_bf16((M, K), 6)
+    dy = randn_bf16((M, N), 7).cuda()
+
+    def run(fused):
+        saved = (Q.FUSED_LATENT, Q.FUSED_A8W8_DX)
+        Q.FUSED_LATENT, Q.FUSED_A8W8_DX = fused, fused
+        try:
+            m = Q.QLinearQAT(K, N, bias=False, lbit=16, gbit=16)
+            m.qscales.data = qs.clone()
+            m.weight.data = wf.clone()
+            m = m.bfloat16().cuda()
+            m.to("cuda")
+            m.weight.requires_grad = True
+            m.add_hook()
+            x = x0.cuda().requires_grad_(True)
+            y = m(x)
+            y.backward(dy)
+            assert len(Q.dict_temp) == 0
+            return y.detach(), x.grad.detach(), m.weight.grad.detach()
+        finally:
+            Q.FUSED_LATENT, Q.FUSED_A8W8_DX = saved
+
+    y1, dx1, dw1 = run(True)
+    y0, dx0, dw0 = run(False)
+    assert torch.equal(y1, y0) and torch.equal(dw1, dw0)
+    assert rel_l2(dx1.float(), dx0.float()) < 3e-3
+    w8 = (wf / qs).round_().clamp_(-128, 127)
+    want_dx = dy.double().cpu() @ (w8 * qs).to(torch.bfloat16).double()
+    assert rel_l2(dx1.float().cpu(), want_dx) < 3e-3
+
+
 # ------------------------------------------------------------------ residual codec ----------
 @pytest.mark.parametrize("mu", [0, 1, 2, 3])
 def test_residual_codec_3fold_bit_exact(Q, mu):
