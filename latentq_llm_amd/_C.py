@@ -33,6 +33,7 @@ SIGNATURES = {
     "lq_act_quant_i8_dynamic": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp],
     "lq_act_quant_i8_per_token": [_vp, _vp, _vp, _i64, _i64, _vp],
     "lq_act_dequant_i8": [_vp, _vp, _i32, _vp, _i64, _i64, _vp],
+    "lq_act_fake_quant": [_vp, _vp, _vp, _i64, _vp],
     "lq_a8w8_fwd_qs": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "lq_residual_quant": [_vp, _vp, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],
     "lq_residual_dequant": [_vp, _vp, _i64, _i32, _i32, _f32, _i32, _f32, _i32, _vp],

@@ -2,6 +2,7 @@
 //   lq_act_quant_i8           per-tensor, clamp value given (a device scalar)
 //   lq_act_quant_i8_dynamic   per-tensor, clamp value = the tensor's own maximum (two launches, no host sync)
 //   lq_act_quant_i8_per_token one scale per token row from the row's absolute maximum (one pass over HBM)
+// and, for the backward passes, lq_act_dequant_i8 (int8 -> bf16) and lq_act_fake_quant (bf16 -> bf16 on the int8 grid)
 #include "lq_common.h"
 
 namespace {
@@ -239,7 +240,47 @@ __global__ __launch_bounds__(256) void act_dequant_kernel(const u32x4_t *__restr
     out[2 * L + 1] = o[1];
 }
 
+// Fake quantisation for the backward pass of the layers that keep the bf16 activations (utils/quant.py:200-202,
+// 358-360): out = bf16(clamp(rne(bf16(x * s)), -128, 127) / s) with the bf16 scalar s = 127 / clampv, i.e. the chain
+// (input * s).round_().clamp_(-128, 127).div_(s) as one pass; 8 elements per thread. The quotient of an integer of at
+// most 8 bits and a bf16 number keeps 2^-17 (relative) from every bf16 rounding tie, so for 2^-40 <= |s| <= 2^40 the
+// product with RN(1 / s) rounds to the same bf16 number as the quotient; other scales take the division. NaN stays NaN.
+__global__ __launch_bounds__(256) void act_fake_quant_kernel(const unsigned short *__restrict__ x, const unsigned short *__restrict__ s_dev,
+                                                             unsigned short *__restrict__ out, long long n) {
+    const float s = lq_bf16_bits_to_f32(s_dev[0]);
+    const bool fast = fabsf(s) >= 0x1p-40f && fabsf(s) <= 0x1p40f;
+    const float r = 1.0f / s;
+    const long long base = ((long long)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (base >= n) return;
+    auto one = [&](float f) {
+        const float a = lq_bf16_bits_to_f32(lq_f32_to_bf16_bits(f * s));
+        const float q = a != a ? a : __builtin_amdgcn_fmed3f(rintf(a), -128.0f, 127.0f);
+        return fast ? q * r : q / s;
+    };
+    if (base + 8 <= n) {
+        const u32x4_t v = *reinterpret_cast<const u32x4_t *>(x + base);
+        u32x4_t o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = lq_pack_bf16(one(lq_bf16_lo(v[j])), one(lq_bf16_hi(v[j])));
+        *reinterpret_cast<u32x4_t *>(out + base) = o;
+    } else {
+        for (long long i = base; i < n; ++i) out[i] = lq_f32_to_bf16_bits(one(lq_bf16_bits_to_f32(x[i])));
+    }
+}
+
 }  // namespace
+
+extern "C" int lq_act_fake_quant(const void *x, const void *s_bf16_dev, void *out, int64_t n, void *stream) {
+    LQ_REQUIRE(x && s_bf16_dev && out && n >= 0, "lq_act_fake_quant: bad argument");
+    LQ_REQUIRE(lq_aligned(x, 16) && lq_aligned(out, 16) && lq_aligned(s_bf16_dev, 2),
+               "lq_act_fake_quant: x and out must be 16-byte aligned");
+    if (n == 0) return LQ_OK;
+    const long long blocks = ((n + 7) / 8 + 255) / 256;
+    LQ_REQUIRE(blocks <= 0x7FFFFFFFll, "lq_act_fake_quant: n too large");
+    hipLaunchKernelGGL(act_fake_quant_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const unsigned short *)x,
+                       (const unsigned short *)s_bf16_dev, (unsigned short *)out, (long long)n);
+    return lq_check_launch("lq_act_fake_quant");
+}
 
 extern "C" int lq_act_dequant_i8(const int8_t *x8, const float *scale, int per_token, void *out, int64_t M, int64_t K,
                                  void *stream) {

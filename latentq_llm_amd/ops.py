@@ -409,6 +409,20 @@ def act_quant_i8_per_token(x):
     return x8, sx
 
 
+def act_fake_quant(x, s):
+    """bf16(clamp(round(bf16(x * s)), -128, 127) / s) (lq_act_fake_quant): x bf16 of any shape, s one bf16 number on
+    the device; the values of ``(x * s).round_().clamp_(-128, 127).div_(s)``."""
+    _chk(x, torch.bfloat16, "x")
+    _chk(s, torch.bfloat16, "s")
+    if s.numel() != 1:
+        raise ValueError("s must hold one element")
+    out = torch.empty_like(x)
+    if x.numel():
+        with torch.cuda.device(x.device):
+            _C.call("lq_act_fake_quant", x.data_ptr(), s.data_ptr(), out.data_ptr(), x.numel(), _stream(x))
+    return out
+
+
 def act_dequant_ok(x8, scale, per_token: bool) -> bool:
     """Whether act_dequant_i8 takes these operands."""
     return (x8.is_cuda and x8.dtype == torch.int8 and x8.dim() == 2 and x8.is_contiguous() and x8.numel() > 0

@@ -321,6 +321,9 @@ def _per_token(qparamaw):
 
 def _fake_quant_activation(input, clampv):
     s = 127. / clampv
+    if (FUSED_A8W8_DX and torch.is_tensor(s) and s.numel() == 1 and s.dtype == torch.bfloat16 and s.is_cuda
+            and input.is_cuda and input.dtype == torch.bfloat16 and input.is_contiguous() and input.data_ptr() % 16 == 0):
+        return ops.act_fake_quant(input, s.reshape(1))  # the chain below as one pass
     return (input * s).round_().clamp_(-128, 127).div_(s)
 
 

@@ -500,6 +500,29 @@ def test_act_dequant_equals_the_two_tensor_operations(ops, shape):
         ops.act_dequant_i8(x8, sx[:-1] if M > 1 else dev(torch.zeros(2)), True)
 
 
+@pytest.mark.parametrize("clampv", [3.984375, 0.0123, 250.0, 2.0 ** -45, 0.0])
+@pytest.mark.parametrize("n", [5, 4096 * 33 + 3])
+def test_act_fake_quant_equals_the_tensor_chain(ops, n, clampv):
+    """lq_act_fake_quant = (x * s).round_().clamp_(-128, 127).div_(s) with s = 127 / clampv in bf16, bit for bit: values
+    on rounding ties, beyond the clamp, infinities and a NaN among the inputs; scales inside and outside the range
+    of the reciprocal product (and the infinite scale of a zero clamp value)."""
+    c = dev(torch.tensor([clampv], dtype=torch.bfloat16))
+    s = 127. / c
+    x = randn_bf16((n,), n, 2.0) * float(c.float().abs().clamp(min=1e-30))
+    x = x.to(torch.bfloat16)
+    sf = float(s.float())
+    if n > 16 and 0 < abs(sf) < float("inf"):
+        x[:8] = (torch.tensor([0.5, 1.5, 2.5, -0.5, -1.5, 126.5, 127.5, -128.5]) / sf).to(torch.bfloat16)
+        x[8], x[9], x[10], x[11] = float("inf"), float("-inf"), float("nan"), 0.0
+    x = dev(x)
+    want = (x * s).round_().clamp_(-128, 127).div_(s)
+    got = ops.act_fake_quant(x, s.reshape(1))
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(got), nan)
+    diff = (got.view(torch.int16) != want.view(torch.int16)) & ~nan
+    assert int(diff.sum()) == 0, (int(diff.sum()), diff.nonzero()[:5].tolist())
+
+
 def test_a8w8_per_token_forward_matches_float64(ops):
     """Per-token x per-channel scaled output of the int8 GEMM (bf16 scales read in the epilogue) against the float64
     product of the dequantised operands."""
