@@ -270,7 +270,7 @@ int lq_act_quant_i8_per_token(const void *x, int8_t *x8, float *sx, int64_t M, i
 int lq_act_dequant_i8(const int8_t *x8, const float *scale, int per_token, void *out, int64_t M, int64_t K, void *stream);
 
 /* Fake quantisation of the activations for the backward pass of the Functions that save the bf16 input
- * (QLinearFunctionA8W8_static.backward, QLinearFunctionQAT_dynamic.backward: utils/quant.py:200-202, 358-360):
+ * (QLinearFunctionA8W8_static.backward, QLinearFunctionQAT_dynamic.backward: utils/quant.py:197-199, 358-360):
  * out = bf16(clamp(rne(bf16(x * s)), -128, 127) / s), the chain (input * s).round_().clamp_(-128, 127).div_(s) with
  * its bf16 roundings as one pass. x, out: bf16[n], 16-byte aligned; s: one bf16 number on the device (127 / clampv). */
 int lq_act_fake_quant(const void *x, const void *s_bf16_dev, void *out, int64_t n, void *stream);
