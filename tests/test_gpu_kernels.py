@@ -29,6 +29,10 @@ def co():
     return c_oracle
 
 
+def bits_t(t):
+    return t.detach().cpu().contiguous().view(torch.int16)
+
+
 def dev(t):
     return t.cuda()
 
@@ -480,21 +484,22 @@ def test_act_dequant_equals_the_two_tensor_operations(ops, shape):
     bf16 numbers, a zero, an infinity and a NaN among them)."""
     M, K = shape
     g = torch.Generator().manual_seed(M + K)
-    x8 = dev(torch.randint(-128, 128, shape, generator=g, dtype=torch.int8))
-    sx = (torch.rand(M, generator=g) * 0.1 + 1e-3)
+    x8c = torch.randint(-128, 128, shape, generator=g, dtype=torch.int8)
+    sxc = (torch.rand(M, generator=g) * 0.1 + 1e-3)
     if M > 4:
-        sx[0], sx[1], sx[2] = 0.0, float("inf"), float("nan")
-    sx = dev(sx)
-    want = x8.to(torch.bfloat16) * sx.view(-1, 1).to(torch.bfloat16)
-    got = ops.act_dequant_i8(x8, sx, True)
+        sxc[0], sxc[1], sxc[2] = 0.0, float("inf"), float("nan")
+    x8, sx = dev(x8c), dev(sxc)
+    want = x8c.to(torch.bfloat16) * sxc.view(-1, 1).to(torch.bfloat16)   # the two operations, on the CPU
+    got = ops.act_dequant_i8(x8, sx, True).cpu()
     # NaNs (0 * inf, x * NaN) in the same places, whatever their payload bits; everything else bit for bit
     nan = torch.isnan(want)
     assert torch.equal(torch.isnan(got), nan)
     diff = (got.view(torch.int16) != want.view(torch.int16)) & ~nan
     assert int(diff.sum()) == 0, (int(diff.sum()), diff.nonzero()[:5].tolist())
-    s1 = dev(torch.tensor([3.0, 0.0123456, 7.0]))[1:2]   # an element inside a larger buffer
-    want = x8.to(torch.bfloat16) * s1[0].to(torch.bfloat16)
-    got = ops.act_dequant_i8(x8, s1, False)
+    s1c = torch.tensor([3.0, 0.0123456, 7.0])
+    s1 = dev(s1c)[1:2]   # an element inside a larger buffer
+    want = x8c.to(torch.bfloat16) * s1c[1].to(torch.bfloat16)
+    got = ops.act_dequant_i8(x8, s1, False).cpu()
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     with pytest.raises(ValueError):
         ops.act_dequant_i8(x8, sx[:-1] if M > 1 else dev(torch.zeros(2)), True)
@@ -506,7 +511,7 @@ def test_act_fake_quant_equals_the_tensor_chain(ops, n, clampv):
     """lq_act_fake_quant = (x * s).round_().clamp_(-128, 127).div_(s) with s = 127 / clampv in bf16, bit for bit: values
     on rounding ties, beyond the clamp, infinities and a NaN among the inputs; scales inside and outside the range
     of the reciprocal product (and the infinite scale of a zero clamp value)."""
-    c = dev(torch.tensor([clampv], dtype=torch.bfloat16))
+    c = torch.tensor([clampv], dtype=torch.bfloat16)
     s = 127. / c
     x = randn_bf16((n,), n, 2.0) * float(c.float().abs().clamp(min=1e-30))
     x = x.to(torch.bfloat16)
@@ -514,9 +519,9 @@ def test_act_fake_quant_equals_the_tensor_chain(ops, n, clampv):
     if n > 16 and 0 < abs(sf) < float("inf"):
         x[:8] = (torch.tensor([0.5, 1.5, 2.5, -0.5, -1.5, 126.5, 127.5, -128.5]) / sf).to(torch.bfloat16)
         x[8], x[9], x[10], x[11] = float("inf"), float("-inf"), float("nan"), 0.0
-    x = dev(x)
-    want = (x * s).round_().clamp_(-128, 127).div_(s)
-    got = ops.act_fake_quant(x, s.reshape(1))
+    want = (x * s).round_().clamp_(-128, 127).div_(s)   # the chain, on the CPU
+    assert torch.equal(bits_t(127. / dev(c)), bits_t(s))  # the scalar the module computes on the device is the same number
+    got = ops.act_fake_quant(dev(x), dev(s).reshape(1)).cpu()
     nan = torch.isnan(want)
     assert torch.equal(torch.isnan(got), nan)
     diff = (got.view(torch.int16) != want.view(torch.int16)) & ~nan
