@@ -351,7 +351,7 @@ def bench_adam8(device):
 
 def bench_dw(device):
     """dW = dY^T X of the two MLP shapes (not part of `value`): the library's own GEMM (operands read as they lie),
-    the same with the int8 accumulator's add_ as its epilogue, and for scale the vendor GEMM on the strided view (as
+    the same with the int8 accumulator's add_ or the bf16 gradient's add_ as its epilogue, and for scale the vendor GEMM on the strided view (as
     the reference calls it) and on a transposed copy of dY."""
     from latentq_llm_amd import ops
     out = []
@@ -365,11 +365,15 @@ def bench_dw(device):
         q8 = torch.zeros((N, K), dtype=torch.int8, device=device)
         sc = torch.full((N, 1), 1e-3, dtype=torch.bfloat16, device=device)
         t_acc = event_time(lambda: ops.weight_grad_acc8(dy, x, q8, sc, seed=1, offset=0), 20)
+        gacc = torch.zeros((N, K), dtype=torch.bfloat16, device=device)
+        t_add = event_time(lambda: ops.weight_grad_acc(dy, x, gacc), 20)       # grad.add_(dW) as the epilogue
+        t_add_sep = event_time(lambda: gacc.add_(ops.weight_grad(dy, x)), 20)  # the product stored, then the addition
         out.append({"N": N, "K": K, "strided_mm_us": t_ref * 1e6, "strided_mm_TFLOP/s": flop / t_ref / 1e12,
                     "transposed_copy_mm_us": t_tr * 1e6, "transposed_copy_mm_TFLOP/s": flop / t_tr / 1e12,
                     "weight_grad_us": t_new * 1e6, "weight_grad_TFLOP/s": flop / t_new / 1e12,
                     "frac_mfma_bf16": flop / t_new / PEAK_BF16,
-                    "weight_grad_acc8_us": t_acc * 1e6, "weight_grad_acc8_TFLOP/s": flop / t_acc / 1e12})
+                    "weight_grad_acc8_us": t_acc * 1e6, "weight_grad_acc8_TFLOP/s": flop / t_acc / 1e12,
+                    "weight_grad_acc_bf16_us": t_add * 1e6, "weight_grad_then_add_us": t_add_sep * 1e6})
     return out
 
 

@@ -414,6 +414,9 @@ int lq_gradq8_quant(const void *dw, int8_t *q_inout, void *scale_inout, int accu
  * utils/quant.py:141-142, 207, 248, 289, 370). Both operands are read as they lie in memory (no transposed
  * copy). dy: bf16 [M,N]; x: bf16 [M,K]; M % 64 == 0, N % 8 == 0; dy, x and the output 16-byte aligned.
  *   lq_weight_grad:      dw_out = bf16(dW), bf16 [N,K], K % 8 == 0.
+ *   lq_weight_grad_acc:  dw_inout = bf16(dw_inout + bf16(dW)): the `module.weight.grad.add_(dW)` of backward_hook_fn
+ *     (utils/quant.py:398-411) on every micro-batch after the first when the gradient is kept in bf16 (gbit = 16),
+ *     as the GEMM's epilogue; the same bits as lq_weight_grad followed by a bf16 tensor addition.
  *   lq_weight_grad_acc8: the product with the add_ form of the 8-bit gradient accumulator as its epilogue
  *     (GradientQTensor.add_, utils/quant.py:891-898, reached from backward_hook_fn :398-411 on every
  *     micro-batch after the first): with d = bf16(dW),
@@ -422,6 +425,7 @@ int lq_gradq8_quant(const void *dw, int8_t *q_inout, void *scale_inout, int accu
  *     arguments, without dW ever being stored. q_inout: int8 [N,K]; scale: bf16 [N] (read); K % 16 == 0.
  * ------------------------------------------------------------------------- */
 int lq_weight_grad(const void *dy, const void *x, void *dw_out, int64_t M, int64_t N, int64_t K, void *stream);
+int lq_weight_grad_acc(const void *dy, const void *x, void *dw_inout, int64_t M, int64_t N, int64_t K, void *stream);
 int lq_weight_grad_acc8(const void *dy, const void *x, int8_t *q_inout, const void *scale, int64_t M, int64_t N,
                         int64_t K, const void *noise_or_null, uint64_t philox_seed, uint64_t philox_offset,
                         void *stream);

@@ -46,6 +46,7 @@ SIGNATURES = {
     "lq_residual_quant_s": [_vp, _vp, _i64, _i32, _vp],
     "lq_gradq8_quant": [_vp, _vp, _vp, _i32, _i64, _i64, _vp, _u64, _u64, _vp],
     "lq_weight_grad": [_vp, _vp, _vp, _i64, _i64, _i64, _vp],
+    "lq_weight_grad_acc": [_vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "lq_weight_grad_acc8": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _u64, _u64, _vp],
     "lq_repack_gptq_to_native": [_vp, _vp, _i64, _i64, _vp],
     "lq_repack_native_to_gptq": [_vp, _vp, _i64, _i64, _vp],

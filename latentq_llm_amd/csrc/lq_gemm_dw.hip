@@ -37,6 +37,7 @@ struct DwParams {
     const unsigned char *dy;  // bf16 [M, N]
     const unsigned char *x;   // bf16 [M, K]
     unsigned short *dw;       // store: bf16 [N, K]
+    int accumulate;           // store: dw = bf16(dw + bf16(product)) instead of dw = bf16(product)
     signed char *q;           // acc8: int8 [N, K], updated in place
     const unsigned short *scale;  // acc8: bf16 [N]
     const unsigned short *noise;  // acc8: bf16 [N, K] or null (Philox)
@@ -235,7 +236,20 @@ __global__ __launch_bounds__(NT) void gemm_dw_kernel(DwParams p) {
                 const int row = it * 8 + ep_row;
                 const u32x4_t o = *reinterpret_cast<const u32x4_t *>(ep + row * EP + ep_chunk * 16);
                 const int nn = nrow0 + row;
-                if (nn < p.N && kc < p.K) *reinterpret_cast<u32x4_t *>(p.dw + (long long)nn * p.K + kc) = o;
+                if (nn < p.N && kc < p.K) {
+                    unsigned short *dst = p.dw + (long long)nn * p.K + kc;
+                    if (p.accumulate) {
+                        // the bf16 addition a tensor `add_` of the stored product would make
+                        const u32x4_t old = *reinterpret_cast<const u32x4_t *>(dst);
+                        u32x4_t sum;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            sum[e] = lq_pack_bf16(lq_bf16_lo(old[e]) + lq_bf16_lo(o[e]), lq_bf16_hi(old[e]) + lq_bf16_hi(o[e]));
+                        *reinterpret_cast<u32x4_t *>(dst) = sum;
+                    } else {
+                        *reinterpret_cast<u32x4_t *>(dst) = o;
+                    }
+                }
             }
         }
     } else {
@@ -327,6 +341,17 @@ extern "C" int lq_weight_grad(const void *dy, const void *x, void *dw_out, int64
     p.dy = (const unsigned char *)dy; p.x = (const unsigned char *)x; p.dw = (unsigned short *)dw_out;
     p.M = (int)M; p.N = (int)N; p.K = (int)K;
     return launch_dw(p, false, (hipStream_t)stream, "lq_weight_grad");
+}
+
+extern "C" int lq_weight_grad_acc(const void *dy, const void *x, void *dw_inout, int64_t M, int64_t N, int64_t K, void *stream) {
+    int rc = check_dw("lq_weight_grad_acc", dy, x, M, N, K, 8);
+    if (rc) return rc;
+    LQ_REQUIRE(dw_inout && lq_aligned(dw_inout, 16), "lq_weight_grad_acc: dw_inout must be given, 16-byte aligned");
+    DwParams p = {};
+    p.dy = (const unsigned char *)dy; p.x = (const unsigned char *)x; p.dw = (unsigned short *)dw_inout;
+    p.accumulate = 1;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    return launch_dw(p, false, (hipStream_t)stream, "lq_weight_grad_acc");
 }
 
 extern "C" int lq_weight_grad_acc8(const void *dy, const void *x, int8_t *q_inout, const void *scale, int64_t M, int64_t N,

@@ -612,6 +612,24 @@ def weight_grad(dy, x):
     return dy.t().mm(x)
 
 
+def weight_grad_acc_ok(dy, x, g) -> bool:
+    """Whether weight_grad_acc can add dY^T X onto the gradient tensor g in place."""
+    return (_weight_grad_native_ok(dy, x) and torch.is_tensor(g) and g.is_cuda and g.device == dy.device
+            and g.dtype == torch.bfloat16 and g.is_contiguous() and tuple(g.shape) == (dy.shape[1], x.shape[1])
+            and g.data_ptr() % 16 == 0)
+
+
+def weight_grad_acc(dy, x, g):
+    """g = bf16(g + bf16(dY^T X)) in place (lq_weight_grad_acc): the weight-gradient GEMM with the bf16 ``add_`` of the
+    gradient accumulation as its epilogue; the same bits as ``g.add_(weight_grad(dy, x))``."""
+    if not weight_grad_acc_ok(dy, x, g):
+        raise ValueError("weight_grad_acc needs contiguous bf16 GPU operands, M % 64 == 0, N % 8 == 0, K % 8 == 0 and g [N, K]")
+    N, K = dy.shape[1], x.shape[1]
+    with torch.cuda.device(dy.device):
+        _C.call("lq_weight_grad_acc", dy.data_ptr(), x.data_ptr(), g.data_ptr(), dy.shape[0], N, K, _stream(dy))
+    return g
+
+
 def weight_grad_acc8(dy, x, q, scale, noise=None, seed: int = 0, offset: int = 0):
     """q = quant(dequant(q) + dY^T X) in place (lq_weight_grad_acc8): the weight-gradient GEMM with the add_ form of
     the 8-bit gradient accumulator as its epilogue. dy bf16 [M,N], x bf16 [M,K], q int8 [N,K], scale bf16 [N,1]."""

@@ -502,6 +502,9 @@ def backward_hook_fn(module, grad_out, grad_in):
         if isinstance(g, GradientQTensor) and g.acc_ite > 0 and g.can_add_product(dw.dy, dw.x):
             g.add_product_(dw.dy, dw.x)
             return
+        if FUSED_GRADQ and torch.is_tensor(g) and ops.weight_grad_acc_ok(dw.dy, dw.x, g):
+            ops.weight_grad_acc(dw.dy, dw.x, g)  # g.add_(dW) as the GEMM's epilogue
+            return
         dw = dw.tensor()
     if isinstance(g, GradientQTensor):
         if g.acc_ite == 0:

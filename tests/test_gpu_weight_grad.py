@@ -100,3 +100,52 @@ def test_weight_grad_acc8_epilogue_bit_exact(ops, M, N, K, mode):
         mism = int((q.cpu().numpy().reshape(-1) != want_q).sum())
         assert mism == 0, f"{mism} of {N * K} int8 values differ from the oracle at micro-batch {i}"
     assert np.array_equal(bits(s).reshape(-1), want_s)  # the scales are read, never written
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_weight_grad_accumulating_form_equals_a_bf16_add(ops, M, N, K):
+    """lq_weight_grad_acc: g = bf16(g + bf16(dY^T X)), bit for bit what `g.add_(dW)` makes of the stored product (the
+    addition done by the tensor library on the CPU), partial tiles included."""
+    dy, x = randn_bf16((M, N), 11).cuda(), randn_bf16((M, K), 12).cuda()
+    g0 = randn_bf16((N, K), 13, 20.0)
+    dw = ops.weight_grad(dy, x)
+    want = g0.clone().add_(dw.cpu())
+    g = g0.cuda()
+    assert ops.weight_grad_acc(dy, x, g) is g
+    assert torch.equal(g.cpu().view(torch.int16), want.view(torch.int16))
+    with pytest.raises(ValueError):
+        ops.weight_grad_acc(dy, x, g[:, :-8] if K > 8 else g.float())
+
+
+def test_bf16_gradient_accumulation_through_the_gemm_epilogue(hip_lib):
+    """gbit = 16 (the reference's default): from the second micro-batch on the backward hook adds dW onto
+    module.weight.grad inside the GEMM; the accumulated gradient equals the sum of the separately formed products,
+    added in bf16 one after the other, bit for bit, and no product tensor is materialised."""
+    from latentq_llm_amd import ops as O
+    from latentq_llm_amd import quant as Q
+    from tests.util import make_w4
+    N, K, M = 128, 256, 192
+    codes, packed, scales, zeros = make_w4(N, K, 31)
+    m = Q.QLinearA16W4(K, N, bias=False, lbit=0, gbit=16)
+    m.zeros.data, m.scales.data, m.wshape = zeros.clone(), scales.clone(), [N, K]
+    m.weight.set_value(packed, [m.scales, m.zeros, m.wshape])
+    m = m.bfloat16().cuda()
+    m.to("cuda")
+    m.weight.requires_grad = True
+    m.add_hook()
+    x = randn_bf16((M, K), 32).cuda().requires_grad_(True)
+    dys = [randn_bf16((M, N), 33 + i).cuda() for i in range(3)]
+    calls = {"store": 0, "acc": 0}
+    real_store, real_acc = O.weight_grad, O.weight_grad_acc
+    try:
+        O.weight_grad = lambda *a, **k: (calls.__setitem__("store", calls["store"] + 1), real_store(*a, **k))[1]
+        O.weight_grad_acc = lambda *a, **k: (calls.__setitem__("acc", calls["acc"] + 1), real_acc(*a, **k))[1]
+        for dy in dys:
+            m(x).backward(dy)
+        assert calls == {"store": 1, "acc": 2} and len(Q.dict_temp) == 0
+    finally:
+        O.weight_grad, O.weight_grad_acc = real_store, real_acc
+    want = O.weight_grad(dys[0], x.detach())
+    for dy in dys[1:]:
+        want.add_(O.weight_grad(dy, x.detach()))
+    assert torch.equal(m.weight.grad, want)
