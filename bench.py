@@ -294,6 +294,43 @@ def bench_a8w8(device):
     return out
 
 
+def bench_a8w8_layer_step(device):
+    """One A8W8 layer's training micro-step at the configs[3] shapes (not part of `value`): forward, input gradient and
+    weight gradient accumulated in bf16, on the library's kernels and as the tensor-operation chain the reference's
+    Functions run (utils/quant.py:254-293 with backward_hook_fn; the vendor's int8 product standing in for its
+    external GEMM, and without the host synchronisation its `.item()` costs). Wall time of the launches from the
+    host: for the smallest shape that is launch overhead as much as kernel time."""
+    from latentq_llm_amd import ops
+    M, out = TOKENS, []
+    for (N, K) in [(2048, 2048), (8192, 2048), (2048, 8192)]:
+        g = torch.Generator(device="cpu").manual_seed(N + K)
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(device)
+        dy = torch.randn(M, N, generator=g).to(torch.bfloat16).to(device)
+        w8 = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).to(device)
+        qs = (torch.rand(N, 1, generator=g) * 0.01 + 1e-3).to(torch.bfloat16).to(device)
+        grad = torch.zeros(N, K, dtype=torch.bfloat16, device=device)
+
+        def fused():
+            x8, sx, work = ops.act_quant_i8_dynamic(x, True)
+            ops.a8w8_forward(x8, w8, sx, qs.view(-1))
+            xf = ops.act_dequant_i8(x8, work[1:2], False)
+            ops.a8w8_dx(dy, w8, qs.view(-1))
+            ops.weight_grad_acc(dy, xf, grad)
+
+        def chain():
+            clampv = x.max()
+            x8 = (x * 127. / clampv).round_().clamp_(-128, 127).to(torch.int8)
+            acc = torch._int_mm(x8, w8.t())
+            _ = ((acc.float() * (clampv.float() / 127.)).to(torch.bfloat16)) * qs.view(1, -1)
+            xf = x8.to(torch.bfloat16) * (clampv / 127.)
+            wf = (w8.to(torch.bfloat16) * qs).to(torch.bfloat16)
+            dy.mm(wf)
+            grad.add_(dy.t().mm(xf))
+        out.append({"N": N, "K": K, "library_kernels_us": event_time(fused, 20) * 1e6,
+                    "tensor_op_chain_us": event_time(chain, 20) * 1e6})
+    return out
+
+
 def bench_adam8(device):
     """One Adam step on uint8 block-wise moments over 8192 x 2048 elements: the fused kernel and, for
     scale, the chain of tensor operations it replaces (latentq_llm_amd.quant with FUSED_ADAM8 off)."""
@@ -885,6 +922,7 @@ def main():
         line["latent_lbit4"] = bench_latent(dev)
         line["gemv"] = bench_gemv(dev)
         line["a8w8"] = bench_a8w8(dev)
+        line["a8w8_layer_step"] = bench_a8w8_layer_step(dev)
         line["adam8"] = bench_adam8(dev)
         line["dw"] = bench_dw(dev)
         line["hbm_copy"] = bench_copy(dev)
