@@ -40,7 +40,10 @@
 // already prepares the first operands of the next step, so the MFMA stream never drains. The
 // global loads are inline assembly with explicit s_waitcnt so that they stay in flight across
 // barriers and the compiler's wait insertion never sees them; they are spread over the step, one
-// kind per half-slice.
+// kind per half-slice. Only the odd step's wait covers the codes, scales and zeros requested during the even step before
+// it (they are first read after that wait), so a request has 1.75 steps to return: weights come from HBM in any real
+// use, and with the wait of the requesting step itself (0.75 steps) the forward down launch ran 5 % slower inside a
+// training step than in a loop over the one launch, where they come from the last-level cache.
 //
 // The chip is power-limited on this kernel (under sustained load the shader clock sits at 1.64 GHz with two
 // workgroups per compute unit and at 2.0 GHz with one, against 1.81 GHz for a loop of nothing but MFMAs on
@@ -260,7 +263,10 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
     auto wait_and_meet = [&](auto newest, auto with_qparams) {
         constexpr int NEWEST = decltype(newest)::value;
         (void)cn; (void)qs; (void)qz;  // named outside the constexpr branches so that the lambda captures them
-        if constexpr (NT == 2) {
+        if constexpr (decltype(with_qparams)::value == 2) {
+            // a wait that releases no loaded register: nothing requested since the previous wait is read before the next one
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(NEWEST) : "memory");
+        } else if constexpr (NT == 2) {
             if constexpr (decltype(with_qparams)::value != 0) {
                 asm volatile("s_waitcnt vmcnt(%8) lgkmcnt(0)\n\ts_barrier"
                              : "+v"(cn[0][0]), "+v"(cn[0][1]), "+v"(cn[NT - 1][0]), "+v"(cn[NT - 1][1]), "+v"(qs[0]), "+v"(qs[NT - 1]),
@@ -308,7 +314,14 @@ __global__ __launch_bounds__(256, 2) void gemm_fwd_direct_kernel(FwdParams p) {
 #pragma unroll
             for (int i = 0; i < NT; ++i) {
                 if (t == 3 && i == 0) {
-                    wait_and_meet(ic<2>(), ic<ODD ? 0 : 1>());
+                    // Odd step: everything but the two LDS-direct loads just issued has to be here (tile kt+1, and the
+                    // codes, scales and zeros the even step before requested: slice 3 starts on them). Even step: only
+                    // what earlier steps requested (tile kt+1); its own requests (2 NT code loads, then 2 LDS-direct
+                    // loads; on every eighth step 2 NT scale / zero loads in between, which makes the count
+                    // conservative there) may stay in flight until the next step's wait, so that codes coming from
+                    // HBM have 1.75 steps to arrive instead of 0.75.
+                    if constexpr (ODD) wait_and_meet(ic<2>(), ic<1>());
+                    else wait_and_meet(ic<2 * NT + 2>(), ic<2>());
                     if (ODD) use_qparams((kt + 1) >> 1);
                 }
                 const unsigned char *src = t < 3 ? la : la_after;
