@@ -280,13 +280,18 @@ def bench_a8w8(device):
     M = TOKENS
     out = []
     for (N, K) in [(2048, 2048), (8192, 2048), (2048, 8192)]:
-        x8 = torch.randint(-127, 128, (M, K), device=device, dtype=torch.int8)
-        w8 = torch.randint(-127, 128, (N, K), device=device, dtype=torch.int8)
+        # HIP graphs over rotating weight matrices, 0.4 GB of them (the weights come from HBM, as in any real use; the
+        # activations are where the previous kernel left them), and over one matrix (everything cached) for comparison
+        nb = (400 << 20) // (N * K) + 1
         sx = (torch.randn(M, device=device) * 0.05).abs()
         sw = (torch.randn(N, device=device) * 0.01).abs()
-        sec = event_time(lambda: ops.a8w8_forward(x8, w8, sx, sw), 20)
+        x8 = torch.randint(-127, 128, (M, K), device=device, dtype=torch.int8)
+        ws = [torch.randint(-127, 128, (N, K), device=device, dtype=torch.int8) for _ in range(nb)]
+        sec = graph_time([(lambda w=w: ops.a8w8_forward(x8, w, sx, sw)) for w in ws])
+        sec_cached = graph_time([(lambda: ops.a8w8_forward(x8, ws[0], sx, sw)) for _ in range(8)])
+        del ws
         out.append({"M": M, "N": N, "K": K, "us": sec * 1e6, "TOP/s": 2 * M * N * K / sec / 1e12,
-                    "frac_mfma_i8": 2 * M * N * K / sec / PEAK_I8})
+                    "frac_mfma_i8": 2 * M * N * K / sec / PEAK_I8, "weight_matrices": nb, "us_cached_weights": sec_cached * 1e6})
     # what the int8 matrix pipes deliver with nothing else in the loop (random and all-zero operands, two waves per SIMD)
     ceil = {}
     for name, zero in (("random_operands", False), ("zero_operands", True)):
@@ -298,15 +303,23 @@ def bench_a8w8(device):
     out.append({"ceiling": ceil})
     # the activation quantisers in front of the GEMM (bf16 -> int8): given clamp value, the tensor's own maximum
     # found on the device (two launches), one scale per token row
-    x = torch.randn(M, 8192, device=device).to(torch.bfloat16)
-    clampv = x.float().abs().max().reshape(1)
-    sec = event_time(lambda: ops.act_quant_i8(x, clampv), 20)
-    out.append({"act_quant": [M, 8192], "us": sec * 1e6, "GB/s": 3 * x.numel() / sec / 1e9})
-    sec = event_time(lambda: ops.act_quant_i8_dynamic(x), 20)
-    out.append({"act_quant_dynamic": [M, 8192], "us": sec * 1e6, "GB/s": 5 * x.numel() / sec / 1e9,
-                "bytes_per_element": 5, "what": "max pass (2 B read) + quantise pass (2 B read, 1 B written)"})
-    sec = event_time(lambda: ops.act_quant_i8_per_token(x), 20)
-    out.append({"act_quant_per_token": [M, 8192], "us": sec * 1e6, "GB/s": 3 * x.numel() / sec / 1e9})
+    # (ten activation tensors in turn: 0.5 GB with their outputs, more than the last-level cache holds)
+    xs = [torch.randn(M, 8192, device=device).to(torch.bfloat16) for _ in range(10)]
+    numel = xs[0].numel()
+    clampv = xs[0].float().abs().max().reshape(1)
+    sec = event_time(_rotate([(lambda x=x: ops.act_quant_i8(x, clampv)) for x in xs]), 20)
+    out.append({"act_quant": [M, 8192], "us": sec * 1e6, "GB/s": 3 * numel / sec / 1e9})
+    sec = event_time(_rotate([(lambda x=x: ops.act_quant_i8_dynamic(x)) for x in xs]), 20)
+    out.append({"act_quant_dynamic": [M, 8192], "us": sec * 1e6, "GB/s": 5 * numel / sec / 1e9,
+                "bytes_per_element": 5, "what": "max pass (2 B read) + quantise pass (2 B read, 1 B written; the second read may come from the last-level cache)"})
+    sec = event_time(_rotate([(lambda x=x: ops.act_quant_i8_per_token(x)) for x in xs]), 20)
+    out.append({"act_quant_per_token": [M, 8192], "us": sec * 1e6, "GB/s": 3 * numel / sec / 1e9})
+    x8s = [ops.act_quant_i8_per_token(x) for x in xs]
+    sec = event_time(_rotate([(lambda t=t: ops.act_dequant_i8(t[0], t[1], True)) for t in x8s]), 20)
+    out.append({"act_dequant": [M, 8192], "us": sec * 1e6, "GB/s": 3 * numel / sec / 1e9})
+    s127 = (127. / clampv.to(torch.bfloat16)).reshape(1)
+    sec = event_time(_rotate([(lambda x=x: ops.act_fake_quant(x, s127)) for x in xs]), 20)
+    out.append({"act_fake_quant": [M, 8192], "us": sec * 1e6, "GB/s": 4 * numel / sec / 1e9})
     return out
 
 
@@ -347,55 +360,73 @@ def bench_a8w8_layer_step(device):
     return out
 
 
+def _rotate(calls):
+    """A callable that runs the next of `calls` each time (operand sets larger than the last-level cache in turn)."""
+    state = {"i": -1}
+
+    def run():
+        state["i"] = (state["i"] + 1) % len(calls)
+        calls[state["i"]]()
+    return run
+
+
 def bench_adam8(device):
     """One Adam step on uint8 block-wise moments over 8192 x 2048 elements: the fused kernel and, for
-    scale, the chain of tensor operations it replaces (latentq_llm_amd.quant with FUSED_ADAM8 off)."""
+    scale, the chain of tensor operations it replaces (latentq_llm_amd.quant with FUSED_ADAM8 off); then the whole
+    optimizer step of an lbit = 4 layer as one kernel, for 4-bit and for 8-bit weights. Every launch works on the
+    next of four operand sets (0.5-0.7 GB together: operands come from HBM, not from the last-level cache)."""
     from latentq_llm_amd import ops, quant as q
-    n, block = 8192 * 2048, 2048
+    N, K = 8192, 2048
+    n, block = N * K, 2048
     nblk = n // block
-    grad = (torch.randn(n, device=device) * 1e-3).to(torch.bfloat16)
-    param = (torch.randn(n, device=device) * 0.02).to(torch.bfloat16)
-    s1 = torch.randint(0, 256, (n,), device=device, dtype=torch.uint8)
-    s2 = torch.randint(0, 256, (n,), device=device, dtype=torch.uint8)
-    sc1 = torch.full((nblk, 1), 1e-5, device=device); mx1 = torch.full((nblk, 1), 1.3e-3, device=device)
-    sc2 = torch.full((nblk, 1), 1e-5, device=device); mx2 = torch.full((nblk, 1), 2.6e-3, device=device)
-    sec = event_time(lambda: ops.adam8_update(grad, s1, s2, sc1, mx1, sc2, mx2, 0.9, 0.95, 1e-8, 1e-3, param=param), 20)
+    curve = (2, 0.1875, 3, 0.375, 3)
+    sets = []
+    for i in range(4):
+        t = {"grad": (torch.randn(n, device=device) * 1e-3).to(torch.bfloat16),
+             "param": (torch.randn(n, device=device) * 0.02).to(torch.bfloat16),
+             "s1": torch.randint(0, 256, (n,), device=device, dtype=torch.uint8),
+             "s2": torch.randint(0, 256, (n,), device=device, dtype=torch.uint8),
+             "sc1": torch.full((nblk, 1), 1e-5, device=device), "mx1": torch.full((nblk, 1), 1.3e-3, device=device),
+             "sc2": torch.full((nblk, 1), 1e-5, device=device), "mx2": torch.full((nblk, 1), 2.6e-3, device=device),
+             "res": torch.randint(-2**31, 2**31 - 1, (n // 8,), device=device, dtype=torch.int64).to(torch.int32),
+             "w8": torch.randint(-128, 128, (N, K), device=device, dtype=torch.int8),
+             "qs": ((torch.randn(N, device=device) * 0.01).abs() + 1e-3).to(torch.bfloat16)}
+        t["codes"], t["scales"], t["zeros"] = synth_w4(N, K, 7 + i, device)
+        sets.append(t)
+    mom = lambda t: (t["s1"], t["s2"], t["sc1"], t["mx1"], t["sc2"], t["mx2"])
+    sec = event_time(_rotate([(lambda t=t: ops.adam8_update(t["grad"], *mom(t), 0.9, 0.95, 1e-8, 1e-3, param=t["param"]))
+                              for t in sets]), 20)
     nbytes = 10 * n + 32 * nblk
 
-    def chain():
-        m = q.DeQfunc_8bit_opt(s1, [sc1, mx1]).to(grad.dtype)
-        t = q.DeQfunc_8bit_opt(s2, [sc2, mx2])
-        v = (t * t).to(grad.dtype)
-        m.mul_(0.9).add_(grad, alpha=0.1)
-        v.mul_(0.95).addcmul_(grad, grad, value=0.05)
+    def chain(t=sets[0]):
+        m = q.DeQfunc_8bit_opt(t["s1"], [t["sc1"], t["mx1"]]).to(torch.bfloat16)
+        v = q.DeQfunc_8bit_opt(t["s2"], [t["sc2"], t["mx2"]])
+        v = (v * v).to(torch.bfloat16)
+        m.mul_(0.9).add_(t["grad"], alpha=0.1)
+        v.mul_(0.95).addcmul_(t["grad"], t["grad"], value=0.05)
         d = v.sqrt_().add_(1e-8)
-        param.addcdiv_(m, d, value=-1e-3)
+        t["param"].addcdiv_(m, d, value=-1e-3)
         q.Qfunc_8bit_opt(m.float(), blocksize=nblk)
         q.Qfunc_8bit_opt(d.float(), blocksize=nblk)
     sec_chain = event_time(chain, 5, warm=2)
-    # the whole optimizer step of an lbit = 4 layer as one kernel: codes + residual words in and out
-    N, K = 8192, 2048
-    codes, scales, zeros = synth_w4(N, K, 7, device)
-    res = torch.randint(-2**31, 2**31 - 1, (n // 8,), device=device, dtype=torch.int64).to(torch.int32)
-    curve = (2, 0.1875, 3, 0.375, 3)
-    sec_step = event_time(lambda: ops.adam8_latent_w4_step(grad, codes, res, scales.view(-1), zeros.view(-1), (N, K), s1, s2,
-                                                           sc1, mx1, sc2, mx2, curve, curve, 0.9, 0.95, 1e-8, 1e-3), 20)
+    # the whole optimizer step of an lbit = 4 layer as one kernel: codes + residual words in and out.
     # per element: 2 B of gradient, 2 + 2 B of moments in and out, 0.5 + 0.5 B of codes and of residual in and out
+    sec_step = event_time(_rotate([(lambda t=t: ops.adam8_latent_w4_step(
+        t["grad"], t["codes"], t["res"], t["scales"].view(-1), t["zeros"].view(-1), (N, K), *mom(t), curve, curve,
+        0.9, 0.95, 1e-8, 1e-3)) for t in sets]), 20)
     step_bytes = 8 * n + 32 * nblk + 4 * n // 128
     # the same for an 8-bit-weight layer (int8 codes, one scale per row): the single kernel against its three passes
-    w8 = torch.randint(-128, 128, (N, K), device=device, dtype=torch.int8)
-    qs = ((torch.randn(N, device=device) * 0.01).abs() + 1e-3).to(torch.bfloat16)
-    sec_w8 = event_time(lambda: ops.adam8_latent_w8_step(grad, w8, res, qs, s1, s2, sc1, mx1, sc2, mx2, curve, curve,
-                                                         0.9, 0.95, 1e-8, 1e-3), 20)
+    sec_w8 = event_time(_rotate([(lambda t=t: ops.adam8_latent_w8_step(
+        t["grad"], t["w8"], t["res"], t["qs"], *mom(t), curve, curve, 0.9, 0.95, 1e-8, 1e-3)) for t in sets]), 20)
 
-    def three_passes():
-        lat = ops.latent_w8_reconstruct(w8, qs, res, *curve)
-        ops.adam8_update(grad, s1, s2, sc1, mx1, sc2, mx2, 0.9, 0.95, 1e-8, 1e-3, param=lat.view(-1))
-        ops.latent_w8_requant(lat, qs, res, *curve)
-    sec_w8_3 = event_time(three_passes, 20)
+    def three_passes(t):
+        lat = ops.latent_w8_reconstruct(t["w8"], t["qs"], t["res"], *curve)
+        ops.adam8_update(t["grad"], *mom(t), 0.9, 0.95, 1e-8, 1e-3, param=lat.view(-1))
+        ops.latent_w8_requant(lat, t["qs"], t["res"], *curve)
+    sec_w8_3 = event_time(_rotate([(lambda t=t: three_passes(t)) for t in sets]), 20)
     w8_bytes = 9 * n + 32 * nblk + 2 * N  # as above with 1 + 1 B of codes
     return {"elements": n, "block": block, "bytes": nbytes, "us": sec * 1e6, "GB/s": nbytes / sec / 1e9,
-            "frac_hbm": nbytes / sec / PEAK_HBM, "tensor_op_chain_us": sec_chain * 1e6,
+            "frac_hbm": nbytes / sec / PEAK_HBM, "tensor_op_chain_us": sec_chain * 1e6, "operand_sets": len(sets),
             "latent_w4_step": {"bytes": step_bytes, "us": sec_step * 1e6, "GB/s": step_bytes / sec_step / 1e9,
                                "frac_hbm": step_bytes / sec_step / PEAK_HBM},
             "latent_w8_step": {"bytes": w8_bytes, "us": sec_w8 * 1e6, "GB/s": w8_bytes / sec_w8 / 1e9,
@@ -409,22 +440,25 @@ def bench_dw(device):
     from latentq_llm_amd import ops
     out = []
     for (N, K) in [(FFN, HID), (HID, FFN)]:
-        dy = torch.randn(TOKENS, N, device=device).to(torch.bfloat16)
-        x = torch.randn(TOKENS, K, device=device).to(torch.bfloat16)
+        # five operand / output sets in turn (0.9 GB: dY, X and the gradient come from HBM, as inside a training step)
+        sets = [(torch.randn(TOKENS, N, device=device).to(torch.bfloat16), torch.randn(TOKENS, K, device=device).to(torch.bfloat16),
+                 torch.zeros((N, K), dtype=torch.bfloat16, device=device), torch.zeros((N, K), dtype=torch.int8, device=device))
+                for _ in range(5)]
+        dy, x = sets[0][0], sets[0][1]
         flop = 2 * TOKENS * N * K
-        t_ref = event_time(lambda: dy.t().mm(x), 20)
-        t_tr = event_time(lambda: ops.transpose_bf16(dy).mm(x), 20)
-        t_new = event_time(lambda: ops.weight_grad(dy, x), 20)
-        q8 = torch.zeros((N, K), dtype=torch.int8, device=device)
+        t_ref = event_time(_rotate([(lambda t=t: t[0].t().mm(t[1])) for t in sets]), 20)
+        t_tr = event_time(_rotate([(lambda t=t: ops.transpose_bf16(t[0]).mm(t[1])) for t in sets]), 20)
+        t_new = event_time(_rotate([(lambda t=t: ops.weight_grad(t[0], t[1])) for t in sets]), 20)
+        t_cached = event_time(lambda: ops.weight_grad(dy, x), 20)
         sc = torch.full((N, 1), 1e-3, dtype=torch.bfloat16, device=device)
-        t_acc = event_time(lambda: ops.weight_grad_acc8(dy, x, q8, sc, seed=1, offset=0), 20)
-        gacc = torch.zeros((N, K), dtype=torch.bfloat16, device=device)
-        t_add = event_time(lambda: ops.weight_grad_acc(dy, x, gacc), 20)       # grad.add_(dW) as the epilogue
-        t_add_sep = event_time(lambda: gacc.add_(ops.weight_grad(dy, x)), 20)  # the product stored, then the addition
+        t_acc = event_time(_rotate([(lambda t=t: ops.weight_grad_acc8(t[0], t[1], t[3], sc, seed=1, offset=0)) for t in sets]), 20)
+        t_add = event_time(_rotate([(lambda t=t: ops.weight_grad_acc(t[0], t[1], t[2])) for t in sets]), 20)  # grad.add_(dW) as the epilogue
+        t_add_sep = event_time(_rotate([(lambda t=t: t[2].add_(ops.weight_grad(t[0], t[1]))) for t in sets]), 20)  # product stored, then added
+        del sets
         out.append({"N": N, "K": K, "strided_mm_us": t_ref * 1e6, "strided_mm_TFLOP/s": flop / t_ref / 1e12,
                     "transposed_copy_mm_us": t_tr * 1e6, "transposed_copy_mm_TFLOP/s": flop / t_tr / 1e12,
                     "weight_grad_us": t_new * 1e6, "weight_grad_TFLOP/s": flop / t_new / 1e12,
-                    "frac_mfma_bf16": flop / t_new / PEAK_BF16,
+                    "frac_mfma_bf16": flop / t_new / PEAK_BF16, "weight_grad_cached_operands_us": t_cached * 1e6,
                     "weight_grad_acc8_us": t_acc * 1e6, "weight_grad_acc8_TFLOP/s": flop / t_acc / 1e12,
                     "weight_grad_acc_bf16_us": t_add * 1e6, "weight_grad_then_add_us": t_add_sep * 1e6})
     return out

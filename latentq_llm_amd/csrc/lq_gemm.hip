@@ -1,11 +1,11 @@
-// Kernels (2a) and (3): LDS-tiled MFMA GEMMs for gfx950.
+// Kernel (2a): LDS-tiled MFMA GEMMs for gfx950.
 //
 //   MODE_W4_FWD : Y[M,N]  = X[M,K]  . deq(W)[N,K]^T     (bf16 MFMA, int4 W dequantised into LDS)
 //   MODE_W4_DX  : dX[M,K] = dY[M,N] . deq(W)[N,K]       (same, W tile transposed on the way out of LDS)
-//   MODE_I8     : acc     = X8[M,K] . W8[N,K]^T         (int8 MFMA, int32 accumulate, scaled epilogue)
 //   MODE_W8_DX  : dX[M,K] = dY[M,N] . (W8 * qs)[N,K]    (MODE_W4_DX with int8 codes and one bf16 scale per row n)
 //
-// (The forward pass of large grids runs the weights-direct kernel of lq_gemm_fwd.hip instead.)
+// (The forward pass of large grids runs the weights-direct kernel of lq_gemm_fwd.hip instead; the int8 GEMM of the
+// A8W8 layers is lq_gemm_i8.hip, dispatched from this file.)
 //
 // Common structure. "A" is the activation-side operand, row-major with the reduction
 // dimension contiguous. "B" is the weight-side operand, presented in LDS as
@@ -13,7 +13,7 @@
 // over n, the tile is kept in the weights' own [n][k] order (64 rows of 256 bytes, written as
 // plain 16-byte pieces) and the math waves fetch their operands with the transposing LDS read
 // ds_read_b64_tr_b16, so that the weight waves do the same cheap work in both directions.
-// A tile row holds 128 bytes (64 bf16 or 128 int8) = eight 16-byte chunks; one MFMA step
+// A tile row holds 128 bytes (64 bf16) = eight 16-byte chunks; one MFMA step
 // consumes 32 bytes of every row (chunks 2s and 2s+1), i.e. 4 steps per tile. Bank conflicts of
 // the 16-byte fragment reads (consecutive rows, same chunk) are avoided by XOR swizzles:
 //   * chunk c of A row r sits at position c ^ ((r >> 1) & 7);
@@ -47,22 +47,18 @@
 
 namespace {
 
-enum { MODE_W4_FWD = 0, MODE_W4_DX = 1, MODE_I8 = 2, MODE_W8_DX = 3 };
+enum { MODE_W4_FWD = 0, MODE_W4_DX = 1, MODE_W8_DX = 3 };
 
 struct GemmParams {
-    const void *a;        // activations: bf16 [M, R] or int8 [M, R]
-    const void *b;        // weights: packed codes or int8 [N, K]
+    const void *a;        // activations: bf16 [M, R]
+    const void *b;        // weights: packed int4 codes, or int8 [N, K] (MODE_W8_DX)
     const unsigned short *scales;
     const unsigned short *zeros;
     const unsigned short *bias;  // bf16 [out cols] or null
-    const float *sx;             // MODE_I8: per-row scale
-    const float *sw;             // MODE_I8: per-column scale (fp32, or bf16 when sw_bf16 is set)
-    int sw_bf16;
     void *c;                     // bf16 [M, C]
-    int *acc_out;                // MODE_I8: optional int32 [M, C]
     int M;                       // rows of A / C
-    int C;                       // output columns (N for fwd/i8, K for dx)
-    int R;                       // reduction length (K for fwd/i8, N for dx)
+    int C;                       // output columns (N for fwd, K for dx)
+    int R;                       // reduction length (K for fwd, N for dx)
     int Kw;                      // K of the weight matrix (row length of W in elements)
     int tiles_m, tiles_n;
     // split reduction: workgroup (tile, blockIdx.y) covers steps_per_split reduction steps from
@@ -125,8 +121,8 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
     constexpr int AROW = 128;                  // bytes per LDS row of A
     constexpr int APT = BM * 8 / NT;           // 16-byte LDS slots of A filled per math thread per tile
     constexpr int A_BYTES = APT * NT * 16, B_BYTES = BN * ROWB;
-    constexpr int ESZ = (MODE == MODE_I8) ? 1 : 2;
-    constexpr int RT = ROWB / ESZ;  // reduction elements per tile (64 bf16 / 128 int8)
+    constexpr int ESZ = 2;
+    constexpr int RT = ROWB / ESZ;  // reduction elements per tile: 64
     static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of 32x32");
     static_assert((BN * 8) % NT == 0, "B staging must divide evenly");
     static_assert(A_BYTES == BM * AROW && (BM * 8) % NT == 0, "A staging must divide evenly");
@@ -188,37 +184,24 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
 
     if (is_weight_wave) {
         // ======================= weight waves: B tiles =======================
-        //   I8      : BPT 16-byte chunks per thread, copied through registers.
         //   W4_FWD  : NW code words (8 k each) of one weight row -> NW 16-byte chunks of that row.
         //   W4_DX   : 4 code words (32 k) of one weight row n -> four 16-byte pieces of LDS row n. The
         //             tile stays in the weights' own [n][k] order; the math waves transpose it on
         //             the way out of LDS (ds_read_b64_tr_b16).
-        constexpr int BPT = (MODE == MODE_I8) ? BN * 8 / NT : 1;
         constexpr int NW = (MODE == MODE_W4_FWD) ? BN * 8 / NT : 1;  // tile has BN rows x 8 words
         static_assert(MODE != MODE_W4_FWD || NW == 2 || NW == 4 || NW == 8, "bad fwd staging split");
         static_assert(!kDx || (BN == 128 && NT == 256), "dX staging: 64 rows x 4 threads");
         constexpr int NSZ = 1;
         constexpr int NWORDS = (MODE == MODE_W4_DX) ? 4 : (MODE == MODE_W8_DX) ? 8 : NW;
 
-        const unsigned char *b_src[MODE == MODE_I8 ? BPT : 1];
-        int b_dst[MODE == MODE_I8 ? BPT : 1];
+        const unsigned char *b_src[1];
         const unsigned short *s_src[NSZ];
         const unsigned short *z_src[NSZ];
         const unsigned char *b_src2 = nullptr;  // W4_DX: the second product's codes, scales and zeros
         const unsigned short *s_src2 = nullptr, *z_src2 = nullptr;
         int b_row = 0, b_w0 = 0;  // W4_FWD: LDS row and first word; W4_DX: LDS row (n) and quarter of the row
 
-        if constexpr (MODE == MODE_I8) {
-#pragma unroll
-            for (int i = 0; i < BPT; ++i) {
-                const int c = i * NT + tid;
-                const int row = c >> 3, ch = c & 7;
-                int gr = c0 + row;
-                gr = gr < p.C ? gr : p.C - 1;
-                b_src[i] = (const unsigned char *)p.b + (long long)gr * p.Kw + ch * 16 + (long long)k0 * ROWB;
-                b_dst[i] = row * ROWB + ((ch ^ swz(row)) << 4);
-            }
-        } else if constexpr (MODE == MODE_W4_FWD) {
+        if constexpr (MODE == MODE_W4_FWD) {
             constexpr int TPR = 8 / NW;  // threads per weight row
             b_row = tid / TPR;
             b_w0 = (tid % TPR) * NW;
@@ -248,17 +231,13 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
         }
 
         struct Stage {
-            u32x4_t b[BPT];      // I8
-            unsigned w[NWORDS];  // W4 code words
+            unsigned w[NWORDS];  // code words
             unsigned short s[NSZ], z[NSZ];
         };
         Stage S0, S1;
 
         auto load_b = [&](int kt, Stage &S) {
-            if constexpr (MODE == MODE_I8) {
-#pragma unroll
-                for (int i = 0; i < BPT; ++i) S.b[i] = *reinterpret_cast<const u32x4_t *>(b_src[i] + (long long)kt * ROWB);
-            } else if constexpr (MODE == MODE_W4_FWD) {
+            if constexpr (MODE == MODE_W4_FWD) {
                 const unsigned char *src = b_src[0] + (long long)kt * 32;
                 if constexpr (NW == 8) {
                     u32x4_t v0 = *reinterpret_cast<const u32x4_t *>(src), v1 = *reinterpret_cast<const u32x4_t *>(src + 16);
@@ -293,10 +272,7 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
         };
 
         auto store_b = [&](unsigned char *lb, Stage &S) {
-            if constexpr (MODE == MODE_I8) {
-#pragma unroll
-                for (int i = 0; i < BPT; ++i) *reinterpret_cast<u32x4_t *>(lb + b_dst[i]) = S.b[i];
-            } else if constexpr (MODE == MODE_W4_FWD) {
+            if constexpr (MODE == MODE_W4_FWD) {
                 const float s = lq_bf16_bits_to_f32(S.s[0]);
                 const float nzs = -(lq_bf16_bits_to_f32(S.z[0]) * s);
                 const float s512 = s * 512.0f;  // the codes come out of the conversion as q/512
@@ -402,8 +378,7 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
         for (int q = 0; q < 4; ++q) issue_a_part(kt, la, q);
     };
 
-    using acc_t = typename std::conditional<MODE == MODE_I8, i32x16_t, f32x16_t>::type;
-    acc_t acc[FN][FM];
+    f32x16_t acc[FN][FM];
 #pragma unroll
     for (int i = 0; i < FN; ++i)
 #pragma unroll
@@ -463,15 +438,9 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
 #pragma unroll
         for (int i = 0; i < FN; ++i)
 #pragma unroll
-            for (int j = 0; j < FM; ++j) {
-                if constexpr (MODE == MODE_I8) {
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4_t, bf[i]),
-                                                                     __builtin_bit_cast(i32x4_t, af[j]), acc[i][j], 0, 0, 0);
-                } else {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[i]),
-                                                                       __builtin_bit_cast(bf16x8_t, af[j]), acc[i][j], 0, 0, 0);
-                }
-            }
+            for (int j = 0; j < FM; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf[i]),
+                                                                   __builtin_bit_cast(bf16x8_t, af[j]), acc[i][j], 0, 0, 0);
     };
 
     // Tile kt: A in buffer kt%3, B in buffer kt%2; the fragments of its first reduction slice are
@@ -566,7 +535,7 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
     constexpr int RPI = 64 / LPR;      // rows per store instruction
     const int ep_row = lane / LPR, ep_chunk = lane % LPR;
     const int c_lane = c0 + wn * TN + ep_chunk * 8;
-    float bias_v[FN][4][4], sw_v[FN][4][4];
+    float bias_v[FN][4][4];
 #pragma unroll
     for (int i = 0; i < FN; ++i)
 #pragma unroll
@@ -576,15 +545,10 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
             for (int r = 0; r < 4; ++r) {
                 const bool in = c + r < p.C;
                 bias_v[i][q][r] = (p.bias && in) ? lq_bf16_bits_to_f32(p.bias[c + r]) : 0.0f;
-                if (MODE == MODE_I8)
-                    sw_v[i][q][r] = !in ? 0.0f : p.sw_bf16 ? lq_bf16_bits_to_f32(reinterpret_cast<const unsigned short *>(p.sw)[c + r]) : p.sw[c + r];
             }
         }
 #pragma unroll
     for (int j = 0; j < FM; ++j) {
-        const int m = m0 + wm * TM + j * 32 + frag_row;
-        float sxm = 1.0f;
-        if (MODE == MODE_I8) sxm = m < p.M ? p.sx[m] : 0.0f;
 #pragma unroll
         for (int i = 0; i < FN; ++i) {
 #pragma unroll
@@ -592,20 +556,11 @@ __global__ __launch_bounds__(128 * WM * WN) void gemm_kernel(GemmParams p) {
                 float v[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    if (MODE == MODE_I8) v[r] = ((float)acc[i][j][4 * q + r] * sxm) * sw_v[i][q][r];
-                    else v[r] = acc[i][j][4 * q + r];
+                    v[r] = acc[i][j][4 * q + r];
                     if (p.bias) v[r] += bias_v[i][q][r];
                 }
                 u32x2_t o = {lq_pack_bf16(v[0], v[1]), lq_pack_bf16(v[2], v[3])};
                 *reinterpret_cast<u32x2_t *>(ep + frag_row * EP + (i * 32 + 8 * q + 4 * kh) * 2) = o;
-                if (MODE == MODE_I8 && p.acc_out) {
-                    const int c = c0 + wn * TN + i * 32 + 8 * q + 4 * kh;
-                    if (m < p.M && c < p.C) {
-                        i32x4_t a4 = {(int)acc[i][j][4 * q], (int)acc[i][j][4 * q + 1], (int)acc[i][j][4 * q + 2],
-                                      (int)acc[i][j][4 * q + 3]};
-                        *reinterpret_cast<i32x4_t *>(p.acc_out + (long long)m * p.C + c) = a4;
-                    }
-                }
             }
         }
 #pragma unroll
@@ -662,7 +617,7 @@ int launch_gemm(GemmParams p, hipStream_t st, const char *who) {
     auto kern = gemm_kernel<MODE, BM, BN, WM, WN>;
     const long long nwg = (long long)p.tiles_m * p.tiles_n;
     if (nwg > 0x7FFFFFFFll) return lq_fail(LQ_ERR_BAD_ARG, "%s: problem too large", who);
-    const int total_steps = p.R / ((MODE == MODE_I8) ? 128 : 64);
+    const int total_steps = p.R / 64;
     const unsigned splits = p.partial ? (unsigned)((total_steps + p.steps_per_split - 1) / p.steps_per_split) : 1u;
     hipLaunchKernelGGL(kern, dim3((unsigned)nwg, splits), dim3(128 * WM * WN), 0, st, p);
     return lq_check_launch(who);
@@ -691,17 +646,6 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
 }
 
 }  // namespace
-
-// 128 x 128 or 256 x 128 tiles. Measured: a workgroup alone on a compute unit takes ~0.54 us per
-// 64-deep step with the small tile and ~0.75 with the large one, and a second small-tile workgroup
-// on the same unit adds its full time, so a grid costs about (rounds of one workgroup per unit) x
-// pace: small tiles while they fit in one round, large ones otherwise.
-static bool small_tiles(const GemmParams &p) {
-    const long long cus = lq_device_cu_count();
-    const long long cols = (p.C + 127) / 128;
-    const long long small = (long long)((p.M + 127) / 128) * cols, big = (long long)((p.M + 255) / 256) * cols;
-    return 0.54 * (double)((small + cus - 1) / cus) < 0.75 * (double)((big + cus - 1) / cus);
-}
 
 // weights-direct forward GEMM (lq_gemm_fwd.hip)
 long long lq_gemm_fwd_direct_workgroups(int M, int N);
@@ -848,7 +792,7 @@ static W4Plan plan_fwd(long long M, long long N, long long K, size_t ws_bytes, l
 }
 
 // dX: rounds of one workgroup per compute unit at ~0.54 us per 64-deep step for 128 x 128 tiles,
-// ~0.75 for 256 x 128 (the comparison small_tiles() makes for the int8 path), or a split reduction.
+// ~0.75 for 256 x 128 (a second small-tile workgroup on the same unit adds its full time), or a split reduction.
 static W4Plan plan_dx(long long M, long long N, long long K, size_t ws_bytes, long long cus) {
     W4Plan out;
     const long long cols = (K + 127) / 128;
@@ -1173,23 +1117,13 @@ static int a8w8_fwd_impl(const void *x, const void *w, const float *sx, const vo
     const long long cus = lq_device_cu_count();
     if (tiles128 > cus)
         return lq_gemm_i8_tile_launch(x, w, sx, sw, sw_bf16, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 2, (hipStream_t)stream);
-    // a workgroup with a CU to itself: four 32 KB stages (loads three steps ahead) instead of two whenever a
-    // quarter of the CUs stay idle (15-17 against 20-22 us for the staged kernel on 128-512 tokens x 4096 x 4096,
-    // 13.9 against 15.8 for two stages on 512 x 6144 x 2048), and on long reductions with every CU busy
-    // (41 -> 37 us on 2048 x 2048 x 8192, 146 -> 127 on K = 32768)
-    if (4 * tiles128 <= 3 * cus || K >= 6144)
-        return lq_gemm_i8_tile_launch(x, w, sx, sw, sw_bf16, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 4, (hipStream_t)stream);
-    // every CU busy with one workgroup: two stages for short reductions (<= 16 steps: less to set up than the
-    // staged kernel's producer waves; 16.0 -> 13.1 us on 2048^3), the staged kernel in between (25.3 against
-    // 27.7 us on 1024 x 4096 x 4096)
-    if (K <= 2048)
-        return lq_gemm_i8_tile_launch(x, w, sx, sw, sw_bf16, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 2, (hipStream_t)stream);
-    GemmParams p = {};
-    p.a = x; p.b = w; p.sx = sx; p.sw = (const float *)sw; p.sw_bf16 = sw_bf16; p.bias = (const unsigned short *)bias_or_null; p.c = y;
-    p.acc_out = acc_or_null;
-    p.M = (int)M; p.C = (int)N; p.R = (int)K; p.Kw = (int)K;
-    if (small_tiles(p)) return launch_gemm<MODE_I8, 128, 128, 2, 2>(p, (hipStream_t)stream, "lq_a8w8_fwd");
-    return launch_gemm<MODE_I8, 256, 128, 2, 2>(p, (hipStream_t)stream, "lq_a8w8_fwd");
+    // A workgroup with a CU to itself: four 32 KB stages (loads three steps ahead). Nothing covers such a workgroup's
+    // waits but its own prefetch distance, and the weights come from HBM in any real use: timed over 0.4 GB of rotating
+    // weight matrices, 14.0 against 18.2 us for two stages on 2048^3, 10.0 against 11.9 at K = 1024, 23.4-24.2
+    // against 26.4-26.9 for the staged kernel on 2048 x 2048 x 4096 and 1024 x 4096 x 4096, 30.3 against 33.3 at
+    // K = 5120 (with the one weight matrix of a timing loop sitting in the last-level cache the three are within 10 %
+    // of each other, in no fixed order).
+    return lq_gemm_i8_tile_launch(x, w, sx, sw, sw_bf16, bias_or_null, y, acc_or_null, (int)M, (int)N, (int)K, 128, 4, (hipStream_t)stream);
 }
 
 extern "C" int lq_a8w8_fwd(const void *x, const void *w, const float *sx, const float *sw, const void *bias_or_null,
